@@ -1,0 +1,232 @@
+"""Pins for the CPU oracle: closed forms, invariants and float64 brute force.
+
+None of these retype the oracle's formula in the oracle's own arithmetic: the
+brute-force twins are numpy float64 loops / expressions written from the
+mathematical definition, and the rest are properties the mathematics fixes.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import layers as O
+
+
+# ----------------------------------------------------------------------------- YaRN parameters
+def test_yarn_constants_closed_form():
+    conc, inv = O.yarn_concentration_and_inv_freq()
+    assert conc == pytest.approx(1.3465735902799727, abs=1e-15)
+    assert inv.dtype == torch.float32 and inv.shape == (32,)
+    low = 32 * math.log(4096 / (32 * 2 * math.pi)) / math.log(150000.0)
+    high = 32 * math.log(4096 / (2 * math.pi)) / math.log(150000.0)
+    assert low == pytest.approx(8.092779, abs=1e-5)
+    assert high == pytest.approx(17.398024, abs=1e-5)
+    inv64 = inv.double().numpy()
+    assert inv64[0] == 1.0
+    for i in range(32):
+        f = 150000.0 ** (-i / 32)
+        if i <= 8:      # pure extrapolation below `low`
+            assert inv64[i] == pytest.approx(f, rel=2e-6)
+        elif i >= 18:   # pure interpolation above `high`
+            assert inv64[i] == pytest.approx(f / 32, rel=2e-6)
+        else:           # blended band
+            m = 1 - min(max((i - low) / (high - low), 0.0), 1.0)
+            assert inv64[i] == pytest.approx(f / 32 * (1 - m) + f * m, rel=5e-6)
+    assert np.all(np.diff(inv64) < 0)  # strictly decreasing frequencies
+
+
+def test_yarn_scaling_one_is_textbook_rope():
+    conc, inv = O.yarn_concentration_and_inv_freq(scaling_factor=1.0, base=10000.0, head_dim=128)
+    assert conc == 1.0
+    expect = 10000.0 ** (-np.arange(0, 128, 2) / 128)
+    np.testing.assert_allclose(inv.double().numpy(), expect, rtol=2e-6)
+
+
+def test_yarn_cos_sin_vs_float64():
+    pos = torch.tensor([0, 1, 4095, 4096, 8191, 131071], dtype=torch.int64)
+    cos, sin = O.yarn_cos_sin(pos)
+    conc, inv = O.yarn_concentration_and_inv_freq()
+    # angle is the *fp32* product; evaluate cos/sin of that fp32 angle in float64
+    ang32 = (pos.float()[:, None] * inv[None, :]).double().numpy()
+    np.testing.assert_allclose(cos.double().numpy(), np.cos(ang32) * conc, atol=4e-7)
+    np.testing.assert_allclose(sin.double().numpy(), np.sin(ang32) * conc, atol=4e-7)
+    assert torch.all(cos[0] == np.float32(conc)) and torch.all(sin[0] == 0)
+
+
+def test_token_positions_wrap():
+    p = O.token_positions(2, 3, 131071, 131072)
+    assert p.tolist() == [131071, 0, 1, 131071, 0, 1]
+
+
+# ----------------------------------------------------------------------------- RMSNorm
+def test_rmsnorm_bruteforce_float64():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(3, 40, generator=g).bfloat16()
+    s = (1 + 0.1 * torch.randn(40, generator=g)).bfloat16()
+    ref = np.empty((3, 40))
+    xn, sn = x.double().numpy(), s.double().numpy()
+    for r in range(3):
+        acc = 0.0
+        for c in range(40):
+            acc += xn[r, c] * xn[r, c]
+        inv = 1.0 / math.sqrt(acc / 40 + 1e-5)
+        for c in range(40):
+            ref[r, c] = xn[r, c] * inv * sn[c]
+    np.testing.assert_allclose(O.rmsnorm_ref(x, s, 1e-5).double().numpy(), ref, rtol=2e-6, atol=1e-7)
+
+
+def test_rmsnorm_invariants():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(4, 2880, generator=g)
+    one = torch.ones(2880)
+    y = O.rmsnorm_ref(x, one, 1e-5)
+    ms = x.pow(2).mean(-1)
+    torch.testing.assert_close(y.pow(2).mean(-1).sqrt(), 1 / torch.sqrt(1 + 1e-5 / ms), rtol=1e-5, atol=0)
+    torch.testing.assert_close(O.rmsnorm_ref(8 * x, one, 1e-5), y, rtol=1e-4, atol=1e-6)   # scale invariance up to eps
+    c, s = -3.0, torch.linspace(0.5, 1.5, 2880)
+    const = O.rmsnorm_ref(torch.full((1, 2880), c), s, 1e-5)
+    torch.testing.assert_close(const[0], -s / math.sqrt(1 + 1e-5 / c**2), rtol=1e-6, atol=0)
+    assert torch.all(O.rmsnorm_ref(torch.zeros(2, 2880), s, 1e-5) == 0)
+
+
+# ----------------------------------------------------------------------------- embedding / linear
+def test_embedding_is_row_gather():
+    g = torch.Generator().manual_seed(3)
+    table = torch.randn(97, 16, generator=g).bfloat16()
+    ids = torch.tensor([[0, 96, 5, 5, 0]], dtype=torch.int32)
+    out = O.embedding_ref(table, ids)
+    assert out.shape == (1, 5, 16)
+    for j, i in enumerate(ids[0].tolist()):
+        assert torch.equal(out[0, j], table[i])
+
+
+def test_linear_bruteforce_and_selectors():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(3, 24, generator=g).bfloat16()
+    w = torch.randn(10, 24, generator=g).bfloat16()
+    b = torch.randn(10, generator=g).bfloat16()
+    ref = x.double().numpy() @ w.double().numpy().T + b.double().numpy()
+    np.testing.assert_allclose(O.linear_ref(x, w, b).double().numpy(), ref, rtol=1e-5, atol=1e-5)
+    e = torch.zeros(1, 24)
+    e[0, 7] = 1.0
+    torch.testing.assert_close(O.linear_ref(e, w, b)[0], w.float()[:, 7] + b.float())
+
+
+# ----------------------------------------------------------------------------- rotary
+def _rot(x, pos, **kw):
+    cos, sin = O.yarn_cos_sin(torch.as_tensor(pos, dtype=torch.int64), **kw)
+    return O.rope_rotate_ref(x, cos, sin)
+
+
+def test_rope_layout_is_half_split():
+    x = torch.zeros(1, 1, 64)
+    x[0, 0, 3] = 1.0
+    y = _rot(x, [5])
+    nz = torch.nonzero(y[0, 0]).flatten().tolist()
+    assert nz == [3, 35]   # partner of d is d+32, not d^1
+    cos, sin = O.yarn_cos_sin(torch.tensor([5]))
+    assert y[0, 0, 3] == cos[0, 3] and y[0, 0, 35] == sin[0, 3]
+
+
+def test_rope_norm_and_position_zero():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(6, 8, 64, generator=g)
+    conc, _ = O.yarn_concentration_and_inv_freq()
+    y = _rot(x, [0, 1, 77, 4096, 8191, 100000])
+    n_in = x[..., :32] ** 2 + x[..., 32:] ** 2
+    n_out = y[..., :32] ** 2 + y[..., 32:] ** 2
+    torch.testing.assert_close(n_out, conc**2 * n_in, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(y[0], np.float32(conc) * x[0], rtol=1e-6, atol=0)
+
+
+def test_rope_relative_position_property():
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(1, 1, 64, generator=g).double()
+    k = torch.randn(1, 1, 64, generator=g).double()
+
+    def dot(m, n):
+        return float((_rot(q, [m]).double() * _rot(k, [n]).double()).sum())
+
+    # positions small enough that fp32 angles carry ~1e-6 absolute error
+    assert dot(10, 3) == pytest.approx(dot(107, 100), rel=2e-4, abs=2e-4)
+    assert dot(50, 50) == pytest.approx(dot(0, 0), rel=2e-4, abs=2e-4)
+
+
+def test_rope_additivity():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(1, 2, 64, generator=g)
+    conc, _ = O.yarn_concentration_and_inv_freq()
+    ab = _rot(_rot(x, [40]), [60])
+    torch.testing.assert_close(ab, np.float32(conc) * _rot(x, [100]), rtol=1e-4, atol=1e-4)
+
+
+def test_rope_textbook_when_unscaled():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, 1, 8, generator=g)
+    y = _rot(x, [3, 9], head_dim=8, base=10000.0, scaling_factor=1.0).double().numpy()
+    xn = x.double().numpy()
+    for r, p in enumerate([3, 9]):
+        for d in range(4):
+            th = p * 10000.0 ** (-2 * d / 8)
+            a, b = xn[r, 0, d], xn[r, 0, d + 4]
+            assert y[r, 0, d] == pytest.approx(a * math.cos(th) - b * math.sin(th), abs=2e-6)
+            assert y[r, 0, d + 4] == pytest.approx(b * math.cos(th) + a * math.sin(th), abs=2e-6)
+
+
+def test_qkv_rope_composition():
+    d = O.make_inputs(3, seed=9)
+    q, k, v = O.qkv_rope_ref(d["x"], d["w"], d["b"], d["positions"])
+    qkv = O.linear_ref(d["x"], d["w"], d["b"])
+    assert torch.equal(v, qkv[:, 4608:])            # v is the raw slice
+    cos, sin = O.yarn_cos_sin(d["positions"])
+    # head 5 of q, pair (d=7, d+32)
+    a, b = qkv[:, 5 * 64 + 7], qkv[:, 5 * 64 + 39]
+    torch.testing.assert_close(q[:, 5 * 64 + 7], a * cos[:, 7] - b * sin[:, 7])
+    torch.testing.assert_close(k[:, 2 * 64 + 39], qkv[:, 4096 + 2 * 64 + 39] * cos[:, 7] + qkv[:, 4096 + 2 * 64 + 7] * sin[:, 7])
+    qa, ka, va = O.qkv_rope_ref(d["x"], d["w"], d["b"], d["positions"], round_qkv_first=True)
+    torch.testing.assert_close(qa, q, rtol=1.6e-2, atol=1e-2)
+    torch.testing.assert_close(ka, k, rtol=1.6e-2, atol=1e-2)
+
+
+# ----------------------------------------------------------------------------- SwiGLU
+def test_swiglu_bruteforce_float64_edge_grid():
+    gs = [-30.0, -7.0, 0.0, 6.99, 7.0, 7.01, 30.0]
+    ls = [-30.0, -7.01, -7.0, -1.0, 0.0, 7.0, 30.0]
+    rows = []
+    for gv in gs:
+        row = []
+        for lv in ls:
+            row += [gv, lv]
+        rows.append(row)
+    x = torch.tensor(rows, dtype=torch.float32)
+    out = O.swiglu_ref(x).double().numpy()
+    for i, gv in enumerate(gs):
+        for j, lv in enumerate(ls):
+            gg = min(gv, 7.0)
+            ll = min(max(lv, -7.0), 7.0)
+            expect = gg / (1 + math.exp(-1.702 * gg)) * (ll + 1)
+            assert out[i, j] == pytest.approx(expect, rel=2e-6, abs=1e-12), (gv, lv)
+    j1 = ls.index(-1.0)
+    assert np.all(out[:, j1] == 0)                          # l = -1  =>  exact zero
+    sat = 7.0 / (1 + math.exp(-1.702 * 7.0))
+    assert out[gs.index(30.0), ls.index(0.0)] == pytest.approx(sat, rel=1e-6)
+    assert out[gs.index(-30.0), ls.index(0.0)] < 0 and out[gs.index(-30.0), ls.index(0.0)] > -1e-18  # no lower clamp on gate
+
+
+def test_swiglu_interleaved_equals_chunked_under_permutation():
+    g = torch.Generator().manual_seed(10)
+    x = (2 * torch.randn(5, 64, generator=g)).bfloat16()
+    perm = torch.cat((x[:, ::2], x[:, 1::2]), dim=-1)
+    assert torch.equal(O.swiglu_ref(x, interleaved=True), O.swiglu_ref(perm, interleaved=False))
+
+
+def test_eager_twins_within_tolerance_of_upcast_oracle():
+    d = O.make_inputs(8, swiglu_rows=32, seed=0)
+    torch.testing.assert_close(O.rmsnorm_eager(d["x"], d["norm_scale"]).float(), O.rmsnorm_ref(d["x"], d["norm_scale"]), rtol=1.6e-2, atol=1e-2)
+    torch.testing.assert_close(O.swiglu_eager(d["swiglu_x"]).float(), O.swiglu_ref(d["swiglu_x"]), rtol=5e-2, atol=5e-2)
+    cos_t, sin_t = O.yarn_cos_sin(torch.arange(8192))
+    q, k, v = O.qkv_rope_eager(d["x"], d["w"], d["b"], cos_t, sin_t, d["positions"])
+    qr, kr, vr = O.qkv_rope_ref(d["x"], d["w"], d["b"], d["positions"])
+    torch.testing.assert_close(q.float(), qr, rtol=5e-2, atol=5e-2)
+    torch.testing.assert_close(v.float(), vr, rtol=1.6e-2, atol=1e-2)
