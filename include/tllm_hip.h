@@ -1,0 +1,151 @@
+/*
+ * tllm_hip.h -- C ABI of libtllm_hip.so: the gpt-oss layer kernels for MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers and sizes, launches on the HIP
+ * stream it is given (a hipStream_t passed as void*; NULL = the null stream),
+ * never allocates, never synchronises and never throws. It returns 0 on
+ * success or a negative TLLM_E_* code; tllm_last_error() then holds a
+ * thread-local message. All tensors are dense row-major unless a stride is
+ * part of the signature. bf16 is the IEEE bfloat16 bit pattern (uint16_t).
+ *
+ * The "replaces" notes name the reference call each entry point stands in for
+ * (paths relative to the reference checkout, tritonllm/gpt_oss/triton/).
+ */
+#ifndef TLLM_HIP_H
+#define TLLM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TLLM_ABI_VERSION 1
+
+enum {
+  TLLM_OK = 0,
+  TLLM_E_ARG = -1,      /* null pointer, negative size, bad flag            */
+  TLLM_E_SHAPE = -2,    /* shape the kernels do not support                  */
+  TLLM_E_ALIGN = -3,    /* pointer / stride not aligned as required          */
+  TLLM_E_LAUNCH = -4    /* hipLaunchKernel reported an error                 */
+};
+
+#define TLLM_MAX_ROPE_FREQS 128
+
+/* YaRN rotary parameters, built on the host from the restated formula of
+ * model.py:267-305 (RotaryEmbedding._compute_concentration_and_inv_freq):
+ * inv_freq[i], i < n_freq = head_dim/2, and the concentration that scales
+ * both cos and sin. */
+typedef struct TllmYarn {
+  float inv_freq[TLLM_MAX_ROPE_FREQS];
+  float concentration;
+  int32_t n_freq;
+} TllmYarn;
+
+/* Where a rotary kernel takes its angles from.
+ *   position of row r:  positions ? positions[r]
+ *                                 : (r % tokens_per_batch) + (offset ? offset[0] : 0)
+ *   then wrapped modulo max_ctx (triton_kernels.py:57-59, 1066-1070).
+ *   cos/sin:  yarn != NULL  -> computed in registers:
+ *                              angle = float(pos) * inv_freq[i] (one fp32 product),
+ *                              cos(angle) * concentration, sin(angle) * concentration
+ *             else          -> read from the fp32 tables cos_table/sin_table
+ *                              [max_ctx, head_dim/2] (row stride table_row_stride floats)
+ * positions / offset are DEVICE pointers (int64), so a captured graph can
+ * replay with new positions. */
+typedef struct TllmRope {
+  const TllmYarn* yarn;          /* host pointer, copied into the launch          */
+  const float* cos_table;        /* device, used when yarn == NULL                */
+  const float* sin_table;        /* device, used when yarn == NULL                */
+  int64_t table_row_stride;      /* floats between table rows                     */
+  const int64_t* positions;      /* device [rows] or NULL                         */
+  const int64_t* offset;         /* device (1,) or NULL                           */
+  int64_t tokens_per_batch;      /* T of a [B,T,...] input; >= 1                  */
+  int64_t max_ctx;               /* positions wrap modulo this; >= 1              */
+} TllmRope;
+
+int tllm_abi_version(void);
+const char* tllm_last_error(void);
+
+/* y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * scale[:], fp32 inside, one
+ * round-to-nearest-even to bf16 on store. out may alias x.
+ * replaces rmsnorm_forward(x, scale, eps, out) triton_kernels.py:28-35
+ * (module RMSNorm.forward, model.py:55-68). scale is fp32 or bf16 [hidden]. */
+int tllm_rmsnorm_bf16(const void* x, const void* scale, int scale_is_bf16, void* out,
+                      int64_t rows, int64_t hidden, float eps, void* stream);
+
+/* out[t,:] = table[ids[t],:], bit-exact row gather.
+ * replaces torch.nn.Embedding forward, model.py:906-908, 920.
+ * ids are int32 (the reference's token tensors, model.py:1170) or int64.
+ * An id outside [0, vocab) writes a zero row and, if oob_flag != NULL, stores
+ * 1 into *oob_flag (device int32) -- no fault, no host sync. */
+int tllm_embedding_bf16(const void* table, const void* ids, int ids_is_i64, void* out,
+                        int64_t n_tokens, int64_t hidden, int64_t vocab, int32_t* oob_flag,
+                        void* stream);
+
+/* Clamped SwiGLU: gate g and linear l are the even/odd columns of x
+ * (interleaved != 0) or its first/second half (interleaved == 0);
+ * if has_limit: g = min(g, limit), l = clamp(l, -limit, limit);
+ * out = g * sigmoid(alpha * g) * (l + 1), fp32 inside, one RNE to bf16.
+ * x is [rows, 2*n_out] with row stride x_row_stride elements (last stride 1),
+ * out is [rows, n_out] dense.
+ * replaces swiglu(x, alpha, limit, interleaved) moe.py:25-33 and
+ * triton_kernels/swiglu.py:85-100 (swiglu / swiglu_torch). */
+int tllm_swiglu_bf16(const void* x, void* out, int64_t rows, int64_t n_out, int64_t x_row_stride,
+                     float alpha, float limit, int has_limit, int interleaved, void* stream);
+
+/* cos[p - start, i] = cos(float(p) * inv_freq[i]) * concentration (and sin),
+ * p in [start, start + n_pos): the tables RotaryEmbedding._compute_cos_sin
+ * builds (model.py:307-313), computed with the same device routine the fused
+ * kernels use in registers. cos/sin are fp32 [n_pos, n_freq] dense. */
+int tllm_yarn_table_f32(float* cos, float* sin, int64_t start, int64_t n_pos,
+                        const TllmYarn* yarn, void* stream);
+
+/* In-place half-split rotary on q [rows, n_q_heads, head_dim] and
+ * k [rows, n_kv_heads, head_dim] (bf16, dense): for d < head_dim/2
+ *   o[d]      = x[d] * cos - x[d + hd/2] * sin
+ *   o[d+hd/2] = x[d + hd/2] * cos + x[d] * sin      (fp32, one RNE per output).
+ * replaces rope_forward(query, key, sin, cos, max_context_length, offset)
+ * triton_kernels.py:90-108 (RotaryEmbedding.forward, model.py:329-337).
+ * k may be NULL (n_kv_heads ignored). */
+int tllm_rope_bf16(void* q, void* k, int64_t rows, int n_q_heads, int n_kv_heads, int head_dim,
+                   const TllmRope* rope, void* stream);
+
+/* Fused QKV projection + bias (+ rotary on q and k when rope != NULL).
+ *   qkv[r, :] = x[r, :] . W^T + b       (bf16 in, fp32 accumulate)
+ *   columns [0, n_q*hd) -> q, next n_kv*hd -> k, last n_kv*hd -> v;
+ *   rotary is applied to the fp32 accumulator of q and k, then one RNE to bf16.
+ * x [rows, hidden] dense; W [(n_q + 2 n_kv) * hd, hidden] dense; b bf16 or NULL.
+ * Row r of q/k/v is written at q + r*q_row_stride, k + r*k_row_stride
+ * + slot*kv_slot_stride, v likewise, strides in elements, where
+ * slot = (kv_slot_stride != 0 && rope && rope->offset) ? rope->offset[0] : 0
+ * is read on the device: with k/v pointing at a [B, n_ctx, n_kv, hd] cache,
+ * k_row_stride = n_ctx*n_kv*hd and kv_slot_stride = n_kv*hd this is the
+ * reference's write of the new token into the KV cache.
+ *
+ * _decode: weight-streaming kernel for few rows (any rows accepted; the
+ *   weight is streamed once per 16 rows).
+ *   replaces qkv_rope_cache_decode_forward triton_kernels.py:1109-1255 and,
+ *   with rope == NULL, qkv_decode_forward triton_kernels.py:615-659.
+ * _prefill: LDS-staged bf16 MFMA GEMM with the bias + rotary epilogue.
+ *   replaces F.linear + split + 3x contiguous + rope_forward,
+ *   model.py:506-522. */
+int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const void* b,
+                              void* q, void* k, void* v,
+                              int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                              int64_t kv_slot_stride,
+                              int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
+                              const TllmRope* rope, void* stream);
+
+int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const void* b,
+                               void* q, void* k, void* v,
+                               int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                               int64_t kv_slot_stride,
+                               int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
+                               const TllmRope* rope, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TLLM_HIP_H */

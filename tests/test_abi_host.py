@@ -1,0 +1,112 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every symbol the
+header declares, and rejects bad arguments on the host before anything is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from tritonllm_amd import _lib
+from tritonllm_amd.yarn import YarnParams, gpt_oss_yarn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "tllm_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tllm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    declared = _header_symbols()
+    assert declared, "no declarations parsed"
+    assert sorted(_lib.SIGNATURES) == declared
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.tllm_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_header():
+    assert C.sizeof(_lib.TllmYarn) == 128 * 4 + 4 + 4
+    assert C.sizeof(_lib.TllmRope) == 8 * 8
+
+
+def _err():
+    return _lib.lib().tllm_last_error().decode()
+
+
+def test_argument_errors_are_reported_not_launched():
+    lib = _lib.lib()
+    assert lib.tllm_rmsnorm_bf16(None, None, 0, None, 4, 2880, 1e-5, None) == -1
+    assert "null" in _err()
+    assert lib.tllm_rmsnorm_bf16(None, None, 0, None, -1, 2880, 1e-5, None) == -1
+    assert lib.tllm_rmsnorm_bf16(None, None, 0, None, 0, 2880, 1e-5, None) == 0     # empty input is a no-op
+    assert lib.tllm_embedding_bf16(None, None, 0, None, 0, 2880, 10, None, None) == 0
+    assert lib.tllm_embedding_bf16(None, None, 0, None, 3, 2880, 10, None, None) == -1
+    assert lib.tllm_swiglu_bf16(None, None, 0, 2880, 5760, 1.702, 7.0, 1, 1, None) == 0
+    assert lib.tllm_swiglu_bf16(None, None, 2, 2880, 100, 1.702, 7.0, 1, 1, None) == -1
+    assert "x_row_stride" in _err()
+    rope = _lib.TllmRope()
+    assert lib.tllm_rope_bf16(None, None, 0, 64, 8, 64, C.byref(rope), None) == -1   # no yarn, no tables, max_ctx 0
+    y = gpt_oss_yarn()
+    rope.yarn = y.c_pointer()
+    rope.max_ctx = 131072
+    rope.tokens_per_batch = 1
+    assert lib.tllm_rope_bf16(None, None, 0, 64, 8, 64, C.byref(rope), None) == 0
+    assert lib.tllm_rope_bf16(None, None, 0, 64, 8, 128, C.byref(rope), None) == -2  # head_dim vs yarn.n_freq
+    assert "n_freq" in _err()
+    assert lib.tllm_rope_bf16(None, None, 0, 64, 8, 63, C.byref(rope), None) == -2
+    qkv = lib.tllm_qkv_rope_decode_bf16
+    assert qkv(None, None, None, None, None, None, 4096, 512, 512, 0, 8, 2880, 64, 8, 64, None, None) == -1
+    assert qkv(None, None, None, None, None, None, 4096, 512, 512, 0, 8, 2880, 64, 8, 63, None, None) == -2
+    assert lib.tllm_yarn_table_f32(None, None, 0, 0, None, None) == -1
+
+
+def test_yarn_params_match_closed_form():
+    y = gpt_oss_yarn()
+    assert y.concentration == pytest.approx(1.3465735902799727, abs=1e-15)
+    assert len(y.inv_freq) == 32 and y.inv_freq[0] == 1.0
+    for i in (1, 5, 8):
+        assert y.inv_freq[i] == pytest.approx(150000.0 ** (-i / 32), rel=2e-6)
+    for i in (18, 25, 31):
+        assert y.inv_freq[i] == pytest.approx(150000.0 ** (-i / 32) / 32, rel=2e-6)
+    s = y.c_struct()
+    assert s.n_freq == 32 and s.inv_freq[3] == torch.tensor(y.inv_freq[3], dtype=torch.float32).item()
+    plain = YarnParams(head_dim=128, base=10000.0)
+    assert plain.concentration == 1.0 and plain.inv_freq[1] == pytest.approx(10000.0 ** (-2 / 128), rel=2e-6)
+    with pytest.raises(ValueError):
+        YarnParams(head_dim=63, base=10000.0)
+
+
+def test_yarn_params_agree_with_oracle_bitwise():
+    from oracle import layers as O
+
+    conc, inv = O.yarn_concentration_and_inv_freq()
+    y = gpt_oss_yarn()
+    assert conc == y.concentration
+    assert inv.tolist() == list(y.inv_freq)
+
+
+def test_ops_refuse_cpu_tensors():
+    import tritonllm_amd as T
+
+    x = torch.zeros(2, 2880, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        T.rmsnorm_forward(x, torch.ones(2880), 1e-5)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        T.swiglu(torch.zeros(2, 8, dtype=torch.bfloat16))
+
+
+def test_scratch_pool_returns_same_buffer():
+    from tritonllm_amd import scratch_pool
+
+    scratch_pool.clear()
+    a = scratch_pool.get((2, 3), torch.float32, torch.device("cpu"))
+    b = scratch_pool.get((2, 3), torch.float32, torch.device("cpu"))
+    c = scratch_pool.get((2, 4), torch.float32, torch.device("cpu"))
+    assert a.data_ptr() == b.data_ptr() and a.data_ptr() != c.data_ptr()
+    assert scratch_pool.stats()["num_buffers"] == 2
+    scratch_pool.clear()

@@ -1,0 +1,388 @@
+"""GPU parity: the HIP kernels (through ops -> ctypes -> C ABI) against the CPU oracle.
+
+Bar: bit-exact for the embedding gather; rtol 1.6e-2 / atol 1e-2 against the fp32-upcast
+oracle for every bf16 output. Inputs are the seeded synthetic tensors of the benchmark
+configurations plus edge cases (ragged rows, wrap-around positions, clamps, odd sizes).
+"""
+import pytest
+import torch
+
+import tritonllm_amd as T
+from oracle import layers as O
+from tritonllm_amd import scratch_pool
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1.6e-2, 1e-2
+
+
+def close(out, ref, rtol=RTOL, atol=ATOL):
+    torch.testing.assert_close(out.float().cpu(), ref.float(), rtol=rtol, atol=atol)
+
+
+@pytest.fixture(scope="module")
+def yarn():
+    return T.gpt_oss_yarn()
+
+
+# ----------------------------------------------------------------------------------- RMSNorm
+@pytest.mark.parametrize("rows", [1, 8, 32, 513, 2048, 8192])
+@pytest.mark.parametrize("scale_dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_parity(gpu, rows, scale_dtype):
+    d = O.make_inputs(rows, seed=rows, norm_scale_dtype=scale_dtype)
+    out = T.rmsnorm_forward(d["x"].to(gpu), d["norm_scale"].to(gpu), 1e-5)
+    assert out.dtype == torch.bfloat16 and out.shape == (rows, 2880)
+    close(out, O.rmsnorm_ref(d["x"], d["norm_scale"], 1e-5))
+
+
+def test_rmsnorm_in_place_leading_dims_and_pool(gpu):
+    d = O.make_inputs(24, seed=3)
+    x = d["x"].view(2, 12, 2880).to(gpu)
+    s = d["norm_scale"].float().to(gpu)
+    ref = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).view(2, 12, 2880)
+    a = T.rmsnorm_forward(x, s, 1e-5)
+    b = T.rmsnorm_forward(x, s, 1e-5)
+    assert a.data_ptr() == b.data_ptr()            # borrowed pool buffer, as the reference's scratch pool
+    close(a, ref)
+    r = T.rmsnorm_forward(x, s, 1e-5, out=x)       # final-norm style aliasing
+    assert r.data_ptr() == x.data_ptr()
+    close(x, ref)
+
+
+@pytest.mark.parametrize("hidden", [8, 40, 2881, 4096, 8192, 20000])
+def test_rmsnorm_other_hidden_sizes(gpu, hidden):
+    g = torch.Generator().manual_seed(hidden)
+    x = torch.randn(5, hidden, generator=g).bfloat16()
+    s = (1 + 0.1 * torch.randn(hidden, generator=g))
+    close(T.rmsnorm_forward(x.to(gpu), s.to(gpu), 1e-5), O.rmsnorm_ref(x, s, 1e-5))
+    many = torch.randn(700, hidden if hidden < 9000 else 512, generator=g).bfloat16()   # wave-per-row path
+    s2 = torch.ones(many.shape[1])
+    close(T.rmsnorm_forward(many.to(gpu), s2.to(gpu), 1e-5), O.rmsnorm_ref(many, s2, 1e-5))
+
+
+def test_rmsnorm_invariants_on_gpu(gpu):
+    x = torch.zeros(4, 2880, dtype=torch.bfloat16)
+    x[1] = 3.0
+    x[2] = -0.5
+    s = torch.linspace(0.5, 1.5, 2880)
+    out = T.rmsnorm_forward(x.to(gpu), s.to(gpu), 1e-5).float().cpu()
+    assert torch.all(out[0] == 0) and torch.all(out[3] == 0)
+    close(out[1], s / (1 + 1e-5 / 9.0) ** 0.5)
+    close(out[2], -s / (1 + 1e-5 / 0.25) ** 0.5)
+
+
+# ----------------------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("id_dtype", [torch.int32, torch.int64])
+def test_embedding_bit_exact_full_table(gpu, id_dtype):
+    g = torch.Generator().manual_seed(0)
+    table = torch.empty(O.VOCAB, O.HIDDEN, dtype=torch.bfloat16)
+    for lo in range(0, O.VOCAB, 25136):                      # chunked draw keeps host memory modest
+        table[lo:lo + 25136] = (0.02 * torch.randn(min(25136, O.VOCAB - lo), O.HIDDEN, generator=g)).bfloat16()
+    ids = torch.randint(0, O.VOCAB, (1, 2048), generator=g).to(id_dtype)
+    ids[0, 0], ids[0, 1], ids[0, 2], ids[0, 3] = 0, O.VOCAB - 1, 7, 7
+    out = T.embedding_forward(ids.to(gpu), table.to(gpu))
+    assert out.shape == (1, 2048, O.HIDDEN)
+    assert torch.equal(out.cpu(), O.embedding_ref(table, ids))
+
+
+def test_embedding_edges(gpu):
+    g = torch.Generator().manual_seed(1)
+    for hidden in (2880, 24, 7):                               # vector path, small vector path, scalar path
+        table = torch.randn(50, hidden, generator=g).bfloat16()
+        tg = table.to(gpu)
+        ids = torch.tensor([[0, 49], [3, 3]], dtype=torch.int64)
+        assert torch.equal(T.embedding_forward(ids.to(gpu), tg).cpu(), O.embedding_ref(table, ids))
+        empty = T.embedding_forward(torch.zeros((0,), dtype=torch.int32, device=gpu), tg)
+        assert empty.shape == (0, hidden)
+        flag = torch.zeros((), dtype=torch.int32, device=gpu)
+        bad = torch.tensor([1, 50, -1, 2], dtype=torch.int64)
+        out = T.embedding_forward(bad.to(gpu), tg, oob_flag=flag).cpu()
+        assert int(flag.item()) == 1
+        assert torch.equal(out[0], table[1]) and torch.equal(out[3], table[2])
+        assert torch.all(out[1] == 0) and torch.all(out[2] == 0)
+    emb = T.Embedding(50, 24, device=gpu)
+    with torch.no_grad():
+        emb.weight.copy_(torch.randn(50, 24, generator=g).bfloat16())
+    ids = torch.tensor([[4, 9]], dtype=torch.int32, device=gpu)
+    assert torch.equal(emb(ids).cpu(), emb.weight.detach().cpu()[[4, 9]][None])
+    emb.check_ids()
+    emb(torch.tensor([77], device=gpu))
+    with pytest.raises(IndexError):
+        emb.check_ids()
+
+
+# ----------------------------------------------------------------------------------- SwiGLU
+@pytest.mark.parametrize("rows", [4, 32, 128, 4096, 32768])
+def test_swiglu_parity(gpu, rows):
+    g = torch.Generator().manual_seed(rows)
+    x = (2.0 * torch.randn(rows, 5760, generator=g)).bfloat16()
+    out = T.swiglu(x.to(gpu))
+    assert out.shape == (rows, 2880)
+    close(out, O.swiglu_ref(x))
+
+
+def test_swiglu_edges_and_variants(gpu):
+    gs = [-30.0, -7.0, 0.0, 6.99, 7.0, 7.01, 30.0, -100.0]
+    ls = [-30.0, -7.01, -7.0, -1.0, 0.0, 7.0, 30.0, 1.0]
+    x = torch.tensor([[v for l in ls for v in (gv, l)] for gv in gs]).bfloat16()        # [8, 16] interleaved
+    out = T.swiglu(x.to(gpu))
+    close(out, O.swiglu_ref(x), rtol=1e-2, atol=1e-6)
+    assert torch.all(out.cpu()[:, ls.index(-1.0)] == 0)                                  # l = -1 => exact zero
+    g = torch.Generator().manual_seed(5)
+    y = (2.0 * torch.randn(3, 7, 48, generator=g)).bfloat16()
+    close(T.swiglu(y.to(gpu), interleaved=False), O.swiglu_ref(y, interleaved=False))
+    close(T.swiglu(y.to(gpu), alpha=1.0, limit=None), O.swiglu_ref(y, alpha=1.0, limit=None))
+    perm = torch.cat((y[..., ::2], y[..., 1::2]), dim=-1)
+    assert torch.equal(T.swiglu(y.to(gpu)).cpu(), T.swiglu(perm.to(gpu), interleaved=False).cpu())
+    odd = (2.0 * torch.randn(5, 2 * 13, generator=g)).bfloat16()                         # scalar path
+    close(T.swiglu(odd.to(gpu)), O.swiglu_ref(odd))
+    wide = (2.0 * torch.randn(6, 96, generator=g)).bfloat16().to(gpu)
+    close(T.swiglu(wide[:, :64]), O.swiglu_ref(wide.cpu()[:, :64]))                      # row stride > row length
+    from tritonllm_amd.swiglu import PrecisionConfig, swiglu as swiglu_pc
+    close(swiglu_pc(y.to(gpu), 1.702, PrecisionConfig(limit=7.0)), O.swiglu_ref(y))
+    nanrow = torch.tensor([[float("nan"), 1.0, 1.0, float("nan")]]).bfloat16()
+    assert torch.isnan(T.swiglu(nanrow.to(gpu))).all()
+
+
+# ----------------------------------------------------------------------------------- rotary
+def _qk(batch, tokens, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(batch, tokens, 64, 64, generator=g).bfloat16()
+    k = torch.randn(batch, tokens, 8, 64, generator=g).bfloat16()
+    return q, k
+
+
+@pytest.mark.parametrize("batch,tokens,offset", [(1, 1, 0), (8, 1, 4095), (2, 70, 4000), (1, 2048, 0), (1, 8192, 0), (1, 5, 131070)])
+def test_rope_parity_yarn_and_tables(gpu, yarn, batch, tokens, offset):
+    q, k = _qk(batch, tokens, seed=tokens + offset)
+    pos = O.token_positions(batch, tokens, offset)
+    cos, sin = O.yarn_cos_sin(pos)
+    q_ref = O.rope_rotate_ref(q.view(-1, 64, 64), cos, sin).view(q.shape)
+    k_ref = O.rope_rotate_ref(k.view(-1, 8, 64), cos, sin).view(k.shape)
+    off = torch.tensor([offset], dtype=torch.int64, device=gpu)
+    # in-register cos/sin
+    qg, kg = q.to(gpu), k.to(gpu)
+    T.rope_forward(qg, kg, None, None, O.MAX_CTX, off, yarn=yarn)
+    close(qg, q_ref)
+    close(kg, k_ref)
+    # table-driven, with the oracle's own tables (the reference's calling convention)
+    cos_t, sin_t = O.yarn_cos_sin(torch.arange(O.MAX_CTX))
+    qt, kt = q.to(gpu), k.to(gpu)
+    T.rope_forward(qt, kt, sin_t.to(gpu), cos_t.to(gpu), O.MAX_CTX, off)
+    close(qt, q_ref)
+    close(kt, k_ref)
+
+
+def test_rope_module_tables_and_per_row_positions(gpu, yarn):
+    rope = T.RotaryEmbedding(64, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, ntk_alpha=1.0,
+                             ntk_beta=32.0, device=gpu)
+    assert rope.cos.shape == (O.MAX_CTX, 32) and rope.cos.dtype == torch.float32
+    rows = torch.tensor([0, 1, 4095, 4096, 8191, 65537, 131071])
+    cos_ref, sin_ref = O.yarn_cos_sin(rows)
+    torch.testing.assert_close(rope.cos[rows.to(gpu)].cpu(), cos_ref, rtol=0, atol=1e-6)
+    torch.testing.assert_close(rope.sin[rows.to(gpu)].cpu(), sin_ref, rtol=0, atol=1e-6)
+    q, k = _qk(1, 33, seed=11)
+    off = torch.tensor([8000], dtype=torch.int64, device=gpu)
+    q1, k1 = q.to(gpu), k.to(gpu)
+    rope(q1, k1, off)                                      # tables carry YaRN parameters -> register path
+    q2, k2 = q.to(gpu), k.to(gpu)
+    T.rope_forward(q2, k2, rope.sin.clone(), rope.cos.clone(), O.MAX_CTX, off)   # plain tables -> table path
+    assert torch.equal(q1, q2) and torch.equal(k1, k2)     # same device routine either way
+    pos = torch.tensor([5, 8191, 0, 77777], dtype=torch.int64)
+    q, k = _qk(4, 1, seed=12)
+    cos, sin = O.yarn_cos_sin(pos)
+    qg, kg = q.to(gpu), k.to(gpu)
+    T.rope_forward(qg, kg, None, None, O.MAX_CTX, None, yarn=yarn, positions=pos.to(gpu))
+    close(qg, O.rope_rotate_ref(q.view(-1, 64, 64), cos, sin).view(q.shape))
+    close(kg, O.rope_rotate_ref(k.view(-1, 8, 64), cos, sin).view(k.shape))
+
+
+def test_rope_norm_property_full_size(gpu, yarn):
+    q, k = _qk(1, 8192, seed=13)
+    qg, kg = q.to(gpu), k.to(gpu)
+    T.rope_forward(qg, kg, None, None, O.MAX_CTX, torch.zeros(1, dtype=torch.int64, device=gpu), yarn=yarn)
+    n_in = q.float()[..., :32] ** 2 + q.float()[..., 32:] ** 2
+    n_out = qg.float().cpu()[..., :32] ** 2 + qg.float().cpu()[..., 32:] ** 2
+    torch.testing.assert_close(n_out, yarn.concentration ** 2 * n_in, rtol=3e-2, atol=3e-2)
+
+
+# ----------------------------------------------------------------------------------- fused QKV
+def _check_qkv(gpu, yarn, rows, mode, seed, prefill_positions=False, max_pos=8192):
+    d = O.make_inputs(rows, seed=seed, prefill=prefill_positions, max_pos=max_pos)
+    q, k, v = T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn,
+                                 positions=d["positions"].to(gpu), mode=mode)
+    qr, kr, vr = O.qkv_rope_ref(d["x"], d["w"], d["b"], d["positions"])
+    assert q.shape == (rows, 4096) and k.shape == (rows, 512) and v.shape == (rows, 512)
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+
+
+@pytest.mark.parametrize("rows", [1, 8, 15, 16, 17, 32, 50])
+def test_qkv_rope_decode_parity(gpu, yarn, rows):
+    _check_qkv(gpu, yarn, rows, "decode", seed=rows)
+
+
+@pytest.mark.parametrize("rows", [1, 100, 128, 200, 2048])
+def test_qkv_rope_prefill_parity(gpu, yarn, rows):
+    _check_qkv(gpu, yarn, rows, "prefill", seed=100 + rows, prefill_positions=rows >= 128)
+
+
+def test_qkv_rope_prefill_long_context(gpu, yarn):
+    _check_qkv(gpu, yarn, 8192, "prefill", seed=4, prefill_positions=True)
+
+
+def test_qkv_decode_and_prefill_agree(gpu, yarn):
+    d = O.make_inputs(40, seed=21)
+    args = (d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64)
+    kw = dict(yarn=yarn, positions=d["positions"].to(gpu))
+    qd, kd, vd = [t.clone() for t in T.qkv_rope_forward(*args, mode="decode", **kw)]
+    qp, kp, vp = T.qkv_rope_forward(*args, mode="prefill", **kw)
+    close(qd, qp.float().cpu())
+    close(kd, kp.float().cpu())
+    close(vd, vp.float().cpu())
+
+
+def test_qkv_offset_form_tables_and_no_rope(gpu, yarn):
+    d = O.make_inputs(12, seed=22)
+    xg, wg, bg = d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu)
+    off = torch.tensor([131070], dtype=torch.int64, device=gpu)
+    pos = O.token_positions(2, 6, 131070)
+    qr, kr, vr = O.qkv_rope_ref(d["x"], d["w"], d["b"], pos)
+    cos_t, sin_t = O.yarn_cos_sin(torch.arange(O.MAX_CTX))
+    for mode in ("decode", "prefill"):
+        q, k, v = T.qkv_rope_forward(xg, wg, bg, 64, 8, 64, yarn=yarn, offset=off, tokens_per_batch=6, mode=mode)
+        close(q, qr)
+        close(k, kr)
+        q, k, v = T.qkv_rope_forward(xg, wg, bg, 64, 8, 64, cos=cos_t.to(gpu), sin=sin_t.to(gpu), offset=off,
+                                     tokens_per_batch=6, mode=mode)
+        close(q, qr)
+        close(k, kr)
+        close(v, vr)
+        q, k, v = T.qkv_rope_forward(xg, wg, None, 64, 8, 64, rotate=False, mode=mode)
+        plain = O.linear_ref(d["x"], d["w"], None)
+        close(q, plain[:, :4096])
+        close(k, plain[:, 4096:4608])
+        close(v, plain[:, 4608:])
+
+
+def test_qkv_generic_shapes(gpu):
+    g = torch.Generator().manual_seed(23)
+    hidden, nq, nkv, hd = 100, 3, 1, 32                     # hidden % 32 != 0, head_dim != 64 -> generic kernel
+    x = torch.randn(5, hidden, generator=g).bfloat16()
+    w = (0.1 * torch.randn((nq + 2 * nkv) * hd, hidden, generator=g)).bfloat16()
+    b = (0.1 * torch.randn((nq + 2 * nkv) * hd, generator=g)).bfloat16()
+    y = T.YarnParams(head_dim=hd, base=10000.0)
+    pos = torch.tensor([0, 3, 17, 100, 4000], dtype=torch.int64)
+    qr, kr, vr = O.qkv_rope_ref(x, w, b, pos, nq, nkv, hd, base=10000.0, scaling_factor=1.0)
+    for mode in ("decode", "prefill"):
+        q, k, v = T.qkv_rope_forward(x.to(gpu), w.to(gpu), b.to(gpu), nq, nkv, hd, yarn=y, positions=pos.to(gpu), mode=mode)
+        close(q, qr)
+        close(k, kr)
+        close(v, vr)
+    # MFMA kernels at another K and head count (ragged last head tile, K loop with a tail)
+    hidden, nq, nkv, hd = 320, 6, 1, 64
+    x = torch.randn(150, hidden, generator=g).bfloat16()
+    w = (0.05 * torch.randn((nq + 2 * nkv) * hd, hidden, generator=g)).bfloat16()
+    b = (0.05 * torch.randn((nq + 2 * nkv) * hd, generator=g)).bfloat16()
+    pos = torch.randint(0, 8192, (150,), generator=g)
+    yy = T.gpt_oss_yarn()
+    qr, kr, vr = O.qkv_rope_ref(x, w, b, pos, nq, nkv, hd)
+    for mode, n in (("decode", 20), ("prefill", 150)):
+        q, k, v = T.qkv_rope_forward(x[:n].to(gpu), w.to(gpu), b.to(gpu), nq, nkv, hd, yarn=yy, positions=pos[:n].to(gpu), mode=mode)
+        close(q, qr[:n])
+        close(k, kr[:n])
+        close(v, vr[:n])
+
+
+def test_reference_signatures_decode_with_cache(gpu):
+    """qkv_rope_cache_decode_forward / qkv_decode_forward / QKV / RMSNorm modules as model.py calls them."""
+    scratch_pool.clear()
+    d = O.make_inputs(8, seed=31)
+    norm = T.RMSNorm(2880, device=gpu)
+    qkv = T.QKV(2880, 5120, device=gpu)
+    rope = T.RotaryEmbedding(64, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=gpu)
+    with torch.no_grad():
+        norm.scale.copy_(d["norm_scale"].float())
+        qkv.weight.copy_(d["w"])
+        qkv.bias.copy_(d["b"])
+    x = d["x"].view(8, 1, 2880).to(gpu)
+    t = norm(x)
+    t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"].float()).bfloat16()
+    n_ctx, slot = 64, 37
+    cache_k = torch.zeros(8, n_ctx, 8, 64, dtype=torch.bfloat16, device=gpu)
+    cache_v = torch.zeros_like(cache_k)
+    offset = torch.tensor([slot], dtype=torch.int64, device=gpu)
+    q = T.qkv_rope_cache_decode_forward(t, qkv.weight, qkv.bias, rope.sin, rope.cos, rope.max_context_length, cache_k, cache_v,
+                                        offset, 64, 8, 64)
+    assert q.shape == (8, 1, 4096)
+    pos = torch.full((8,), slot, dtype=torch.int64)
+    qr, kr, vr = O.qkv_rope_ref(t.cpu().view(8, 2880), d["w"], d["b"], pos)
+    close(q.view(8, 4096), qr)
+    close(cache_k[:, slot].reshape(8, 512), kr)
+    close(cache_v[:, slot].reshape(8, 512), vr)
+    mask = torch.ones(n_ctx, dtype=torch.bool)
+    mask[slot] = False
+    assert torch.all(cache_k.cpu()[:, mask] == 0) and torch.all(cache_v.cpu()[:, mask] == 0)   # nothing else touched
+    close(t.view(8, 2880), t_ref.float())
+    # unfused decode + F.linear-style forward
+    qd, kd, vd = qkv.decode(t, 4096, 512)
+    assert qd.shape == (8, 1, 4096) and kd.shape == (8, 1, 512)
+    plain = O.linear_ref(t.cpu().view(8, 2880), d["w"], d["b"])
+    close(qd.view(8, 4096), plain[:, :4096])
+    close(kd.view(8, 512), plain[:, 4096:4608])
+    close(vd.view(8, 512), plain[:, 4608:])
+    full = qkv(t)
+    assert full.shape == (8, 1, 5120)
+    close(full.view(8, 5120), plain)
+    seq = O.make_inputs(300, seed=32)["x"].view(1, 300, 2880)
+    close(qkv(seq.to(gpu)).view(300, 5120), O.linear_ref(seq.view(300, 2880), d["w"], d["b"]))
+    # fused prefill through the module
+    qf, kf, vf = qkv.forward_rope(seq.to(gpu), rope, 64, 8, offset=torch.tensor([10], dtype=torch.int64, device=gpu))
+    qr, kr, vr = O.qkv_rope_ref(seq.view(300, 2880), d["w"], d["b"], O.token_positions(1, 300, 10))
+    close(qf.reshape(300, 4096), qr)
+    close(kf.reshape(300, 512), kr)
+    close(vf.reshape(300, 512), vr)
+    with pytest.raises(NotImplementedError):
+        T.qkv_rope_cache_decode_forward(t, qkv.weight, qkv.bias, rope.sin, rope.cos, rope.max_context_length, cache_k, cache_v,
+                                        offset, 64, 8, 64, weight_scale=torch.ones(5120, device=gpu))
+    with pytest.raises(AssertionError):
+        T.qkv_decode_forward(torch.zeros(8, 2, 2880, dtype=torch.bfloat16, device=gpu), qkv.weight, qkv.bias, 4096, 512)
+
+
+def test_qkv_linearity_full_size(gpu):
+    """Size-independent property at T=8192 without the oracle: the projection is linear in x."""
+    g = torch.Generator().manual_seed(41)
+    x1 = torch.randn(8192, 2880, generator=g).bfloat16().to(gpu)
+    w = (0.02 * torch.randn(5120, 2880, generator=g)).bfloat16().to(gpu)
+    y1 = [t.float() for t in T.qkv_rope_forward(x1, w, None, 64, 8, 64, rotate=False, mode="prefill")]
+    y2 = [t.float() for t in T.qkv_rope_forward((2 * x1), w, None, 64, 8, 64, rotate=False, mode="prefill")]
+    for a, b in zip(y1, y2):
+        torch.testing.assert_close(b, 2 * a, rtol=1.6e-2, atol=1e-2)
+
+
+def test_graph_replay_reads_positions_from_device(gpu, yarn):
+    """Capture the decode chain once, replay with new positions: results must follow the device-side offset."""
+    d = O.make_inputs(8, seed=51)
+    xg, wg, bg, sg = d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), d["norm_scale"].to(gpu)
+    offset = torch.zeros(1, dtype=torch.int64, device=gpu)
+    outs = {}
+
+    def chain():
+        t = T.rmsnorm_forward(xg, sg, 1e-5)
+        outs["q"], outs["k"], outs["v"] = T.qkv_rope_forward(t, wg, bg, 64, 8, 64, yarn=yarn, offset=offset, tokens_per_batch=1,
+                                                              mode="decode")
+
+    chain()                                       # warm up (allocates pool buffers)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain()
+    t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"]).bfloat16()
+    for p in (0, 4097, 8191):
+        offset.fill_(p)
+        graph.replay()
+        torch.cuda.synchronize()
+        qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], torch.full((8,), p, dtype=torch.int64))
+        close(outs["q"], qr, rtol=3e-2, atol=2e-2)   # t_ref is the oracle's rounding of the norm, the GPU's may differ by one bf16 ulp
+        close(outs["k"], kr, rtol=3e-2, atol=2e-2)

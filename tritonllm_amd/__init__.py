@@ -1,0 +1,22 @@
+"""MI355X-native gpt-oss layer kernels: RMSNorm, fused QKV + bias + YaRN rotary,
+clamped SwiGLU and the token-embedding gather, as hand-written HIP for gfx950 behind a
+C ABI (``include/tllm_hip.h``) with the reference model's Python call signatures on top."""
+from . import scratch_pool
+from .modules import QKV, Embedding, RMSNorm, RotaryEmbedding
+from .ops import (
+    embedding_forward,
+    linear_qkv_forward,
+    qkv_decode_forward,
+    qkv_rope_cache_decode_forward,
+    qkv_rope_forward,
+    rmsnorm_forward,
+    rope_forward,
+    swiglu,
+)
+from .yarn import YarnParams, gpt_oss_yarn
+
+__all__ = [
+    "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
+    "embedding_forward", "linear_qkv_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
+    "qkv_rope_forward", "rmsnorm_forward", "rope_forward", "swiglu",
+]

@@ -1,0 +1,104 @@
+// Shared device/host helpers for the gfx950 layer kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tllm_hip.h"
+
+namespace tllm {
+
+typedef __bf16 bf16;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;   // 16 bytes
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;   // 8 bytes
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;   // 4 bytes
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+constexpr int kWave = 64;
+
+// ---- host side error plumbing (abi.hip owns the storage) -------------------
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+#define TLLM_REQUIRE(cond, code, ...)      \
+  do {                                     \
+    if (!(cond)) {                         \
+      ::tllm::set_error(__VA_ARGS__);      \
+      return (code);                       \
+    }                                      \
+  } while (0)
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- device helpers --------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Kernel-argument copy of the rotary source (TllmRope with the YaRN block by value).
+struct RopeArgs {
+  const float* cos_table;
+  const float* sin_table;
+  int64_t table_row_stride;
+  const int64_t* positions;
+  const int64_t* offset;
+  int64_t tokens_per_batch;
+  int64_t max_ctx;
+  float concentration;
+  int n_freq;
+  int use_yarn;
+};
+
+struct YarnFreqs {
+  float v[TLLM_MAX_ROPE_FREQS];
+};
+
+// Unwrapped position of a row: only loads and an add, so it can be issued early.
+__device__ __forceinline__ int64_t rope_position_raw(const RopeArgs& r, int64_t row) {
+  if (r.positions) return r.positions[row];
+  int64_t p = row % r.tokens_per_batch;
+  if (r.offset) p += r.offset[0];
+  return p;
+}
+
+// Wrap into [0, max_ctx). The common case is already in range and skips the 64-bit division.
+__device__ __forceinline__ int64_t rope_wrap(int64_t p, int64_t max_ctx) {
+  if (static_cast<uint64_t>(p) >= static_cast<uint64_t>(max_ctx)) {
+    p %= max_ctx;
+    if (p < 0) p += max_ctx;
+  }
+  return p;
+}
+
+__device__ __forceinline__ int64_t rope_position(const RopeArgs& r, int64_t row) {
+  return rope_wrap(rope_position_raw(r, row), r.max_ctx);
+}
+
+// cos/sin of the rotary angle for (position, frequency index), scaled by the
+// concentration. The angle is the single fp32 product float(pos) * inv_freq,
+// exactly as the reference's table construction forms it; sincosf is the
+// full-range routine (angles reach 1.3e5 rad), never the fast intrinsics.
+__device__ __forceinline__ void yarn_cos_sin(int64_t pos, float inv_freq, float concentration, float* c, float* s) {
+  float angle = __fmul_rn(static_cast<float>(pos), inv_freq);
+  float sv, cv;
+  sincosf(angle, &sv, &cv);
+  *c = cv * concentration;
+  *s = sv * concentration;
+}
+
+__device__ __forceinline__ void rope_cos_sin(const RopeArgs& r, const YarnFreqs& f, int64_t pos, int i, float* c, float* s) {
+  if (r.use_yarn) {
+    yarn_cos_sin(pos, f.v[i], r.concentration, c, s);
+  } else {
+    *c = r.cos_table[pos * r.table_row_stride + i];
+    *s = r.sin_table[pos * r.table_row_stride + i];
+  }
+}
+
+// Host: validate a TllmRope and flatten it into kernel arguments.
+int make_rope_args(const TllmRope* rope, int head_dim, RopeArgs* out, YarnFreqs* freqs);
+
+}  // namespace tllm

@@ -1,0 +1,77 @@
+// Token-embedding gather: out[t, :] = table[ids[t], :], a bit-exact row copy.
+//
+// Memory-bound random-row reads: each 64-lane wavefront copies one 5760-byte row
+// (gpt-oss) as 128-bit vectors, so a row is one burst of contiguous 1 KiB requests;
+// a grid-stride loop over tokens keeps every CU busy for long sequences.
+#include "common.h"
+
+namespace tllm {
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void embedding_vec_kernel(const bf16x8* __restrict__ table, const IdT* __restrict__ ids,
+                                                            bf16x8* __restrict__ out, int64_t n_tokens, int nvec, int64_t vocab,
+                                                            int32_t* oob_flag) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave0 = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * 4;
+  for (int64_t t = wave0; t < n_tokens; t += nwaves) {
+    const int64_t id = static_cast<int64_t>(ids[t]);
+    bf16x8* dst = out + t * nvec;
+    if (id >= 0 && id < vocab) {
+      const bf16x8* src = table + id * nvec;
+      for (int i = lane; i < nvec; i += 64) dst[i] = src[i];
+    } else {
+      bf16x8 z;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) z[j] = static_cast<bf16>(0.f);
+      for (int i = lane; i < nvec; i += 64) dst[i] = z;
+      if (oob_flag && lane == 0) *oob_flag = 1;
+    }
+  }
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void embedding_scalar_kernel(const uint16_t* __restrict__ table, const IdT* __restrict__ ids,
+                                                               uint16_t* __restrict__ out, int64_t n_tokens, int64_t hidden,
+                                                               int64_t vocab, int32_t* oob_flag) {
+  for (int64_t t = blockIdx.x; t < n_tokens; t += gridDim.x) {
+    const int64_t id = static_cast<int64_t>(ids[t]);
+    const bool ok = id >= 0 && id < vocab;
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) out[t * hidden + c] = ok ? table[id * hidden + c] : uint16_t(0);
+    if (!ok && oob_flag && threadIdx.x == 0) *oob_flag = 1;
+  }
+}
+
+}  // namespace tllm
+
+using namespace tllm;
+
+extern "C" int tllm_embedding_bf16(const void* table, const void* ids, int ids_is_i64, void* out, int64_t n_tokens, int64_t hidden,
+                                   int64_t vocab, int32_t* oob_flag, void* stream) {
+  TLLM_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, TLLM_E_ARG, "embedding: n_tokens %lld / hidden %lld / vocab %lld invalid",
+               (long long)n_tokens, (long long)hidden, (long long)vocab);
+  if (n_tokens == 0) return TLLM_OK;
+  TLLM_REQUIRE(table && ids && out, TLLM_E_ARG, "embedding: null pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec_ok = hidden % 8 == 0 && aligned16(table) && aligned16(out) && hidden / 8 < (1ll << 31);
+  if (vec_ok) {
+    const int64_t blocks = (n_tokens + 3) / 4;
+    dim3 grid(static_cast<unsigned>(blocks < 16384 ? blocks : 16384)), block(256);
+    const int nvec = static_cast<int>(hidden / 8);
+    if (ids_is_i64)
+      hipLaunchKernelGGL(embedding_vec_kernel<int64_t>, grid, block, 0, st, (const bf16x8*)table, (const int64_t*)ids, (bf16x8*)out,
+                         n_tokens, nvec, vocab, oob_flag);
+    else
+      hipLaunchKernelGGL(embedding_vec_kernel<int32_t>, grid, block, 0, st, (const bf16x8*)table, (const int32_t*)ids, (bf16x8*)out,
+                         n_tokens, nvec, vocab, oob_flag);
+  } else {
+    dim3 grid(static_cast<unsigned>(n_tokens < 65536 ? n_tokens : 65536)), block(256);
+    if (ids_is_i64)
+      hipLaunchKernelGGL(embedding_scalar_kernel<int64_t>, grid, block, 0, st, (const uint16_t*)table, (const int64_t*)ids,
+                         (uint16_t*)out, n_tokens, hidden, vocab, oob_flag);
+    else
+      hipLaunchKernelGGL(embedding_scalar_kernel<int32_t>, grid, block, 0, st, (const uint16_t*)table, (const int32_t*)ids,
+                         (uint16_t*)out, n_tokens, hidden, vocab, oob_flag);
+  }
+  return check_launch("embedding");
+}

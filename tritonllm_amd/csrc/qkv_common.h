@@ -1,0 +1,43 @@
+// Pieces shared by the decode and prefill QKV kernels: argument block, host-side
+// validation, the output-row addressing, and the shape-generic fallback kernel.
+#pragma once
+
+#include "common.h"
+
+namespace tllm {
+
+struct QkvArgs {
+  const bf16* x;
+  const bf16* W;
+  const bf16* bias;   // may be null
+  bf16* q;
+  bf16* k;
+  bf16* v;
+  int64_t q_rs, k_rs, v_rs;   // elements between consecutive rows of q / k / v
+  int64_t kv_slot_stride;     // elements per KV-cache slot (0: no slot offset)
+  int64_t rows;
+  int hidden;
+  int n_q_heads, n_kv_heads, head_dim;
+  int has_rope;
+};
+
+// Start of head `head` (0 .. n_q + 2 n_kv) of output row `row`.
+__device__ __forceinline__ bf16* qkv_out_ptr(const QkvArgs& a, const RopeArgs& ra, int64_t row, int head) {
+  int64_t slot = 0;
+  if (a.kv_slot_stride != 0 && ra.offset != nullptr) slot = ra.offset[0];
+  if (head < a.n_q_heads) return a.q + row * a.q_rs + static_cast<int64_t>(head) * a.head_dim;
+  head -= a.n_q_heads;
+  if (head < a.n_kv_heads) return a.k + row * a.k_rs + slot * a.kv_slot_stride + static_cast<int64_t>(head) * a.head_dim;
+  head -= a.n_kv_heads;
+  return a.v + row * a.v_rs + slot * a.kv_slot_stride + static_cast<int64_t>(head) * a.head_dim;
+}
+
+int qkv_validate(const char* who, const void* x, const void* W, const void* q, const void* k, const void* v, int64_t q_rs,
+                 int64_t k_rs, int64_t v_rs, int64_t kv_slot_stride, int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads,
+                 int head_dim, const TllmRope* rope, QkvArgs* a, RopeArgs* ra, YarnFreqs* fr);
+
+// Any hidden size, any even head_dim: one workgroup per (head, row); each wavefront takes
+// rotation pairs (d, d + hd/2) in turn and reduces the two dot products by shuffle.
+void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, hipStream_t st);
+
+}  // namespace tllm

@@ -1,0 +1,323 @@
+"""The gpt-oss layer ops, with the call signatures the reference model code uses.
+
+Each function validates its tensors the way the reference does (``assert`` on shape
+preconditions, ``.contiguous()`` on a strided last dim), takes raw device pointers and
+hands them to ``libtllm_hip.so`` on the current PyTorch HIP stream. PyTorch is plumbing
+here -- memory, streams, dtypes; all arithmetic happens in the HIP kernels. There is no
+CPU path: tensors must live on the GPU and the shared library must be built.
+
+Reference signatures (paths under ``tritonllm/gpt_oss/triton/``):
+
+    rmsnorm_forward(x, scale, eps, out=None)                         triton_kernels.py:28
+    rope_forward(query, key, sin, cos, max_context_length, offset)   triton_kernels.py:90
+    qkv_decode_forward(hidden, weight, bias, q_dim, kv_dim)          triton_kernels.py:615
+    qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_length,
+        cache_k, cache_v, offset, num_q_heads, num_kv_heads, head_dim,
+        weight_scale=None)                                           triton_kernels.py:1109
+    swiglu(x, alpha=1.702, limit=7.0, interleaved=True)              moe.py:25
+    embedding: torch.nn.Embedding.forward                            model.py:906-920
+
+Outputs that the reference takes from its scratch pool are taken from
+``tritonllm_amd.scratch_pool`` here, with the same borrowed-buffer semantics.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import scratch_pool
+from ._lib import TllmRope, check, lib
+from .yarn import YarnParams
+
+_BF16 = torch.bfloat16
+
+# rows at or below this use the weight-streaming decode kernel, above it the MFMA GEMM
+DECODE_MAX_ROWS = 64
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _on_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("tritonllm_amd ops run on the GPU only (got a CPU tensor); there is no CPU fallback")
+
+
+def _yarn_of(t) -> YarnParams | None:
+    return getattr(t, "_tllm_yarn", None)
+
+
+def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, keep: list) -> TllmRope:
+    """Fill the C descriptor of where the rotary angles come from. ``keep`` collects
+    objects that must stay alive until the launch call has returned."""
+    r = TllmRope()
+    if yarn is None and cos is not None:
+        yarn = _yarn_of(cos)
+        if yarn is not None and _yarn_of(sin) is not yarn:
+            yarn = None
+    if yarn is not None:
+        r.yarn = yarn.c_pointer()
+        keep.append(yarn)
+    else:
+        assert cos is not None and sin is not None, "rotary needs YaRN parameters or cos/sin tables"
+        assert cos.dtype == torch.float32 and sin.dtype == torch.float32
+        assert cos.ndim == 2 and cos.shape == sin.shape
+        if cos.stride(-1) != 1:
+            cos = cos.contiguous()
+        if sin.stride(-1) != 1 or sin.stride(0) != cos.stride(0):
+            sin = sin.contiguous()
+            cos = cos.contiguous()
+        assert cos.shape[0] >= max_ctx, "cos/sin tables shorter than max_context_length"
+        keep += [cos, sin]
+        r.cos_table = cos.data_ptr()
+        r.sin_table = sin.data_ptr()
+        r.table_row_stride = cos.stride(0)
+    if positions is not None:
+        assert positions.dtype == torch.int64 and positions.is_contiguous()
+        r.positions = positions.data_ptr()
+    if offset is not None:
+        assert offset.dtype == torch.int64 and offset.numel() == 1
+        r.offset = offset.data_ptr()
+    r.tokens_per_batch = int(tokens_per_batch)
+    r.max_ctx = int(max_ctx)
+    return r
+
+
+# --------------------------------------------------------------------------------------- RMSNorm
+def rmsnorm_forward(x: torch.Tensor, scale: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``y = x * rsqrt(mean(x^2) + eps) * scale`` over the last dim; ``out`` may alias ``x``."""
+    _on_gpu(x, scale, out)
+    assert x.dtype == _BF16, "rmsnorm_forward: x must be bfloat16"
+    assert scale.dtype in (torch.float32, _BF16), "rmsnorm_forward: scale must be float32 or bfloat16"
+    hidden = x.shape[-1]
+    assert scale.shape == (hidden,)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    if not scale.is_contiguous():
+        scale = scale.contiguous()
+    if out is None:
+        out = scratch_pool.get(tuple(x.shape), x.dtype, x.device)
+    assert out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()
+    rows = x.numel() // hidden if hidden else 0
+    rc = lib().tllm_rmsnorm_bf16(x.data_ptr(), scale.data_ptr(), int(scale.dtype == _BF16), out.data_ptr(), rows, hidden,
+                                 float(eps), _stream())
+    check(rc, "rmsnorm_forward")
+    return out
+
+
+# --------------------------------------------------------------------------------------- embedding
+def embedding_forward(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None,
+                      oob_flag: torch.Tensor | None = None) -> torch.Tensor:
+    """``out[..., :] = table[ids[...], :]`` (bit-exact). ids int32 or int64, any shape.
+
+    An id outside ``[0, vocab)`` produces a zero row and sets ``oob_flag`` (int32 device
+    scalar) to 1 when one is given -- never a device fault."""
+    _on_gpu(ids, table, out, oob_flag)
+    assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
+    assert ids.dtype in (torch.int32, torch.int64)
+    if not ids.is_contiguous():
+        ids = ids.contiguous()
+    vocab, hidden = table.shape
+    shape = (*ids.shape, hidden)
+    if out is None:
+        out = scratch_pool.get(shape, table.dtype, table.device)
+    assert tuple(out.shape) == shape and out.dtype == table.dtype and out.is_contiguous()
+    if oob_flag is not None:
+        assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
+    rc = lib().tllm_embedding_bf16(table.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64), out.data_ptr(), ids.numel(),
+                                   hidden, vocab, oob_flag.data_ptr() if oob_flag is not None else None, _stream())
+    check(rc, "embedding_forward")
+    return out
+
+
+# --------------------------------------------------------------------------------------- SwiGLU
+def swiglu(x: torch.Tensor, alpha: float = 1.702, limit: float | None = 7.0, interleaved: bool = True,
+           out: torch.Tensor | None = None) -> torch.Tensor:
+    """Clamped SwiGLU over the last dim: ``[..., 2n] -> [..., n]``."""
+    _on_gpu(x, out)
+    assert x.dtype == _BF16, "swiglu: x must be bfloat16"
+    assert x.shape[-1] % 2 == 0
+    n_out = x.shape[-1] // 2
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    x2 = x.reshape(-1, x.shape[-1]) if x.ndim != 2 else x
+    if x2.ndim == 2 and x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    shape = (*x.shape[:-1], n_out)
+    if out is None:
+        out = torch.empty(shape, dtype=x.dtype, device=x.device)
+    assert tuple(out.shape) == shape and out.dtype == x.dtype and out.is_contiguous()
+    row_stride = x2.stride(0) if rows > 1 else 2 * n_out
+    rc = lib().tllm_swiglu_bf16(x2.data_ptr(), out.data_ptr(), rows, n_out, row_stride, float(alpha),
+                                float(limit) if limit is not None else 0.0, int(limit is not None), int(bool(interleaved)), _stream())
+    check(rc, "swiglu")
+    return out
+
+
+# --------------------------------------------------------------------------------------- rotary
+def rope_forward(query: torch.Tensor, key: torch.Tensor, sin: torch.Tensor | None, cos: torch.Tensor | None,
+                 max_context_length: int, offset: torch.Tensor | None, *, yarn: YarnParams | None = None,
+                 positions: torch.Tensor | None = None) -> None:
+    """In-place rotary on ``query [B, T, Hq, D]`` and ``key [B, T, Hkv, D]``.
+
+    Token ``t`` of every batch row sits at position ``(t + offset) % max_context_length``.
+    ``sin``/``cos`` are the fp32 ``[max_ctx, D/2]`` tables; tables produced by
+    :class:`tritonllm_amd.modules.RotaryEmbedding` carry their YaRN parameters and the
+    kernel then computes cos/sin in registers instead of reading them. Extensions over
+    the reference: ``yarn=`` to pass parameters without tables, ``positions=`` (int64
+    ``[B*T]``) for an independent position per row."""
+    _on_gpu(query, key, offset, positions)
+    batch_size, num_tokens, num_heads, head_dim = query.shape
+    kb, kt, num_key_value_heads, khd = key.shape
+    assert (kb, kt, khd) == (batch_size, num_tokens, head_dim)
+    assert query.dtype == _BF16 and key.dtype == _BF16
+    assert query.is_contiguous() and key.is_contiguous(), "rope_forward rotates in place and needs dense q/k"
+    keep: list = []
+    desc = _rope_desc(cos, sin, yarn, positions, offset, num_tokens, max_context_length, keep)
+    rc = lib().tllm_rope_bf16(query.data_ptr(), key.data_ptr(), batch_size * num_tokens, num_heads, num_key_value_heads, head_dim,
+                              C.byref(desc), _stream())
+    check(rc, "rope_forward")
+
+
+# --------------------------------------------------------------------------------------- fused QKV
+def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_stride, n_q, n_kv, hd, desc):
+    fn = lib().tllm_qkv_rope_decode_bf16 if kind == "decode" else lib().tllm_qkv_rope_prefill_bf16
+    rc = fn(x2.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
+            q.data_ptr() if q is not None else None, k.data_ptr() if k is not None else None,
+            v.data_ptr() if v is not None else None, q_rs, k_rs, v_rs, kv_slot_stride, x2.shape[0], x2.shape[1], n_q, n_kv, hd,
+            C.byref(desc) if desc is not None else None, _stream())
+    check(rc, f"qkv_rope_{kind}")
+
+
+def _prep_linear(hidden2, weight, bias):
+    assert hidden2.dtype == _BF16 and weight.dtype == _BF16 and (bias is None or bias.dtype == _BF16)
+    if not hidden2.is_contiguous():
+        hidden2 = hidden2.contiguous()
+    if not weight.is_contiguous():
+        weight = weight.contiguous()
+    if bias is not None and not bias.is_contiguous():
+        bias = bias.contiguous()
+    return hidden2, weight, bias
+
+
+def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, num_q_heads: int, num_kv_heads: int,
+                     head_dim: int, *, yarn: YarnParams | None = None, cos: torch.Tensor | None = None,
+                     sin: torch.Tensor | None = None, positions: torch.Tensor | None = None, offset: torch.Tensor | None = None,
+                     tokens_per_batch: int | None = None, max_context_length: int = 131072, rotate: bool = True,
+                     mode: str = "auto", out: tuple | None = None):
+    """RMS-normed activations ``x [rows, hidden]`` -> ``(q [rows, Hq*D], k [rows, Hkv*D], v [rows, Hkv*D])``.
+
+    One fused kernel: projection, bias, rotary on q/k (fp32 accumulator, one rounding),
+    outputs written to three dense tensors. ``mode``: "decode" (weight streaming),
+    "prefill" (MFMA GEMM) or "auto" (by row count). No reference twin as a single call:
+    it is F.linear + split + contiguous + rope_forward of model.py:506-522 in one launch."""
+    _on_gpu(x, weight, bias, positions, offset, cos, sin)
+    assert x.ndim == 2
+    rows, hidden = x.shape
+    total_out, hidden_w = weight.shape
+    assert hidden == hidden_w
+    assert total_out == (num_q_heads + 2 * num_kv_heads) * head_dim
+    assert bias is None or bias.shape == (total_out,)
+    x, weight, bias = _prep_linear(x, weight, bias)
+    q_dim, kv_dim = num_q_heads * head_dim, num_kv_heads * head_dim
+    if out is None:
+        q = scratch_pool.get((rows, q_dim), x.dtype, x.device)
+        kv = scratch_pool.get((2, rows, kv_dim), x.dtype, x.device)   # k and v share a shape: one buffer, two halves
+        k, v = kv[0], kv[1]
+    else:
+        q, k, v = out
+        assert q.shape == (rows, q_dim) and k.shape == (rows, kv_dim) and v.shape == (rows, kv_dim)
+        assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1
+    keep: list = []
+    desc = None
+    if rotate:
+        desc = _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch if tokens_per_batch else max(rows, 1),
+                          max_context_length, keep)
+    if mode == "auto":
+        mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
+    assert mode in ("decode", "prefill")
+    _launch_qkv(mode, x, weight, bias, q, k, v, q.stride(0), k.stride(0), v.stride(0), 0, num_q_heads, num_kv_heads, head_dim, desc)
+    return q, k, v
+
+
+def _split_head_dim(q_dim: int, kv_dim: int) -> int:
+    """A head size that tiles both q_dim and kv_dim (no rotation: any even tiling will do)."""
+    if q_dim % 64 == 0 and kv_dim % 64 == 0:
+        return 64
+    g = math.gcd(q_dim, kv_dim)
+    assert g % 2 == 0, "q_dim and kv_dim need a common even divisor"
+    return g
+
+
+def qkv_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, q_dim: int, kv_dim: int):
+    """Unfused decode projection: ``[B,1,H] -> q [B,1,q_dim], k, v [B,1,kv_dim]`` (no rotary)."""
+    _on_gpu(hidden, weight, bias)
+    batch, num_tokens, hidden_size = hidden.shape
+    total_out, hidden_size_weight = weight.shape
+    assert num_tokens == 1
+    assert hidden_size == hidden_size_weight
+    assert bias.shape == (total_out,)
+    assert total_out == q_dim + 2 * kv_dim
+    x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
+    hd = _split_head_dim(q_dim, kv_dim)
+    q = scratch_pool.get((batch, q_dim), hidden.dtype, hidden.device)
+    kv = scratch_pool.get((2, batch, kv_dim), hidden.dtype, hidden.device)
+    k, v = kv[0], kv[1]
+    _launch_qkv("decode", x2, weight, bias, q, k, v, q_dim, kv_dim, kv_dim, 0, q_dim // hd, kv_dim // hd, hd, None)
+    return q[:, None, :], k[:, None, :], v[:, None, :]
+
+
+def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_length, cache_k, cache_v, offset, num_q_heads,
+                                  num_kv_heads, head_dim, weight_scale=None, *, yarn: YarnParams | None = None,
+                                  positions: torch.Tensor | None = None):
+    """Fused decode step: projection + bias + rotary; the rotated k and the raw v of the
+    new token are written into the KV cache at slot ``offset``; q ``[B,1,Hq*D]`` is returned
+    (a borrowed pool buffer). ``offset`` is an int64 device tensor of shape (1,) and is read
+    on the device, so the call can be replayed from a HIP graph."""
+    _on_gpu(hidden, weight, bias, cache_k, cache_v, offset, positions)
+    if weight_scale is not None:
+        raise NotImplementedError("fp8 weights with per-row scales are not implemented in the HIP path")
+    batch, num_tokens, hidden_size = hidden.shape
+    total_out, hidden_size_weight = weight.shape
+    assert num_tokens == 1
+    assert hidden_size == hidden_size_weight
+    assert total_out == (num_q_heads + 2 * num_kv_heads) * head_dim
+    assert bias.shape == (total_out,)
+    assert cache_k.shape == cache_v.shape
+    assert cache_k.shape[0] == batch
+    assert cache_k.shape[2] == num_kv_heads
+    assert cache_k.shape[3] == head_dim
+    assert offset.shape == (1,)
+    assert cache_k.dtype == _BF16 and cache_v.dtype == _BF16
+    assert cache_k.stride() == cache_v.stride()
+    assert cache_k.stride(3) == 1 and cache_k.stride(2) == head_dim, "KV cache must be dense over (heads, head_dim)"
+    x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
+    q = scratch_pool.get((batch, num_q_heads, head_dim), hidden.dtype, hidden.device)
+    keep: list = []
+    desc = _rope_desc(cos, sin, yarn, positions, offset, 1, max_context_length, keep)
+    _launch_qkv("decode", x2, weight, bias, q, cache_k, cache_v, num_q_heads * head_dim, cache_k.stride(0), cache_v.stride(0),
+                cache_k.stride(1), num_q_heads, num_kv_heads, head_dim, desc)
+    return q.reshape(batch, 1, num_q_heads * head_dim)
+
+
+def linear_qkv_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` for the QKV weight (model.py:136-138): ``[..., H] -> [..., qkv_dim]``
+    through the MFMA kernel (or the streaming kernel for few rows), writing one dense output."""
+    _on_gpu(x, weight, bias)
+    total_out, hidden = weight.shape
+    assert x.shape[-1] == hidden
+    x2, weight, bias = _prep_linear(x.reshape(-1, hidden), weight, bias)
+    rows = x2.shape[0]
+    hd = 64 if total_out % 64 == 0 else 2
+    assert total_out % hd == 0
+    out = torch.empty((*x.shape[:-1], total_out), dtype=x.dtype, device=x.device)
+    o2 = out.view(rows, total_out)
+    mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
+    # all columns as "q heads" of one dense output row
+    _launch_qkv(mode, x2, weight, bias, o2, None, None, total_out, 0, 0, 0, total_out // hd, 0, hd, None)
+    return out
