@@ -138,7 +138,7 @@ def test_swiglu_edges_and_variants(gpu):
     close(T.swiglu(odd.to(gpu)), O.swiglu_ref(odd))
     wide = (2.0 * torch.randn(6, 96, generator=g)).bfloat16().to(gpu)
     close(T.swiglu(wide[:, :64]), O.swiglu_ref(wide.cpu()[:, :64]))                      # row stride > row length
-    from tritonllm_amd.swiglu import PrecisionConfig, swiglu as swiglu_pc
+    from tritonllm_amd.swiglu_compat import PrecisionConfig, swiglu as swiglu_pc
     close(swiglu_pc(y.to(gpu), 1.702, PrecisionConfig(limit=7.0)), O.swiglu_ref(y))
     nanrow = torch.tensor([[float("nan"), 1.0, 1.0, float("nan")]]).bfloat16()
     assert torch.isnan(T.swiglu(nanrow.to(gpu))).all()

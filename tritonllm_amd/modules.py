@@ -122,8 +122,7 @@ class Embedding(torch.nn.Module):
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         if self._oob is None or self._oob.device != self.weight.device:
             self._oob = torch.zeros((), dtype=torch.int32, device=self.weight.device)
-        out = torch.empty((*ids.shape, self.embedding_dim), dtype=self.weight.dtype, device=self.weight.device)
-        return ops.embedding_forward(ids, self.weight, out=out, oob_flag=self._oob)
+        return ops.embedding_forward(ids, self.weight, oob_flag=self._oob)
 
     def check_ids(self) -> None:
         """Synchronising check: raise IndexError if any id seen so far was out of range."""

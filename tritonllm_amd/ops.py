@@ -124,7 +124,7 @@ def embedding_forward(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor 
     vocab, hidden = table.shape
     shape = (*ids.shape, hidden)
     if out is None:
-        out = scratch_pool.get(shape, table.dtype, table.device)
+        out = torch.empty(shape, dtype=table.dtype, device=table.device)   # a fresh tensor, as nn.Embedding returns
     assert tuple(out.shape) == shape and out.dtype == table.dtype and out.is_contiguous()
     if oob_flag is not None:
         assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
