@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the gpt-oss layer-kernel path on one MI355X.
+
+A *step* is one pass of the hot path over one decode batch of B = 8 tokens at gpt-oss-20b
+shapes (BASELINE.json configs[1]): token-embedding gather [8] -> RMSNorm [8, 2880] ->
+QKV + bias + YaRN rotary (2880 -> 5120, weight streaming) -> clamped SwiGLU [32, 5760].
+Every step uses the next of 24 distinct layer weight sets (708 MB of QKV weights), so the
+weights come from HBM, not from the 256 MB Infinity Cache. The K timed steps are captured
+in one HIP graph and replayed, which is how the reference runs its decode loop.
+
+Prints ONE JSON line: whole-job tokens/s, plus `roofline` for the dominant kernel (the
+decode QKV stream), `cpu_baseline` (the eager bf16 PyTorch restatement of the reference
+chain timed on the host cores) and a `kernels` table with every kernel at its decode and
+prefill sizes (GB/s against 8 TB/s, or TFLOP/s against 2.5 PFLOP/s bf16 for prefill QKV).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published (no sparsity)
+
+B = 8
+HIDDEN, QKV_DIM, NQ, NKV, HD = 2880, 5120, 64, 8, 64
+SWIGLU_ROWS = 4 * B
+N_LAYERS = 24
+VOCAB_BENCH = 201088
+
+
+def algorithmic_bytes():
+    """Compulsory HBM traffic per launch (bytes)."""
+    w = QKV_DIM * HIDDEN * 2
+    return {
+        "rmsnorm": lambda r: r * 2 * HIDDEN * 2 + HIDDEN * 2,
+        "embedding": lambda t: t * (2 * HIDDEN * 2 + 4),
+        "swiglu": lambda m: m * (2 * HIDDEN * 2 + HIDDEN * 2),
+        "qkv": lambda r: w + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=480)
+    ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-table", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU; --gpus N with N > 1 is not supported "
+              "(no collectives are part of the layer-kernel path).", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import tritonllm_amd as T
+    from tritonllm_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from tritonllm_amd.build import build_library
+        build_library()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    bytes_of = algorithmic_bytes()
+    yarn = T.gpt_oss_yarn()
+
+    # ---------------------------------------------------------------- synthetic inputs (seed 0)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, HIDDEN, generator=g).bfloat16().to(dev)
+    swiglu_x = (2.0 * torch.randn(SWIGLU_ROWS, 2 * HIDDEN, generator=g)).bfloat16().to(dev)
+    positions = torch.randint(0, 8192, (B,), generator=g, dtype=torch.int64).to(dev)
+    ids = torch.randint(0, VOCAB_BENCH, (B,), generator=g, dtype=torch.int32).to(dev)
+    gg = torch.Generator(device=dev).manual_seed(0)
+    table = torch.empty(VOCAB_BENCH, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
+    weights = [torch.empty(QKV_DIM, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
+    biases = [torch.empty(QKV_DIM, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
+    scales = [(1 + 0.1 * torch.randn(HIDDEN, generator=g)).bfloat16().to(dev) for _ in range(N_LAYERS)]
+    h = torch.empty(B, HIDDEN, dtype=torch.bfloat16, device=dev)
+    t = torch.empty(B, HIDDEN, dtype=torch.bfloat16, device=dev)
+    q = torch.empty(B, NQ * HD, dtype=torch.bfloat16, device=dev)
+    k = torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev)
+    v = torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev)
+    s_out = torch.empty(SWIGLU_ROWS, HIDDEN, dtype=torch.bfloat16, device=dev)
+
+    def step(i: int) -> None:
+        l = i % N_LAYERS
+        T.embedding_forward(ids, table, out=h)
+        T.rmsnorm_forward(x, scales[l], 1e-5, out=t)
+        T.qkv_rope_forward(t, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=positions, mode="decode", out=(q, k, v))
+        T.swiglu(swiglu_x, out=s_out)
+
+    def graph_of(fn, n: int):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for i in range(n):
+                fn(i)
+        return gr
+
+    def time_graph(gr, reps: int = 1) -> float:
+        """Seconds for `reps` replays, HIP events on the current stream."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3
+
+    # ---------------------------------------------------------------- the timed job
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    job = graph_of(step, args.steps)
+    job.replay()                                   # one untimed replay: graph upload / first-touch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    elapsed = time_graph(job)
+    wall = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = B * args.steps / elapsed
+
+    # ---------------------------------------------------------------- dominant kernel, live
+    n_launch = 20 * N_LAYERS
+    qkv_graph = graph_of(lambda i: T.qkv_rope_forward(t, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn,
+                                                      positions=positions, mode="decode", out=(q, k, v)), n_launch)
+    qkv_graph.replay()
+    qkv_s = min(time_graph(qkv_graph) for _ in range(5)) / n_launch
+    qkv_bytes = bytes_of["qkv"](B)
+    roofline = {
+        "kernel": "qkv_decode_kernel (QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)",
+        "bound": "hbm", "achieved": round(qkv_bytes / qkv_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(qkv_bytes / qkv_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+        "bytes_per_launch": qkv_bytes, "avg_launch_us": round(qkv_s * 1e6, 3),
+    }
+
+    # ---------------------------------------------------------------- per-kernel table
+    kernels = {}
+    if not args.no_kernel_table:
+        def bench_kernel(name, fn, nbytes=None, flops=None, n=200):
+            for i in range(3):
+                fn(i)
+            gr = graph_of(fn, n)
+            gr.replay()
+            sec = min(time_graph(gr) for _ in range(5)) / n
+            row = {"us": round(sec * 1e6, 3)}
+            if nbytes is not None:
+                row["GB/s"] = round(nbytes / sec / 1e9, 1)
+                row["hbm_frac"] = round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)
+            if flops is not None:
+                row["TFLOP/s"] = round(flops / sec / 1e12, 1)
+                row["mfma_frac"] = round(flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+            kernels[name] = row
+
+        bench_kernel("rmsnorm_B8", lambda i: T.rmsnorm_forward(x, scales[i % N_LAYERS], 1e-5, out=t), bytes_of["rmsnorm"](B))
+        bench_kernel("embedding_B8", lambda i: T.embedding_forward(ids, table, out=h), bytes_of["embedding"](B))
+        bench_kernel("swiglu_M32", lambda i: T.swiglu(swiglu_x, out=s_out), bytes_of["swiglu"](SWIGLU_ROWS))
+        kernels["qkv_rope_decode_B8"] = {"us": roofline["avg_launch_us"], "GB/s": roofline["achieved"], "hbm_frac": roofline["frac"]}
+        for r in (1, 32):
+            xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
+            pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
+            qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),
+                  torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev))
+            bench_kernel(f"qkv_rope_decode_B{r}",
+                         lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
+                                                                           yarn=yarn, positions=pr, mode="decode", out=qo),
+                         bytes_of["qkv"](r), n=240)
+        # prefill sizes
+        for tt in (2048, 8192):
+            xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            pp = torch.arange(tt, dtype=torch.int64, device=dev)
+            qo = (torch.empty(tt, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(tt, NKV * HD, dtype=torch.bfloat16, device=dev),
+                  torch.empty(tt, NKV * HD, dtype=torch.bfloat16, device=dev))
+            to = torch.empty_like(xp)
+            bench_kernel(f"qkv_rope_prefill_T{tt}",
+                         lambda i, xp=xp, pp=pp, qo=qo: T.qkv_rope_forward(xp, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
+                                                                           yarn=yarn, positions=pp, mode="prefill", out=qo),
+                         flops=2.0 * tt * HIDDEN * QKV_DIM, n=48)
+            bench_kernel(f"rmsnorm_T{tt}", lambda i, xp=xp, to=to: T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=to),
+                         bytes_of["rmsnorm"](tt), n=96)
+            del xp, qo, to
+        idp = torch.randint(0, VOCAB_BENCH, (2048,), generator=g, dtype=torch.int32).to(dev)
+        hp = torch.empty(2048, HIDDEN, dtype=torch.bfloat16, device=dev)
+        bench_kernel("embedding_T2048", lambda i: T.embedding_forward(idp, table, out=hp), bytes_of["embedding"](2048), n=96)
+        sx = torch.empty(32768, 2 * HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 2, generator=gg)
+        so = torch.empty(32768, HIDDEN, dtype=torch.bfloat16, device=dev)
+        bench_kernel("swiglu_M32768", lambda i: T.swiglu(sx, out=so), bytes_of["swiglu"](32768), n=48)
+        del sx, so
+
+    # ---------------------------------------------------------------- CPU baseline (reported only)
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        from oracle import layers as O
+
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        cx, cw, cb, cs = x.cpu(), weights[0].cpu(), biases[0].cpu(), scales[0].cpu()
+        cids, cpos, csw = ids.cpu().long(), positions.cpu(), swiglu_x.cpu()
+        ctable = table[:65536].cpu()                      # the gather touches 8 rows; a 377 MB slice keeps host memory modest
+        cids = cids % 65536
+        cos_t, sin_t = O.yarn_cos_sin(torch.arange(8192))
+
+        def cpu_step():
+            O.embedding_eager(ctable, cids)
+            tt = O.rmsnorm_eager(cx, cs)
+            O.qkv_rope_eager(tt, cw, cb, cos_t, sin_t, cpos)
+            O.swiglu_eager(csw)
+
+        for _ in range(3):
+            cpu_step()
+        n_cpu, t_start = 0, time.perf_counter()
+        while True:
+            cpu_step()
+            n_cpu += 1
+            dt = time.perf_counter() - t_start
+            if dt > args.cpu_seconds or n_cpu >= 2000:
+                break
+        cpu_baseline = {
+            "value": round(B * n_cpu / dt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{n_cpu} steps of the same B=8 step (eager bf16 PyTorch restatement of the reference chain, one weight set) in {dt:.1f} s",
+        }
+
+    out = {
+        "metric": "layer-kernel tokens/s + % HBM/MFMA roofline, gpt-oss-20b shapes, 1 GPU",
+        "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: B=8 decode step = embedding gather[8] + RMSNorm[8,2880] + QKV+bias+YaRN-RoPE(2880->5120) + "
+                               "clamped SwiGLU[32,5760]; 24 rotating weight sets; HIP-graph replay of all steps",
+                   "batch": B, "layers_rotated": N_LAYERS},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
+        "wall_s_timed_region": round(wall, 4),
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -125,7 +125,9 @@ int tllm_rope_bf16(void* q, void* k, int64_t rows, int n_q_heads, int n_kv_heads
  * reference's write of the new token into the KV cache.
  *
  * _decode: weight-streaming kernel for few rows (any rows accepted; the
- *   weight is streamed once per 16 rows).
+ *   weight is streamed once per 32 rows). Needs no workspace: unlike the
+ *   reference's split-K pair of launches (partials at triton_kernels.py:1200)
+ *   the K reduction stays inside a workgroup.
  *   replaces qkv_rope_cache_decode_forward triton_kernels.py:1109-1255 and,
  *   with rope == NULL, qkv_decode_forward triton_kernels.py:615-659.
  * _prefill: LDS-staged bf16 MFMA GEMM with the bias + rotary epilogue.

@@ -37,6 +37,8 @@ int make_rope_args(const TllmRope* rope, int head_dim, RopeArgs* out, YarnFreqs*
                "rope: tokens_per_batch %lld must be >= 1 when positions is NULL", (long long)rope->tokens_per_batch);
   if (rope->yarn) {
     TLLM_REQUIRE(rope->yarn->n_freq == n_freq, TLLM_E_SHAPE, "rope: yarn.n_freq %d != head_dim/2 = %d", rope->yarn->n_freq, n_freq);
+    TLLM_REQUIRE(rope->max_ctx <= (1ll << 24), TLLM_E_SHAPE,
+                 "rope: in-register cos/sin supports max_ctx <= 2^24 (got %lld); pass cos/sin tables instead", (long long)rope->max_ctx);
     memcpy(freqs->v, rope->yarn->inv_freq, sizeof(float) * n_freq);
     out->concentration = rope->yarn->concentration;
     out->use_yarn = 1;

@@ -77,14 +77,38 @@ __device__ __forceinline__ int64_t rope_position(const RopeArgs& r, int64_t row)
   return rope_wrap(rope_position_raw(r, row), r.max_ctx);
 }
 
-// cos/sin of the rotary angle for (position, frequency index), scaled by the
-// concentration. The angle is the single fp32 product float(pos) * inv_freq,
-// exactly as the reference's table construction forms it; sincosf is the
-// full-range routine (angles reach 1.3e5 rad), never the fast intrinsics.
+// sin and cos of an fp32 angle up to ~3e7 rad, to ~1e-7 absolute (about one ulp of 1.0).
+// Three-constant Cody-Waite reduction by pi/2 carried in FMAs (the products are exact inside the
+// FMA, so the only rounding is that of the reduced argument), then the classic single-precision
+// minimax polynomials on [-pi/4, pi/4] and a quadrant fix-up. A dozen registers and ~25
+// instructions; the library routine's Payne-Hanek path costs five times the registers, which
+// would cap the occupancy of every kernel that rotates.
+__device__ __forceinline__ void sincos_reduced(float x, float* s, float* c) {
+  const float kf = rintf(x * 0.636619772367581343f);
+  float r = fmaf(-kf, 1.57079637050628662109375f, x);
+  r = fmaf(-kf, -4.37113882867379e-8f, r);
+  r = fmaf(-kf, -1.7151245e-15f, r);
+  const float z = r * r;
+  float sp = fmaf(z, -1.9515295891e-4f, 8.3321608736e-3f);
+  sp = fmaf(z, sp, -1.6666654611e-1f);
+  const float sv = fmaf(r * z, sp, r);
+  float cp = fmaf(z, 2.443315711809948e-5f, -1.388731625493765e-3f);
+  cp = fmaf(z, cp, 4.166664568298827e-2f);
+  const float cv = fmaf(z * z, cp, fmaf(z, -0.5f, 1.0f));
+  const int q = static_cast<int>(kf);
+  const float ss = (q & 1) ? cv : sv;
+  const float cc = (q & 1) ? sv : cv;
+  *s = (q & 2) ? -ss : ss;
+  *c = ((q + 1) & 2) ? -cc : cc;
+}
+
+// cos/sin of the rotary angle for (position, frequency), scaled by the concentration. The angle is
+// the single fp32 product float(pos) * inv_freq, exactly as the reference's table construction forms
+// it (angles reach 1.3e5 rad at the end of the context: the fast hardware sin/cos are useless here).
 __device__ __forceinline__ void yarn_cos_sin(int64_t pos, float inv_freq, float concentration, float* c, float* s) {
-  float angle = __fmul_rn(static_cast<float>(pos), inv_freq);
+  const float angle = __fmul_rn(static_cast<float>(pos), inv_freq);
   float sv, cv;
-  sincosf(angle, &sv, &cv);
+  sincos_reduced(angle, &sv, &cv);
   *c = cv * concentration;
   *s = sv * concentration;
 }

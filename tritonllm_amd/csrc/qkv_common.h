@@ -21,10 +21,13 @@ struct QkvArgs {
   int has_rope;
 };
 
+// KV-cache slot the new token goes to (0 when the outputs are plain tensors). A global load: call it early.
+__device__ __forceinline__ int64_t qkv_slot(const QkvArgs& a, const RopeArgs& ra) {
+  return (a.kv_slot_stride != 0 && ra.offset != nullptr) ? ra.offset[0] : 0;
+}
+
 // Start of head `head` (0 .. n_q + 2 n_kv) of output row `row`.
-__device__ __forceinline__ bf16* qkv_out_ptr(const QkvArgs& a, const RopeArgs& ra, int64_t row, int head) {
-  int64_t slot = 0;
-  if (a.kv_slot_stride != 0 && ra.offset != nullptr) slot = ra.offset[0];
+__device__ __forceinline__ bf16* qkv_out_ptr(const QkvArgs& a, int64_t slot, int64_t row, int head) {
   if (head < a.n_q_heads) return a.q + row * a.q_rs + static_cast<int64_t>(head) * a.head_dim;
   head -= a.n_q_heads;
   if (head < a.n_kv_heads) return a.k + row * a.k_rs + slot * a.kv_slot_stride + static_cast<int64_t>(head) * a.head_dim;

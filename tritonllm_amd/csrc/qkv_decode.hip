@@ -1,19 +1,15 @@
-// Decode-size fused QKV projection + bias + rotary: a weight-streaming kernel.
+// Decode-size fused QKV projection + bias + rotary: weight-streaming kernels.
 //
-// The 29.5 MB weight is read exactly once per call, so the kernel is HBM-bound and is
-// organised around keeping the whole weight in flight:
-//   * a workgroup owns 16 weight rows of one head -- dims [8p, 8p+8) and their rotation
-//     partners [32+8p, 32+8p+8) -- so a rotation pair never leaves the workgroup;
-//     80 heads x 4 pieces = 320 workgroups, all resident at once on 256 CUs;
-//   * the K dimension is split over the workgroup's wavefronts; every wavefront issues
-//     all of its 128-bit weight loads (and the matching activation loads, which hit L2)
-//     before the first multiply, so ~all of W is requested up front;
-//   * the arithmetic is v_mfma_f32_16x16x32_bf16 with the weight rows as the M side and
-//     up to 16 activation rows as the N side -- the matrix core does the K reduction
-//     across lanes for free and leaves the VALU idle for the rotary epilogue;
-//   * partial tiles of the wavefronts meet in LDS; wavefront 0 adds the bias, rotates the
-//     fp32 accumulator with cos/sin it computed while the loads were in flight, rounds
-//     once to bf16 and writes q / k / v (k and v optionally into a KV-cache slot).
+// With a handful of activation rows the 29.5 MB weight is read once and nothing else matters: the
+// kernels are HBM-bound. All of them use the matrix core with the weight rows on the M side and
+// the activation rows on the N side -- the MFMA does the K reduction across lanes for free and
+// leaves the VALU to the rotary epilogue -- and keep a rotation pair (row d and row d+32 of a
+// head) inside one workgroup so the rotation needs no second pass. Three kernels:
+//   qkv_decode_cu_kernel   hidden == 2880 (gpt-oss): one workgroup per CU, coalesced loads,
+//                          LDS-transposed operands. The fast path; see its comment.
+//   qkv_decode_kernel      head_dim == 64, hidden % 32 == 0: operands loaded straight into MFMA
+//                          layout (simple, ~1.8x slower: every lane is its own cache-line request).
+//   qkv_generic_kernel     anything else: shuffle-reduced dot products.
 #include "qkv_common.h"
 
 namespace tllm {
@@ -67,7 +63,7 @@ __global__ __launch_bounds__(256) void qkv_generic_kernel(QkvArgs a, RopeArgs ra
   const int half = a.head_dim >> 1;
   for (int64_t row = blockIdx.y; row < a.rows; row += gridDim.y) {
   const bf16* xr = a.x + row * a.hidden;
-  bf16* out = qkv_out_ptr(a, ra, row, head);
+  bf16* out = qkv_out_ptr(a, qkv_slot(a, ra), row, head);
   const bool rotate = a.has_rope && head < a.n_q_heads + a.n_kv_heads;
   const int64_t pos = rotate ? rope_position(ra, row) : 0;
   for (int d = wave; d < half; d += 4) {
@@ -108,8 +104,12 @@ void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& f
 }
 
 // ------------------------------------------------------------------------------------------------
-// the weight-streaming MFMA kernel (head_dim == 64, hidden % 32 == 0)
-template <int NW, int SPW, bool kExact>   // kExact: hidden == 32 * NW * SPW, no tail guards anywhere in the loop
+// MFMA kernel for any hidden % 32 == 0 (head_dim 64). A workgroup owns 16 weight rows of one head --
+// dims [8p, 8p+8) and their partners [32+8p, 32+8p+8) -- and up to 16 activation rows; its wavefronts
+// split K in runs of SPW k32-steps whose loads are all issued before the first multiply.
+// v_mfma_f32_16x16x32_bf16: tile row 4*qd + i is dim 8p + 2*qd + (i & 1), plus 32 when i >= 2, so
+// each lane's four accumulators are two complete (lo, hi) pairs.
+template <int NW, int SPW>
 __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   __shared__ float red[NW][4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -119,62 +119,29 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   const int nsteps = a.hidden >> 5;     // MFMA k-steps of 32
   const int m = lane & 15, g = lane >> 4;
 
-  // A side: weight row held by this lane. Tile row m = 4*qd + i maps to dim
-  // 8*piece + 2*qd + (i & 1), plus 32 when i >= 2, so that after the MFMA each lane's
-  // four accumulators are two (lo, hi) rotation pairs.
   const int dim_a = 8 * piece + 2 * (m >> 2) + (m & 1) + ((m & 2) ? 32 : 0);
   const bf16x8* wrow = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * 64 + dim_a) * kvec + g;
-  // B side: activation row n = lane % 16 of this 16-row chunk. Lanes past the last row re-read
-  // a valid row (same addresses as a live lane, so no extra traffic); their output column is dropped.
+  // Lanes past the last activation row re-read a live lane's row (same addresses, no extra traffic);
+  // their output column is dropped.
   const int64_t xrow_idx = row0 + m;
   const bool xvalid = xrow_idx < a.rows;
   const int nvalid = static_cast<int>(a.rows - row0 < 16 ? a.rows - row0 : 16);
   const bf16x8* xrow = reinterpret_cast<const bf16x8*>(a.x) + (row0 + (xvalid ? m : m % nvalid)) * kvec + g;
-
   const bool rotate = a.has_rope && head < a.n_q_heads + a.n_kv_heads;
-  // position first: its load is then the oldest outstanding one and can be waited for alone
-  // and the two YaRN frequencies of this lane's pairs come out of the kernel-argument block now,
-  // so nothing issued after the weight loads has to be waited for before the cos/sin math.
-  int64_t pos = 0;
-  const float f0 = fr.v[8 * piece + 2 * g], f1 = fr.v[8 * piece + 2 * g + 1];   // zeros when no YaRN block was given
-  if (rotate && wave == 0) pos = rope_position_raw(ra, xvalid ? xrow_idx : row0);
-  __builtin_amdgcn_sched_barrier(0);
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  float cs[2] = {1.f, 1.f}, sn[2] = {0.f, 0.f};
-
   for (int s0 = wave * SPW; s0 < nsteps; s0 += NW * SPW) {
     bf16x8 wa[SPW], xb[SPW];
 #pragma unroll
+    for (int i = 0; i < SPW; ++i) {       // clamped, never predicated: a tail step re-reads the last one and is masked below
+      const int step = s0 + i < nsteps ? s0 + i : nsteps - 1;
+      wa[i] = __builtin_nontemporal_load(wrow + step * 4);
+      xb[i] = xrow[step * 4];
+    }
+#pragma unroll
     for (int i = 0; i < SPW; ++i) {
-      const int step = s0 + i;
-      if (kExact || step < nsteps) {
-        wa[i] = __builtin_nontemporal_load(wrow + step * 4);
-        xb[i] = xrow[step * 4];
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          wa[i][j] = static_cast<bf16>(0.f);
-          xb[i][j] = static_cast<bf16>(0.f);
-        }
-      }
+      if (s0 + i < nsteps) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[i], xb[i], acc, 0, 0, 0);
     }
-    __builtin_amdgcn_sched_barrier(0);
-    if (wave == 0 && s0 == 0 && rotate) {
-      // cos/sin for this lane's two pairs, computed while the weight loads are in flight
-      const int d0 = 8 * piece + 2 * g;
-      pos = rope_wrap(pos, ra.max_ctx);
-      if (ra.use_yarn) {
-        yarn_cos_sin(pos, f0, ra.concentration, &cs[0], &sn[0]);
-        yarn_cos_sin(pos, f1, ra.concentration, &cs[1], &sn[1]);
-      } else {
-        rope_cos_sin(ra, fr, pos, d0, &cs[0], &sn[0]);
-        rope_cos_sin(ra, fr, pos, d0 + 1, &cs[1], &sn[1]);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < SPW; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[i], xb[i], acc, 0, 0, 0);
-    if (kExact) break;
   }
 
 #pragma unroll
@@ -188,8 +155,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   }
   if (!xvalid) return;
 
-  // Output side: lane holds activation row n = lane % 16 and, with qd = lane / 16,
-  // dims d0 = 8*piece + 2*qd and d0 + 1 (acc[0], acc[1]) and their partners (acc[2], acc[3]).
+  // the lane holds activation row xrow_idx and dims d0, d0 + 1 (acc[0], acc[1]) with their partners (acc[2], acc[3])
   const int d0 = 8 * piece + 2 * g;
   const int col = head * 64 + d0;
   float lo0 = acc[0], lo1 = acc[1], hi0 = acc[2], hi1 = acc[3];
@@ -200,14 +166,18 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
     hi1 += static_cast<float>(a.bias[col + 33]);
   }
   if (rotate) {
-    const float r0 = lo0 * cs[0] - hi0 * sn[0], r1 = lo1 * cs[1] - hi1 * sn[1];
-    const float r2 = hi0 * cs[0] + lo0 * sn[0], r3 = hi1 * cs[1] + lo1 * sn[1];
+    const int64_t pos = rope_position(ra, xrow_idx);
+    float c0, s0, c1, s1;
+    rope_cos_sin(ra, fr, pos, d0, &c0, &s0);
+    rope_cos_sin(ra, fr, pos, d0 + 1, &c1, &s1);
+    const float r0 = lo0 * c0 - hi0 * s0, r1 = lo1 * c1 - hi1 * s1;
+    const float r2 = hi0 * c0 + lo0 * s0, r3 = hi1 * c1 + lo1 * s1;
     lo0 = r0;
     lo1 = r1;
     hi0 = r2;
     hi1 = r3;
   }
-  bf16* out = qkv_out_ptr(a, ra, xrow_idx, head);
+  bf16* out = qkv_out_ptr(a, qkv_slot(a, ra), xrow_idx, head);
   bf16x2 plo, phi;
   plo[0] = static_cast<bf16>(lo0);
   plo[1] = static_cast<bf16>(lo1);
@@ -215,6 +185,164 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   phi[1] = static_cast<bf16>(hi1);
   *reinterpret_cast<bf16x2*>(out + d0) = plo;
   *reinterpret_cast<bf16x2*>(out + d0 + 32) = phi;
+}
+
+// ------------------------------------------------------------------------------------------------
+// One-workgroup-per-CU variant for hidden == 2880 (the default decode kernel).
+//
+// The 2560 rotation pairs are dealt out ten at a time: 256 workgroups, each needing most of a CU's
+// LDS, so the dispatcher has to place exactly one per CU and every CU streams exactly 1/256 of the
+// weight (20 rows x 5760 B). Fifteen wavefronts split K (six k32-steps each); all loads of the
+// kernel -- the small ones the epilogue needs first, then activations, then weights -- are issued
+// unconditionally (indices clamped, never predicated) before anything is consumed, so the compiler
+// has no join to wait at and ~180 KB per CU is in flight from the first microsecond.
+// Loads are coalesced along K; the MFMA operand layout is produced by a pass through a
+// wavefront-private LDS patch. v_mfma_f32_32x32x16_bf16: M = 32 tile rows (pair slot p at row p, its
+// partner at row p + 16), N = up to XR activation rows. After one barrier the fifteen partial tiles
+// are summed by 16 x XR threads, one (pair, activation row) each, which also add the bias, rotate
+// with cos/sin they computed while the loads were in flight, round once and store.
+template <int XR, int CH>
+__global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
+  constexpr int NW = 15, SPW = 6, NCH = SPW / CH, PAIRS = 10;
+  constexpr int KV = 360;                 // 16-byte vectors per row (hidden 2880)
+  constexpr int WROW = CH * 64 + 16;      // padded patch row, bytes
+  constexpr int CPR = CH * 4;             // 16-byte chunks per row per patch
+  constexpr int WL = (2 * PAIRS * CPR + 63) / 64;   // weight load instructions per patch
+  constexpr int XL = (XR * CPR + 63) / 64;          // activation load instructions per patch
+  constexpr int PATCH = (32 + XR) * WROW;
+  constexpr int RED = XR * 32;            // floats per wavefront in the reduction buffer
+  static_assert(SPW % CH == 0, "patches must tile the K slice");
+  static_assert(NW * RED * 4 <= NW * PATCH, "reduction buffer aliases the patches");
+  static_assert(16 * XR <= 960, "one epilogue thread per (pair slot, activation row)");
+  __shared__ __align__(16) unsigned char lds[NW * PATCH];
+  __shared__ float s_pin[16];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int total_pairs = (a.n_q_heads + 2 * a.n_kv_heads) * 32;
+  const int pair0 = blockIdx.x * PAIRS;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
+  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+
+  // ---- epilogue role of this thread: pair slot es, activation row en (clamped to real ones for the loads)
+  const int es = tid & 15, en = tid >> 4;
+  const bool evalid = tid < 16 * XR && es < PAIRS && pair0 + es < total_pairs && en < nvalid;
+  const int egp = evalid ? pair0 + es : 0;
+  const int ehead = egp >> 5, ed = egp & 31;
+  const int64_t erow = row0 + (evalid ? en : 0);
+  const bool erot = a.has_rope && ehead < a.n_q_heads + a.n_kv_heads;
+
+  // ---- every global load of the kernel, oldest first
+  const int64_t* pos_ptr = ra.positions ? ra.positions + erow : reinterpret_cast<const int64_t*>(a.W);
+  const int64_t* off_ptr = ra.offset ? ra.offset : reinterpret_cast<const int64_t*>(a.W);
+  const unsigned short* bias_ptr = reinterpret_cast<const unsigned short*>(a.bias ? a.bias : a.W);
+  const int64_t pos_ld = *pos_ptr;
+  const int64_t off_ld = *off_ptr;
+  const unsigned short b_lo = bias_ptr[ehead * 64 + ed], b_hi = bias_ptr[ehead * 64 + 32 + ed];
+  const float freq = fr.v[ed];
+  __builtin_amdgcn_sched_barrier(0);
+
+  const bf16x8* xg = reinterpret_cast<const bf16x8*>(a.x) + row0 * KV + wave * (SPW * 4);
+  const bf16x8* wg = reinterpret_cast<const bf16x8*>(a.W) + wave * (SPW * 4);
+  bf16x8 xr[NCH * XL], wr[NCH * WL];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {          // patch chunk e -> activation row e / CPR, chunk e % CPR
+      int e = i * 64 + lane;
+      e = e < XR * CPR ? e : XR * CPR - 1;
+      int r = e / CPR;
+      const int kc = e - r * CPR;
+      r = r < nvalid ? r : nvalid - 1;
+      xr[j * XL + i] = xg[r * KV + j * CPR + kc];
+    }
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {          // patch chunk e -> weight row e / CPR: the ten low rows, then their partners
+      int e = i * 64 + lane;
+      e = e < 2 * PAIRS * CPR ? e : 2 * PAIRS * CPR - 1;
+      const int r = e / CPR, kc = e - r * CPR;
+      int gp = pair0 + (r < PAIRS ? r : r - PAIRS);
+      gp = gp < total_pairs ? gp : total_pairs - 1;
+      const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + (r < PAIRS ? 0u : 32u);
+      wr[j * WL + i] = __builtin_nontemporal_load(wg + wrow * static_cast<unsigned>(KV) + j * CPR + kc);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- cos/sin of this thread's (pair, row) while the weights are in flight.
+  // The store pins the frequency load above the weight stream: with its only use inside the
+  // conditional below, the compiler would sink it there and then have to drain every load to read it.
+  s_pin[es] = freq;
+  float cs = 1.f, sn = 0.f;
+  const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
+  if (a.has_rope) {
+    int64_t pos = ra.positions ? pos_ld : (erow % ra.tokens_per_batch) + (ra.offset ? off_ld : 0);
+    pos = rope_wrap(pos, ra.max_ctx);
+    if (ra.use_yarn) yarn_cos_sin(pos, freq, ra.concentration, &cs, &sn);
+    else rope_cos_sin(ra, fr, pos, ed, &cs, &sn);
+  }
+
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  const int m = lane & 31, h = lane >> 5;
+  unsigned char* wp = lds + wave * PATCH;            // 32 tile rows (only those of real pairs are written)
+  unsigned char* xp = wp + 32 * WROW;                // XR activation rows
+  const unsigned char* wfrag = wp + m * WROW + h * 16;
+  const unsigned char* xfrag = xp + (m & (XR - 1)) * WROW + h * 16;   // stale LDS in unused rows/columns is never stored
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int e = i * 64 + lane;
+      const int r = e / CPR, kc = e - r * CPR;
+      if (e < XR * CPR && r < nvalid) *reinterpret_cast<bf16x8*>(xp + r * WROW + kc * 16) = xr[j * XL + i];
+    }
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+      const int e = i * 64 + lane;
+      const int r = e / CPR, kc = e - r * CPR;
+      const int trow = r < PAIRS ? r : r - PAIRS + 16;
+      if (e < 2 * PAIRS * CPR) *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 16) = wr[j * WL + i];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < 2 * CH; ++t) {
+      const bf16x8 fa = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
+      const bf16x8 fb = *reinterpret_cast<const bf16x8*>(xfrag + t * 32);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // ---- fifteen partial tiles -> LDS as [wave][tile row][activation row] (lanes of one store hit distinct banks)
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lds);
+  if (m < XR) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[wave * RED + (8 * (v >> 2) + 4 * h + (v & 3)) * XR + m] = acc[v];
+  }
+  __syncthreads();
+  if (!evalid) return;
+  float lo = 0.f, hi = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    lo += red[w * RED + es * XR + en];
+    hi += red[w * RED + (16 + es) * XR + en];
+  }
+  if (a.bias) {
+    lo += __uint_as_float(static_cast<unsigned>(b_lo) << 16);
+    hi += __uint_as_float(static_cast<unsigned>(b_hi) << 16);
+  }
+  if (erot) {
+    const float rl = lo * cs - hi * sn, rh = hi * cs + lo * sn;
+    lo = rl;
+    hi = rh;
+  }
+  bf16* out = qkv_out_ptr(a, slot, erow, ehead);
+  out[ed] = static_cast<bf16>(lo);
+  out[ed + 32] = static_cast<bf16>(hi);
 }
 
 }  // namespace tllm
@@ -234,21 +362,31 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
   a.bias = (const bf16*)b;
   if (rows == 0) return TLLM_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool fast = head_dim == 64 && hidden % 32 == 0 && aligned16(x) && aligned16(W) &&
-                    (reinterpret_cast<uintptr_t>(q) % 4 == 0) && (reinterpret_cast<uintptr_t>(k) % 4 == 0) &&
+  const int heads = n_q_heads + 2 * n_kv_heads;
+  const bool mfma_ok = head_dim == 64 && hidden % 32 == 0 && aligned16(x) && aligned16(W);
+  if (mfma_ok && hidden == 2880 && aligned16(b) && static_cast<int64_t>(heads) * 64 * hidden < (1ll << 31)) {
+    // 32-bit element offsets inside W and x are enough here; outputs are written element-wise, any alignment
+    const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
+    const int64_t chunks = (rows + xr - 1) / xr;
+    TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
+    dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
+    if (xr == 8)
+      hipLaunchKernelGGL((qkv_decode_cu_kernel<8, 3>), grid, dim3(960), 0, st, a, ra, fr);
+    else if (xr == 16)
+      hipLaunchKernelGGL((qkv_decode_cu_kernel<16, 3>), grid, dim3(960), 0, st, a, ra, fr);
+    else
+      hipLaunchKernelGGL((qkv_decode_cu_kernel<32, 2>), grid, dim3(960), 0, st, a, ra, fr);
+    return check_launch("qkv_rope_decode");
+  }
+  const bool out4 = (reinterpret_cast<uintptr_t>(q) % 4 == 0) && (reinterpret_cast<uintptr_t>(k) % 4 == 0) &&
                     (reinterpret_cast<uintptr_t>(v) % 4 == 0) && q_row_stride % 2 == 0 && k_row_stride % 2 == 0 &&
                     v_row_stride % 2 == 0 && kv_slot_stride % 2 == 0;
-  if (!fast) {
-    launch_qkv_generic(a, ra, fr, st);
-    return check_launch("qkv_rope_decode(generic)");
+  if (mfma_ok && out4) {
+    const int64_t chunks = (rows + 15) / 16;
+    TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
+    hipLaunchKernelGGL((qkv_decode_kernel<4, 16>), dim3((unsigned)(heads * 4), (unsigned)chunks), dim3(4 * 64), 0, st, a, ra, fr);
+    return check_launch("qkv_rope_decode");
   }
-  const int heads = n_q_heads + 2 * n_kv_heads;
-  const int64_t chunks = (rows + 15) / 16;
-  TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
-  dim3 grid((unsigned)(heads * 4), (unsigned)chunks);
-  if (hidden == 32 * 5 * 18)   // 2880: five wavefronts x 18 k-steps, the whole weight in flight at once
-    hipLaunchKernelGGL((qkv_decode_kernel<5, 18, true>), grid, dim3(5 * 64), 0, st, a, ra, fr);
-  else
-    hipLaunchKernelGGL((qkv_decode_kernel<4, 16, false>), grid, dim3(4 * 64), 0, st, a, ra, fr);
-  return check_launch("qkv_rope_decode");
+  launch_qkv_generic(a, ra, fr, st);
+  return check_launch("qkv_rope_decode(generic)");
 }

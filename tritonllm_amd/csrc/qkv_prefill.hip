@@ -174,9 +174,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
     __syncthreads();
   }
 
-  int64_t slot = 0;
-  if (a.kv_slot_stride != 0 && ra.offset != nullptr) slot = ra.offset[0];
-  const int64_t slot_off = slot * a.kv_slot_stride;
+  const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
 
   // The wavefront's three heads: two whole ones (blocks 0-1, 2-3) and its half of the middle head (block 4).
 #pragma unroll
