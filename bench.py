@@ -46,6 +46,56 @@ def algorithmic_bytes():
     }
 
 
+def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg) -> int:
+    """One kernel-table entry on its own (a clean target for rocprofv3)."""
+    name = args.only
+    kind, _, size = name.rpartition("_")
+    n = int(size[1:])
+    flops = nbytes = None
+    if kind in ("qkv_rope_prefill", "qkv_rope_decode"):
+        xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        pp = torch.arange(n, dtype=torch.int64, device=dev) if kind.endswith("prefill") else \
+            torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
+        qo = (torch.empty(n, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev),
+              torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev))
+        mode = "prefill" if kind.endswith("prefill") else "decode"
+        fn = lambda i: T.qkv_rope_forward(xp, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn, positions=pp,
+                                          mode=mode, out=qo)
+        flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of["qkv"](n)
+    elif kind == "rmsnorm":
+        xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        to = torch.empty_like(xp)
+        fn = lambda i: T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=to)
+        nbytes = bytes_of["rmsnorm"](n)
+    elif kind == "swiglu":
+        sx = torch.empty(n, 2 * HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 2, generator=gg)
+        so = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev)
+        fn = lambda i: T.swiglu(sx, out=so)
+        nbytes = bytes_of["swiglu"](n)
+    elif kind == "embedding":
+        idp = torch.randint(0, VOCAB_BENCH, (n,), generator=g, dtype=torch.int32).to(dev)
+        hp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev)
+        fn = lambda i: T.embedding_forward(idp, table, out=hp)
+        nbytes = bytes_of["embedding"](n)
+    else:
+        print(f"bench.py: unknown --only target {name}", file=sys.stderr)
+        return 2
+    reps = max(args.steps // 10, 24)
+    for i in range(3):
+        fn(i)
+    gr = graph_of(fn, reps)
+    gr.replay()
+    sec = min(time_graph(gr) for _ in range(5)) / reps
+    row = {"kernel": name, "us": round(sec * 1e6, 3), "launches_per_replay": reps}
+    if nbytes is not None:
+        row["GB/s"] = round(nbytes / sec / 1e9, 1)
+    if flops is not None and kind.endswith("prefill"):
+        row["TFLOP/s"] = round(flops / sec / 1e12, 1)
+        row["mfma_frac"] = round(flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+    print(json.dumps(row))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -54,6 +104,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--only", default=None,
+                    help="run just one entry of the kernel table (e.g. qkv_rope_prefill_T2048) and print its row; for profiling")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a rocprofv3 --pmc run of this command "
                          "holds a dispatch of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -119,6 +171,9 @@ def main() -> int:
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3
+
+    if args.only:
+        return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg)
 
     # ---------------------------------------------------------------- the timed job
     for i in range(args.warmup):

@@ -25,7 +25,7 @@ HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("TLLM_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def _hipcc() -> str:
