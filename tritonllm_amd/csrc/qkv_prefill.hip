@@ -6,16 +6,20 @@
 // so T = 2048 is exactly 16 x 16 = 256 tiles -- one per CU, no tail wave -- and T = 8192 is
 // exactly four per CU. Four wavefronts form a 2 x 2 grid; each owns 64 x 160 of the tile as
 // 2 x 5 v_mfma_f32_32x32x16_bf16 blocks (160 fp32 accumulators per lane) and reads 7 operand
-// fragments from LDS per 10 MFMAs. K is walked in slices of 32 through a five-stage LDS ring
-// filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers, no ds_write)
-// issued four slices ahead: with one tile per CU nothing else hides memory latency, and an L2
-// miss costs several slices' worth of MFMA time. Such a load puts the 64 lanes' 16-byte chunks at
-// consecutive LDS addresses, so rows cannot be padded; instead the chunk order inside each
-// 64-byte row is XOR-swizzled with the row index -- applied by choosing which *global* chunk a
-// lane fetches -- and the fragment reads undo it, which makes the 128-bit fragment reads of 16
-// consecutive rows conflict-free. The one barrier per slice sits between the slice's two MFMA
-// groups, so both fragment fetches (second half of this slice, first half of the next) overlap
-// with MFMAs.
+// fragments from LDS per 10 MFMAs. K is walked in slices of 64 (one 128-byte line per row) through
+// two LDS stages filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers,
+// no ds_write). Such a load puts the 64 lanes' 16-byte chunks at consecutive LDS addresses, so rows
+// cannot be padded; instead the chunk order inside each row is XOR-swizzled with the row index --
+// applied by choosing which *global* chunk a lane fetches -- and the fragment reads undo it, which
+// keeps the 128-bit fragment reads of 16 consecutive rows conflict-free.
+// With one tile per CU nothing but the kernel's own schedule hides memory latency:
+//   * the one barrier per slice sits before the slice's last MFMA group, and the loads of the slice
+//     after next are issued right behind it, so their latency overlaps a whole slice of MFMAs and
+//     both fragment prefetches (rest of this slice, head of the next) overlap MFMAs too;
+//   * an L2 miss still costs more than a slice of MFMAs and LDS has no room for a third stage, so
+//     three slices ahead every workgroup touches (one dword per line) its share of the lines its
+//     XCD's tiles are going to need, which pulls them into that XCD's L2 in time;
+//   * measured: the loop is bound by the L2->LDS feed (57 KB per slice per CU), not by the MFMAs.
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
@@ -26,28 +30,21 @@
 // The W rows are permuted accordingly when they are copied into LDS, which costs nothing.
 //
 // Epilogue: cos/sin of the tile's 128 positions x 32 frequencies are computed once per
-// workgroup from the YaRN parameters into the (by then idle) LDS stage, then every lane adds
-// the bias to its fp32 accumulators, rotates q/k pairs, rounds once to bf16 and stores
-// straight into the separate q / k / v outputs (no split / contiguous copies afterwards).
+// workgroup from the YaRN parameters into their own LDS region while the first slices are in
+// flight; after the loop every lane adds the bias to its fp32 accumulators, rotates q/k pairs,
+// rounds once to bf16 into an LDS image of the tile, and the image leaves as coalesced 128-bit
+// stores straight into the separate q / k / v outputs (no split / contiguous copies afterwards).
 #include "qkv_common.h"
 
 namespace tllm {
 
 namespace {
-#ifndef TLLM_PREFILL_BK
-#define TLLM_PREFILL_BK 64
-#endif
-#ifndef TLLM_TOUCH_DIST
-#define TLLM_TOUCH_DIST 3
-#endif
-#ifndef TLLM_PREFILL_NS
-#define TLLM_PREFILL_NS 2
-#endif
 constexpr int BM = 128;            // tokens per tile
 constexpr int HPT = 5;             // heads per tile
 constexpr int BN = HPT * 64;       // 320 columns per tile
-constexpr int BK = TLLM_PREFILL_BK;   // K slice
-constexpr int NS = TLLM_PREFILL_NS;   // LDS stages
+constexpr int BK = 64;             // K slice: one 128-byte line per row
+constexpr int NS = 2;              // LDS stages
+constexpr int kTouchDist = 3;      // slices of lead of the L2 warm-up
 constexpr int KS = BK / 16;        // k16 MFMA steps per slice
 constexpr int CHUNKS = BK / 8;     // 16-byte chunks per LDS row
 constexpr int LROW = BK * 2;       // LDS row, bytes (unpadded: rows are swizzled instead)
@@ -63,12 +60,12 @@ static_assert(BM * OROW * 2 <= NS * STAGE, "the epilogue's output image reuses t
 static_assert(SMEM <= 160 * 1024, "LDS per workgroup");
 constexpr int BLOCKS = STAGE / 1024;      // 1 KiB blocks per stage
 constexpr int LPW = BLOCKS / 4;           // load instructions per wavefront per stage
-static_assert(KS % 2 == 0 && BLOCKS % 4 == 0, "slice must be whole load instructions and an even number of MFMA steps");
+static_assert(KS % 2 == 0 && BLOCKS % 4 == 0 && CHUNKS == 8 && NS == 2, "the schedule and the swizzle below are written for BK = 64, two stages");
 }  // namespace
 
 // Chunk swizzle of LDS row r: the 16-byte chunk c of the row is stored at chunk position c ^ swz(r).
 // Chosen so that the 16 consecutive rows one fragment read touches land in 16 different bank groups.
-__device__ __forceinline__ int swz(int r) { return CHUNKS == 8 ? ((r ^ (r >> 3)) & 7) : ((r >> 2) & 3); }
+__device__ __forceinline__ int swz(int r) { return (r ^ (r >> 3)) & 7; }
 
 // LDS row i of the W tile -> (head within tile, dim within head); see the header comment.
 __device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
@@ -113,11 +110,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   const int head0 = tile_n * HPT;
   const int total_heads = a.n_q_heads + 2 * a.n_kv_heads;
   const int kvec = a.hidden >> 3;
-#ifdef TLLM_PROBE_NO_LOOP
-  const int n_iter = 1;
-#else
   const int n_iter = a.hidden / BK;
-#endif
 
   // ---- loader setup. Load instruction j of wavefront w fills LDS block w*LPW + j (RPB rows of LROW bytes);
   // lane L lands at row RPB*blk + L/CHUNKS, chunk position L%CHUNKS, so it fetches global chunk (L%CHUNKS) ^ swz(row).
@@ -134,21 +127,13 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
     const int r = (wave * LPW + bj) * RPB + lane / CHUNKS;  // LDS row: 0..127 activations, 128..447 weights
     const int c = (lane % CHUNKS) ^ swz(r);
     if (r < BM) {
-#ifdef TLLM_PROBE_SAME_TILE
-      int64_t gr = r;
-#else
       int64_t gr = row0 + r;
-#endif
       if (gr >= a.rows) gr = a.rows - 1;                // clamp: valid memory, result rows are never stored
       src[j] = reinterpret_cast<const bf16x8*>(a.x) + gr * kvec + c;
     } else {
       int hl, dim;
       w_tile_row(r - BM, &hl, &dim);
-#ifdef TLLM_PROBE_SAME_TILE
-      int h = hl;
-#else
       int h = head0 + hl;
-#endif
       if (h >= total_heads) h = total_heads - 1;        // clamp for a ragged last tile
       src[j] = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(h) * 64 + dim) * kvec + c;
     }
@@ -211,9 +196,6 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
     for (int nb = 0; nb < 5; ++nb) fb_off[kk][nb] = (fb_row + 32 * nb) * LROW + (((2 * kk + lh) ^ swz(fb_row + 32 * nb)) << 4);
   }
   auto load_frags = [&](const unsigned char* st, int kk, bf16x8 (&fa)[2], bf16x8 (&fb)[5]) {
-#ifdef TLLM_PROBE_NO_FRAG
-    return;
-#endif
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(st + fa_off[kk][mb]);
 #pragma unroll
@@ -224,11 +206,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int nb = 0; nb < 5; ++nb) {
-#ifdef TLLM_PROBE_NO_MFMA
-        acc[mb][nb][0] += static_cast<float>(fa[mb][0]) + static_cast<float>(fb[nb][0]);
-#else
         acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nb], fa[mb], acc[mb][nb], 0, 0, 0);   // weights on M, tokens on N
-#endif
       }
   };
 
@@ -265,7 +243,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   // is handed to slice it+NS (all reads of it have been issued), so the next loads start a whole MFMA
   // group before the iteration ends and their latency overlaps the following slice's MFMAs.
   issue_loads(NS - 1);
-  issue_touch(TLLM_TOUCH_DIST);
+  issue_touch(kTouchDist);
   for (int it = 0; it < n_iter; ++it) {
     const unsigned char* st = smem + (it % NS) * STAGE;
 #pragma unroll
@@ -276,7 +254,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * (LPW + kTouch) + kTouch) : "memory");   // slice it+1 has landed (this wavefront's share)
         __syncthreads();                                // ... everyone's share; and everyone has issued its last reads of slice it
         issue_loads(it + NS);
-        issue_touch(it + 1 + TLLM_TOUCH_DIST);          // youngest in the queue: the wait above leaves it outstanding
+        issue_touch(it + 1 + kTouchDist);          // youngest in the queue: the wait above leaves it outstanding
         load_frags(smem + ((it + 1) % NS) * STAGE, 0, fa[0], fb[0]);
       }
       mfma_group(fa[kk & 1], fb[kk & 1]);
@@ -292,19 +270,6 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   // rotation with the cos/sin table, one RNE) into the image; then the tile leaves as coalesced
   // 128-bit stores, eight columns of one head per lane.
   bf16* img = reinterpret_cast<bf16*>(smem);
-#ifdef TLLM_PROBE_NO_EPI
-  {
-    float t = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int nb = 0; nb < 5; ++nb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) t += acc[mb][nb][v];
-    if (t == 1.2345f) a.q[0] = static_cast<bf16>(1.f);
-    return;
-  }
-#endif
 
   // Accumulator layout (weights on the MFMA's M side): the lane owns token l32 of each 32-token block and,
   // in each 32-column block, columns 8*(v>>2) + 4*lh + (v&3) -- runs of four consecutive columns, so
@@ -368,10 +333,6 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   }
   __syncthreads();
 
-#ifdef TLLM_PROBE_NO_COPYOUT
-  if (img[tid] == static_cast<bf16>(1.2345f)) a.q[0] = static_cast<bf16>(1.f);
-  return;
-#endif
   // copy-out: chunk = 8 consecutive dims of one head of one row
   const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
   const bool vec_ok = (reinterpret_cast<uintptr_t>(a.q) % 16 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 16 == 0) &&
