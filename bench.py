@@ -43,6 +43,7 @@ def algorithmic_bytes():
         "embedding": lambda t: t * (2 * HIDDEN * 2 + 4),
         "swiglu": lambda m: m * (2 * HIDDEN * 2 + HIDDEN * 2),
         "qkv": lambda r: w + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
+        "norm_qkv": lambda r: w + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
     }
 
 
@@ -52,16 +53,17 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
     kind, _, size = name.rpartition("_")
     n = int(size[1:])
     flops = nbytes = None
-    if kind in ("qkv_rope_prefill", "qkv_rope_decode"):
+    if kind in ("qkv_rope_prefill", "qkv_rope_decode", "norm_qkv_rope_decode"):
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         pp = torch.arange(n, dtype=torch.int64, device=dev) if kind.endswith("prefill") else \
             torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
         qo = (torch.empty(n, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev),
               torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev))
         mode = "prefill" if kind.endswith("prefill") else "decode"
+        fused = kind.startswith("norm_")
         fn = lambda i: T.qkv_rope_forward(xp, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn, positions=pp,
-                                          mode=mode, out=qo)
-        flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of["qkv"](n)
+                                          mode=mode, out=qo, norm_scale=scales[i % N_LAYERS] if fused else None)
+        flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of["norm_qkv" if fused else "qkv"](n)
     elif kind == "rmsnorm":
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         to = torch.empty_like(xp)
@@ -101,6 +103,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--unfused", action="store_true",
+                    help="run RMSNorm as its own launch in front of the QKV kernel (default: normalised inside the QKV decode kernel)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -150,8 +154,12 @@ def main() -> int:
     def step(i: int) -> None:
         l = i % N_LAYERS
         T.embedding_forward(ids, table, out=h)
-        T.rmsnorm_forward(x, scales[l], 1e-5, out=t)
-        T.qkv_rope_forward(t, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=positions, mode="decode", out=(q, k, v))
+        if args.unfused:
+            T.rmsnorm_forward(x, scales[l], 1e-5, out=t)
+            T.qkv_rope_forward(t, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=positions, mode="decode", out=(q, k, v))
+        else:
+            T.qkv_rope_forward(x, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=positions, mode="decode", out=(q, k, v),
+                               norm_scale=scales[l], norm_eps=1e-5)
         T.swiglu(swiglu_x, out=s_out)
 
     def graph_of(fn, n: int):
@@ -190,13 +198,23 @@ def main() -> int:
 
     # ---------------------------------------------------------------- dominant kernel, live
     n_launch = 20 * N_LAYERS
-    qkv_graph = graph_of(lambda i: T.qkv_rope_forward(t, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn,
-                                                      positions=positions, mode="decode", out=(q, k, v)), n_launch)
+    T.rmsnorm_forward(x, scales[0], 1e-5, out=t)
+    if args.unfused:
+        dominant = lambda i: T.qkv_rope_forward(t, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn,
+                                                positions=positions, mode="decode", out=(q, k, v))
+        qkv_bytes = bytes_of["qkv"](B)
+        kernel_name = "qkv_decode_cu_kernel<8,3,0> (QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
+    else:
+        dominant = lambda i: T.qkv_rope_forward(x, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn,
+                                                positions=positions, mode="decode", out=(q, k, v),
+                                                norm_scale=scales[i % N_LAYERS], norm_eps=1e-5)
+        qkv_bytes = bytes_of["norm_qkv"](B)
+        kernel_name = "qkv_decode_cu_kernel<8,3,2> (RMSNorm + QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
+    qkv_graph = graph_of(dominant, n_launch)
     qkv_graph.replay()
     qkv_s = min(time_graph(qkv_graph) for _ in range(5)) / n_launch
-    qkv_bytes = bytes_of["qkv"](B)
     roofline = {
-        "kernel": "qkv_decode_cu_kernel<8,3> (QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)",
+        "kernel": kernel_name,
         "bound": "hbm", "achieved": round(qkv_bytes / qkv_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(qkv_bytes / qkv_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
         "bytes_per_launch": qkv_bytes, "avg_launch_us": round(qkv_s * 1e6, 3),
@@ -231,8 +249,7 @@ def main() -> int:
         bench_kernel("rmsnorm_B8", lambda i: T.rmsnorm_forward(x, scales[i % N_LAYERS], 1e-5, out=t), bytes_of["rmsnorm"](B))
         bench_kernel("embedding_B8", lambda i: T.embedding_forward(ids, table, out=h), bytes_of["embedding"](B))
         bench_kernel("swiglu_M32", lambda i: T.swiglu(swiglu_x, out=s_out), bytes_of["swiglu"](SWIGLU_ROWS))
-        kernels["qkv_rope_decode_B8"] = {"us": roofline["avg_launch_us"], "GB/s": roofline["achieved"], "hbm_frac": roofline["frac"]}
-        for r in (1, 32):
+        for r in (1, 8, 32):
             xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
             pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
             qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),
@@ -241,6 +258,11 @@ def main() -> int:
                          lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
                                                                            yarn=yarn, positions=pr, mode="decode", out=qo),
                          bytes_of["qkv"](r), n=240)
+            bench_kernel(f"norm_qkv_rope_decode_B{r}",
+                         lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
+                                                                           yarn=yarn, positions=pr, mode="decode", out=qo,
+                                                                           norm_scale=scales[i % N_LAYERS]),
+                         bytes_of["norm_qkv"](r), n=240)
         # prefill sizes
         for tt in (2048, 8192):
             xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
@@ -262,6 +284,39 @@ def main() -> int:
         so = torch.empty(32768, HIDDEN, dtype=torch.bfloat16, device=dev)
         bench_kernel("swiglu_M32768", lambda i: T.swiglu(sx, out=so), bytes_of["swiglu"](32768), n=48)
         del sx, so
+
+    # ---------------------------------------------------------------- 24-layer per-token stack (one graph replay = one token step)
+    stack = {}
+    if not args.no_kernel_table:
+        mlp_scales = [(1 + 0.1 * torch.randn(HIDDEN, generator=g)).bfloat16().to(dev) for _ in range(N_LAYERS + 1)]
+        for r in (1, 8, 32):
+            xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
+            pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
+            qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),
+                  torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev))
+            tr = torch.empty_like(xr)
+            sx = (2.0 * torch.randn(4 * r, 2 * HIDDEN, generator=g)).bfloat16().to(dev)
+            so = torch.empty(4 * r, HIDDEN, dtype=torch.bfloat16, device=dev)
+
+            def token_step(_i, xr=xr, pr=pr, qo=qo, tr=tr, sx=sx, so=so):
+                for l in range(N_LAYERS):
+                    if args.unfused:
+                        T.rmsnorm_forward(xr, scales[l], 1e-5, out=tr)
+                        T.qkv_rope_forward(tr, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=pr, mode="decode", out=qo)
+                    else:
+                        T.qkv_rope_forward(xr, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=pr, mode="decode", out=qo,
+                                           norm_scale=scales[l], norm_eps=1e-5)
+                    T.rmsnorm_forward(xr, mlp_scales[l], 1e-5, out=tr)
+                    T.swiglu(sx, out=so)
+                T.rmsnorm_forward(xr, mlp_scales[N_LAYERS], 1e-5, out=tr)
+
+            token_step(0)
+            gr = graph_of(token_step, 4)
+            gr.replay()
+            sec = min(time_graph(gr) for _ in range(5)) / 4
+            launches = N_LAYERS * (4 if args.unfused else 3) + 1
+            stack[f"B{r}"] = {"us_per_token_step": round(sec * 1e6, 2), "tokens/s": round(r / sec, 1), "launches": launches,
+                              "weight_GB/s": round(N_LAYERS * QKV_DIM * HIDDEN * 2 / sec / 1e9, 1)}
 
     # ---------------------------------------------------------------- CPU baseline (reported only)
     cpu_baseline = None
@@ -303,8 +358,9 @@ def main() -> int:
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: B=8 decode step = embedding gather[8] + RMSNorm[8,2880] + QKV+bias+YaRN-RoPE(2880->5120) + "
                                "clamped SwiGLU[32,5760]; 24 rotating weight sets; HIP-graph replay of all steps",
-                   "batch": B, "layers_rotated": N_LAYERS},
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
+                   "batch": B, "layers_rotated": N_LAYERS,
+                   "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel"},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack,
         "wall_s_timed_region": round(wall, 4),
     }
     print(json.dumps(out))

@@ -140,6 +140,20 @@ int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const void* b,
                               int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
                               const TllmRope* rope, void* stream);
 
+/* tllm_rmsnorm_bf16 followed by tllm_qkv_rope_decode_bf16 in one launch: x is the raw
+ * hidden state, the kernel normalises it (fp32, one RNE to bf16 -- the operand the two
+ * separate calls would pass between them) while the weight streams in.
+ * replaces the pair AttentionBlock.forward issues per decode step, model.py:476 + 489-503.
+ * Exists for hidden == 2880, head_dim == 64 (TLLM_E_SHAPE otherwise). Worth it up to 16
+ * rows; beyond that the kernel's 32-row variant is short of registers and the two
+ * separate calls are the faster form (the result is the same either way). */
+int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps,
+                                   const void* W, const void* b, void* q, void* k, void* v,
+                                   int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                                   int64_t kv_slot_stride,
+                                   int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
+                                   const TllmRope* rope, void* stream);
+
 int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const void* b,
                                void* q, void* k, void* v,
                                int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,

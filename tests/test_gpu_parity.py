@@ -228,6 +228,78 @@ def test_qkv_rope_prefill_parity(gpu, yarn, rows):
     _check_qkv(gpu, yarn, rows, "prefill", seed=100 + rows, prefill_positions=rows >= 128)
 
 
+@pytest.mark.parametrize("rows", [1, 5, 8, 16, 17, 32, 50])
+@pytest.mark.parametrize("scale_dtype", [torch.bfloat16, torch.float32])
+def test_norm_qkv_fused_decode_parity(gpu, yarn, rows, scale_dtype):
+    """RMSNorm inside the decode kernel == oracle rmsnorm (rounded to bf16, as the layer boundary does) -> oracle QKV.
+    Rows carry different magnitudes so that a per-row statistic applied to the wrong row would show."""
+    d = O.make_inputs(rows, seed=300 + rows, norm_scale_dtype=scale_dtype)
+    x = (d["x"].float() * (2.0 ** (torch.arange(rows) % 7 - 3))[:, None]).bfloat16()
+    q, k, v = T.qkv_rope_forward(x.to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu),
+                                 mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    t_ref = O.rmsnorm_ref(x, d["norm_scale"].float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"])
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    # and against the two-launch form on the GPU
+    q, k, v = q.clone(), k.clone(), v.clone()
+    t = T.rmsnorm_forward(x.to(gpu), d["norm_scale"].to(gpu), 1e-5)
+    q2, k2, v2 = T.qkv_rope_forward(t, d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), mode="decode")
+    close(q, q2.float().cpu())
+    close(k, k2.float().cpu())
+    close(v, v2.float().cpu())
+
+
+@pytest.mark.parametrize("rows", [17, 32, 50])
+def test_norm_qkv_fused_entry_point_beyond_16_rows(gpu, yarn, rows, monkeypatch):
+    """The host picks two launches beyond 16 rows (faster there); the C entry point itself must still be right."""
+    from tritonllm_amd import ops
+    monkeypatch.setattr(ops, "_norm_fusable", lambda kind, r, hidden, hd: kind == "decode" and hidden == 2880 and hd == 64)
+    d = O.make_inputs(rows, seed=400 + rows)
+    q, k, v = T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu),
+                                 mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"])
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+
+
+def test_norm_qkv_composed_when_not_fusable_and_cache_form(gpu, yarn):
+    """norm_scale on shapes the decode kernel does not fuse (prefill rows, other hidden sizes) runs rmsnorm first;
+    the cache-writing decode call takes it too."""
+    d = O.make_inputs(100, seed=41, norm_scale_dtype=torch.float32)
+    t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"], 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"])
+    q, k, v = T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn,
+                                 positions=d["positions"].to(gpu), mode="prefill", norm_scale=d["norm_scale"].to(gpu))
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    g = O.make_inputs(6, seed=42, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=32)
+    t_ref = O.rmsnorm_ref(g["x"], g["norm_scale"].float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, g["w"], g["b"], g["positions"], 4, 2, 32, base=10000.0, scaling_factor=1.0)
+    q, k, v = T.qkv_rope_forward(g["x"].to(gpu), g["w"].to(gpu), g["b"].to(gpu), 4, 2, 32, yarn=T.YarnParams(head_dim=32, base=10000.0),
+                                 positions=g["positions"].to(gpu), norm_scale=g["norm_scale"].to(gpu))
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    d = O.make_inputs(8, seed=43)
+    slot = 11
+    cache_k = torch.zeros(8, 16, 8, 64, dtype=torch.bfloat16, device=gpu)
+    cache_v = torch.zeros_like(cache_k)
+    rope = T.RotaryEmbedding(64, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=gpu)
+    q = T.qkv_rope_cache_decode_forward(d["x"].view(8, 1, 2880).to(gpu), d["w"].to(gpu), d["b"].to(gpu), rope.sin, rope.cos,
+                                        rope.max_context_length, cache_k, cache_v, torch.tensor([slot], device=gpu), 64, 8, 64,
+                                        norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], torch.full((8,), slot, dtype=torch.int64))
+    close(q.view(8, 4096), qr)
+    close(cache_k[:, slot].reshape(8, 512), kr)
+    close(cache_v[:, slot].reshape(8, 512), vr)
+
+
 def test_qkv_rope_prefill_long_context(gpu, yarn):
     _check_qkv(gpu, yarn, 8192, "prefill", seed=4, prefill_positions=True)
 

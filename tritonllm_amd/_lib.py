@@ -46,6 +46,7 @@ SIGNATURES = {
     "tllm_rope_bf16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, C.POINTER(TllmRope), _vp]),
     "tllm_qkv_rope_decode_bf16": (_i32, _QKV_SIG),
     "tllm_qkv_rope_prefill_bf16": (_i32, _QKV_SIG),
+    "tllm_norm_qkv_rope_decode_bf16": (_i32, [_vp, _vp, _i32, _f32] + _QKV_SIG[1:]),
 }
 
 _lib = None

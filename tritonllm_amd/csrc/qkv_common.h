@@ -19,6 +19,8 @@ struct QkvArgs {
   int hidden;
   int n_q_heads, n_kv_heads, head_dim;
   int has_rope;
+  const void* norm_scale;     // fused RMSNorm prologue (decode fast path only): scale [hidden], fp32 or bf16
+  float norm_eps;
 };
 
 // KV-cache slot the new token goes to (0 when the outputs are plain tensors). A global load: call it early.

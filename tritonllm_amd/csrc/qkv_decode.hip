@@ -52,6 +52,8 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
   a->n_kv_heads = n_kv_heads;
   a->head_dim = head_dim;
   a->has_rope = rope != nullptr;
+  a->norm_scale = nullptr;
+  a->norm_eps = 0.f;
   return TLLM_OK;
 }
 
@@ -201,7 +203,8 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 // partner at row p + 16), N = up to XR activation rows. After one barrier the fifteen partial tiles
 // are summed by 16 x XR threads, one (pair, activation row) each, which also add the bias, rotate
 // with cos/sin they computed while the loads were in flight, round once and store.
-template <int XR, int CH>
+// NORM: 0 = x is used as it is; 1 / 2 = x is first RMS-normalised with an fp32 / bf16 scale (fused prologue).
+template <int XR, int CH, int NORM>
 __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   constexpr int NW = 15, SPW = 6, NCH = SPW / CH, PAIRS = 10;
   constexpr int KV = 360;                 // 16-byte vectors per row (hidden 2880)
@@ -216,6 +219,8 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   static_assert(16 * XR <= 960, "one epilogue thread per (pair slot, activation row)");
   __shared__ __align__(16) unsigned char lds[NW * PATCH];
   __shared__ float s_pin[16];
+  __shared__ float s_part[NORM ? NW * XR : 1], s_rinv[NORM ? XR : 1];
+  static_assert((NCH * XR * CPR + SPW * 32) * 4 <= PATCH, "sum-of-squares and scale scratch alias the wavefront's patch");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int total_pairs = (a.n_q_heads + 2 * a.n_kv_heads) * 32;
@@ -237,13 +242,26 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   const unsigned short* bias_ptr = reinterpret_cast<const unsigned short*>(a.bias ? a.bias : a.W);
   const int64_t pos_ld = *pos_ptr;
   const int64_t off_ld = *off_ptr;
-  const unsigned short b_lo = bias_ptr[ehead * 64 + ed], b_hi = bias_ptr[ehead * 64 + 32 + ed];
+  // The 32-row variant with the fused norm has no register left to hold the two bias values through the kernel
+  // (the compiler would spill them at the very top, behind a full wait for the first loads): it fetches them
+  // after the MFMAs instead, where the two reduction barriers cover the latency.
+  constexpr bool LATE_BIAS = NORM != 0 && XR == 32;
+  unsigned short b_lo = 0, b_hi = 0;
+  if constexpr (!LATE_BIAS) {
+    b_lo = bias_ptr[ehead * 64 + ed];
+    b_hi = bias_ptr[ehead * 64 + 32 + ed];
+  }
   const float freq = fr.v[ed];
   __builtin_amdgcn_sched_barrier(0);
 
   const bf16x8* xg = reinterpret_cast<const bf16x8*>(a.x) + row0 * KV + wave * (SPW * 4);
   const bf16x8* wg = reinterpret_cast<const bf16x8*>(a.W) + wave * (SPW * 4);
   bf16x8 xr[NCH * XL], wr[NCH * WL];
+  // The norm scale of this wavefront's K slice (SPW * 32 values): one load per wavefront, parked in LDS later.
+  f32x4 sc32 = {};
+  bf16x8 sc16 = {};
+  if constexpr (NORM == 1) sc32 = reinterpret_cast<const f32x4*>(a.norm_scale)[wave * (SPW * 8) + (lane < SPW * 8 ? lane : SPW * 8 - 1)];
+  if constexpr (NORM == 2) sc16 = reinterpret_cast<const bf16x8*>(a.norm_scale)[wave * (SPW * 4) + (lane < SPW * 4 ? lane : SPW * 4 - 1)];
 #pragma unroll
   for (int j = 0; j < NCH; ++j) {
 #pragma unroll
@@ -255,17 +273,27 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
       r = r < nvalid ? r : nvalid - 1;
       xr[j * XL + i] = xg[r * KV + j * CPR + kc];
     }
-#pragma unroll
-    for (int i = 0; i < WL; ++i) {          // patch chunk e -> weight row e / CPR: the ten low rows, then their partners
-      int e = i * 64 + lane;
-      e = e < 2 * PAIRS * CPR ? e : 2 * PAIRS * CPR - 1;
-      const int r = e / CPR, kc = e - r * CPR;
-      int gp = pair0 + (r < PAIRS ? r : r - PAIRS);
-      gp = gp < total_pairs ? gp : total_pairs - 1;
-      const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + (r < PAIRS ? 0u : 32u);
-      wr[j * WL + i] = __builtin_nontemporal_load(wg + wrow * static_cast<unsigned>(KV) + j * CPR + kc);
-    }
   }
+  auto load_w = [&](int idx) {               // weight load idx: patch j = idx / WL, chunk slot i = idx % WL
+    const int j = idx / WL, i = idx % WL;
+    int e = i * 64 + lane;                    // patch chunk e -> weight row e / CPR: the ten low rows, then their partners
+    e = e < 2 * PAIRS * CPR ? e : 2 * PAIRS * CPR - 1;
+    const int r = e / CPR, kc = e - r * CPR;
+    int gp = pair0 + (r < PAIRS ? r : r - PAIRS);
+    gp = gp < total_pairs ? gp : total_pairs - 1;
+    const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + (r < PAIRS ? 0u : 32u);
+    wr[idx] = __builtin_nontemporal_load(wg + wrow * static_cast<unsigned>(KV) + j * CPR + kc);
+  };
+  // A CU holds a bounded number of loads in flight and a wavefront stalls when it issues one beyond that. With
+  // the fused norm every wavefront must see its activations, and meet the others at a barrier, before any MFMA
+  // can start; a wavefront stuck issuing weight loads would get there only when the stream has almost drained.
+  // So only the first NEARLY weight loads are requested up front (enough to keep the memory pipe busy during
+  // the norm), behind a rendezvous that puts every wavefront's activation loads ahead of them in the queue;
+  // the rest follow right after the norm's barriers.
+  constexpr int NEARLY = NORM == 0 ? NCH * WL : (XR == 32 ? 0 : 2);   // XR == 32 has no registers to spare for any
+  if constexpr (NORM != 0) __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int idx = 0; idx < NEARLY; ++idx) load_w(idx);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- cos/sin of this thread's (pair, row) while the weights are in flight.
@@ -274,11 +302,112 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   s_pin[es] = freq;
   float cs = 1.f, sn = 0.f;
   const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
-  if (a.has_rope) {
+  // Only the first 16 * XR threads have an epilogue role; the test is uniform per wavefront, and the other
+  // wavefronts must skip this: the 64-bit position arithmetic and the sincos are some six hundred vector
+  // instructions, and fifteen wavefronts doing them on four SIMDs would take as long as the whole weight stream.
+  if (a.has_rope && tid < 16 * XR) {
     int64_t pos = ra.positions ? pos_ld : (erow % ra.tokens_per_batch) + (ra.offset ? off_ld : 0);
     pos = rope_wrap(pos, ra.max_ctx);
     if (ra.use_yarn) yarn_cos_sin(pos, freq, ra.concentration, &cs, &sn);
     else rope_cos_sin(ra, fr, pos, ed, &cs, &sn);
+  }
+
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- fused RMSNorm prologue: turn the raw activation chunks held in registers into
+  // bf16(x * rsqrt(mean(x^2) + eps) * scale), the exact operand the two-launch form passes between its kernels.
+  // Sum of squares: per-chunk partials -> the wavefront's LDS patch (idle so far) -> one lane per row adds its
+  // row's chunks -> the fifteen K slices meet in s_part -> s_rinv.
+  if constexpr (NORM != 0) {
+    float* tmp = reinterpret_cast<float*>(lds + wave * PATCH);
+    float* wscale = tmp + NCH * XR * CPR;
+    if constexpr (NORM == 1) {
+      if (lane < SPW * 8) reinterpret_cast<f32x4*>(wscale)[lane] = sc32;
+    } else {
+      if (lane < SPW * 4) {
+        f32x4 lo4, hi4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          lo4[q] = static_cast<float>(sc16[q]);
+          hi4[q] = static_cast<float>(sc16[4 + q]);
+        }
+        reinterpret_cast<f32x4*>(wscale)[2 * lane] = lo4;
+        reinterpret_cast<f32x4*>(wscale)[2 * lane + 1] = hi4;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NCH * XL; ++c) {
+      const int e = (c % XL) * 64 + lane;
+      float ssq = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float f = static_cast<float>(xr[c][q]);
+        ssq = fmaf(f, f, ssq);
+      }
+      if (e < XR * CPR) tmp[(c / XL) * (XR * CPR) + e] = ssq;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (lane < XR) {
+      float p = 0.f;
+#pragma unroll
+      for (int j = 0; j < NCH; ++j) {
+#pragma unroll
+        for (int c = 0; c < CPR / 4; ++c) {
+          const f32x4 t4 = *reinterpret_cast<const f32x4*>(tmp + j * (XR * CPR) + lane * CPR + 4 * c);
+          p += (t4[0] + t4[1]) + (t4[2] + t4[3]);
+        }
+      }
+      s_part[wave * XR + lane] = p;
+    }
+    __syncthreads();
+    if (tid < XR) {
+      float ss = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) ss += s_part[w * XR + tid];
+      s_rinv[tid] = rsqrtf(ss * (1.0f / 2880.0f) + a.norm_eps);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int idx = NEARLY; idx < NCH * WL; ++idx) load_w(idx);
+    __builtin_amdgcn_sched_barrier(0);
+    // Chunk c's scale values and 1/rms are fetched from LDS while chunk c-1 is being scaled, and each chunk is
+    // fenced off from the next: written plainly, the compiler either serialises every LDS latency or sinks the
+    // arithmetic down to the patch writes and keeps every chunk's scale values alive until then, next to all the
+    // weight loads' destination registers (it then spills those, with a full drain of the load queue each).
+    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+    constexpr int NC = NCH * XL;
+    f32x4 s_lo, s_hi, n_lo = {}, n_hi = {};
+    float rinv, n_rinv = 0.f;
+    auto fetch = [&](int c, f32x4& lo4, f32x4& hi4, float& ri) {
+      int e = (c % XL) * 64 + lane;
+      e = e < XR * CPR ? e : XR * CPR - 1;
+      const f32x4* sp = reinterpret_cast<const f32x4*>(wscale) + 2 * ((c / XL) * CPR + e % CPR);
+      lo4 = sp[0];
+      hi4 = sp[1];
+      ri = s_rinv[e / CPR];
+    };
+    fetch(0, s_lo, s_hi, rinv);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      if (c + 1 < NC) fetch(c + 1, n_lo, n_hi, n_rinv);
+      __builtin_amdgcn_sched_barrier(0);
+      u32x4 bits = __builtin_bit_cast(u32x4, xr[c]);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        asm volatile("" : "+v"(bits[q]));       // the fp32 copies of the sum-of-squares pass must not stay alive
+        bf16x2 t;
+        t[0] = static_cast<bf16>(__uint_as_float(bits[q] << 16) * rinv * (q < 2 ? s_lo[2 * q] : s_hi[2 * q - 4]));
+        t[1] = static_cast<bf16>(__uint_as_float(bits[q] & 0xffff0000u) * rinv * (q < 2 ? s_lo[2 * q + 1] : s_hi[2 * q - 3]));
+        bits[q] = __builtin_bit_cast(unsigned, t);
+        asm volatile("" : "+v"(bits[q]));       // ... and the arithmetic must not sink to the patch write below
+      }
+      xr[c] = __builtin_bit_cast(bf16x8, bits);
+      __builtin_amdgcn_sched_barrier(0);
+      s_lo = n_lo;
+      s_hi = n_hi;
+      rinv = n_rinv;
+    }
   }
 
   f32x16 acc;
@@ -315,7 +444,10 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
-
+  if constexpr (LATE_BIAS) {
+    b_lo = bias_ptr[ehead * 64 + ed];
+    b_hi = bias_ptr[ehead * 64 + 32 + ed];
+  }
   // ---- fifteen partial tiles -> LDS as [wave][tile row][activation row] (lanes of one store hit distinct banks)
   __syncthreads();
   float* red = reinterpret_cast<float*>(lds);
@@ -349,6 +481,47 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 
 using namespace tllm;
 
+static void launch_cu(int xr, int norm, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+#define TLLM_CU(XR, CH)                                                                                      \
+  do {                                                                                                       \
+    if (norm == 0) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, 0>), grid, dim3(960), 0, st, a, ra, fr);      \
+    else if (norm == 1) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, 1>), grid, dim3(960), 0, st, a, ra, fr); \
+    else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, 2>), grid, dim3(960), 0, st, a, ra, fr);                \
+  } while (0)
+  if (xr == 8) TLLM_CU(8, 3);
+  else if (xr == 16) TLLM_CU(16, 3);
+  else TLLM_CU(32, 2);
+#undef TLLM_CU
+}
+
+extern "C" int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps, const void* W,
+                                              const void* b, void* q, void* k, void* v, int64_t q_row_stride, int64_t k_row_stride,
+                                              int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows, int64_t hidden, int n_q_heads,
+                                              int n_kv_heads, int head_dim, const TllmRope* rope, void* stream) {
+  QkvArgs a;
+  RopeArgs ra;
+  YarnFreqs fr;
+  int rc = qkv_validate("norm_qkv_rope_decode", x, W, q, k, v, q_row_stride, k_row_stride, v_row_stride, kv_slot_stride, rows, hidden,
+                        n_q_heads, n_kv_heads, head_dim, rope, &a, &ra, &fr);
+  if (rc != TLLM_OK) return rc;
+  TLLM_REQUIRE(norm_scale != nullptr, TLLM_E_ARG, "norm_qkv_rope_decode: norm_scale is NULL");
+  TLLM_REQUIRE(hidden == 2880 && head_dim == 64, TLLM_E_SHAPE,
+               "norm_qkv_rope_decode: the fused kernel exists for hidden 2880 / head_dim 64 only (got %lld / %d); "
+               "call tllm_rmsnorm_bf16 and tllm_qkv_rope_decode_bf16", (long long)hidden, head_dim);
+  TLLM_REQUIRE(aligned16(x) && aligned16(W) && aligned16(norm_scale), TLLM_E_ALIGN, "norm_qkv_rope_decode: x, W and norm_scale must be 16-byte aligned");
+  a.bias = (const bf16*)b;
+  a.norm_scale = norm_scale;
+  a.norm_eps = eps;
+  if (rows == 0) return TLLM_OK;
+  const int heads = n_q_heads + 2 * n_kv_heads;
+  TLLM_REQUIRE(static_cast<int64_t>(heads) * 64 * hidden < (1ll << 31), TLLM_E_SHAPE, "norm_qkv_rope_decode: weight too large");
+  const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
+  const int64_t chunks = (rows + xr - 1) / xr;
+  TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "norm_qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
+  launch_cu(xr, scale_is_bf16 ? 2 : 1, dim3((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks), static_cast<hipStream_t>(stream), a, ra, fr);
+  return check_launch("norm_qkv_rope_decode");
+}
+
 extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const void* b, void* q, void* k, void* v, int64_t q_row_stride,
                                          int64_t k_row_stride, int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows,
                                          int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope,
@@ -370,12 +543,7 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
     const int64_t chunks = (rows + xr - 1) / xr;
     TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
     dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
-    if (xr == 8)
-      hipLaunchKernelGGL((qkv_decode_cu_kernel<8, 3>), grid, dim3(960), 0, st, a, ra, fr);
-    else if (xr == 16)
-      hipLaunchKernelGGL((qkv_decode_cu_kernel<16, 3>), grid, dim3(960), 0, st, a, ra, fr);
-    else
-      hipLaunchKernelGGL((qkv_decode_cu_kernel<32, 2>), grid, dim3(960), 0, st, a, ra, fr);
+    launch_cu(xr, 0, grid, st, a, ra, fr);
     return check_launch("qkv_rope_decode");
   }
   const bool out4 = (reinterpret_cast<uintptr_t>(q) % 4 == 0) && (reinterpret_cast<uintptr_t>(k) % 4 == 0) &&

@@ -185,7 +185,29 @@ def rope_forward(query: torch.Tensor, key: torch.Tensor, sin: torch.Tensor | Non
 
 
 # --------------------------------------------------------------------------------------- fused QKV
-def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_stride, n_q, n_kv, hd, desc):
+def _norm_fusable(kind: str, rows: int, hidden: int, hd: int) -> bool:
+    """The decode kernel can normalise its own activations for the gpt-oss shape; beyond 16 rows
+    its 32-row variant is out of registers and the two launches are the faster form."""
+    return kind == "decode" and hidden == 2880 and hd == 64 and rows <= 16
+
+
+def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_stride, n_q, n_kv, hd, desc, norm=None):
+    """``norm = (scale, eps)``: x2 is the raw hidden state and is RMS-normalised first -- inside
+    the decode kernel where it can, by a preceding rmsnorm launch otherwise."""
+    if norm is not None:
+        scale, eps = norm
+        assert scale.dtype in (torch.float32, _BF16) and scale.shape == (x2.shape[1],)
+        if not scale.is_contiguous():
+            scale = scale.contiguous()
+        if _norm_fusable(kind, x2.shape[0], x2.shape[1], hd):
+            rc = lib().tllm_norm_qkv_rope_decode_bf16(
+                x2.data_ptr(), scale.data_ptr(), int(scale.dtype == _BF16), float(eps), weight.data_ptr(),
+                bias.data_ptr() if bias is not None else None, q.data_ptr() if q is not None else None,
+                k.data_ptr() if k is not None else None, v.data_ptr() if v is not None else None, q_rs, k_rs, v_rs,
+                kv_slot_stride, x2.shape[0], x2.shape[1], n_q, n_kv, hd, C.byref(desc) if desc is not None else None, _stream())
+            check(rc, "norm_qkv_rope_decode")
+            return
+        x2 = rmsnorm_forward(x2, scale, eps)
     fn = lib().tllm_qkv_rope_decode_bf16 if kind == "decode" else lib().tllm_qkv_rope_prefill_bf16
     rc = fn(x2.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
             q.data_ptr() if q is not None else None, k.data_ptr() if k is not None else None,
@@ -209,14 +231,18 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
                      head_dim: int, *, yarn: YarnParams | None = None, cos: torch.Tensor | None = None,
                      sin: torch.Tensor | None = None, positions: torch.Tensor | None = None, offset: torch.Tensor | None = None,
                      tokens_per_batch: int | None = None, max_context_length: int = 131072, rotate: bool = True,
-                     mode: str = "auto", out: tuple | None = None):
+                     mode: str = "auto", out: tuple | None = None, norm_scale: torch.Tensor | None = None,
+                     norm_eps: float = 1e-5):
     """RMS-normed activations ``x [rows, hidden]`` -> ``(q [rows, Hq*D], k [rows, Hkv*D], v [rows, Hkv*D])``.
+
+    With ``norm_scale`` given, ``x`` is the raw hidden state and the call also performs the
+    ``RMSNorm(x)`` of model.py:476 (inside the same kernel for decode-sized gpt-oss shapes).
 
     One fused kernel: projection, bias, rotary on q/k (fp32 accumulator, one rounding),
     outputs written to three dense tensors. ``mode``: "decode" (weight streaming),
     "prefill" (MFMA GEMM) or "auto" (by row count). No reference twin as a single call:
     it is F.linear + split + contiguous + rope_forward of model.py:506-522 in one launch."""
-    _on_gpu(x, weight, bias, positions, offset, cos, sin)
+    _on_gpu(x, weight, bias, positions, offset, cos, sin, norm_scale)
     assert x.ndim == 2
     rows, hidden = x.shape
     total_out, hidden_w = weight.shape
@@ -241,7 +267,8 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     if mode == "auto":
         mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
     assert mode in ("decode", "prefill")
-    _launch_qkv(mode, x, weight, bias, q, k, v, q.stride(0), k.stride(0), v.stride(0), 0, num_q_heads, num_kv_heads, head_dim, desc)
+    _launch_qkv(mode, x, weight, bias, q, k, v, q.stride(0), k.stride(0), v.stride(0), 0, num_q_heads, num_kv_heads, head_dim, desc,
+                norm=None if norm_scale is None else (norm_scale, norm_eps))
     return q, k, v
 
 
@@ -274,12 +301,14 @@ def qkv_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias: torch.T
 
 def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_length, cache_k, cache_v, offset, num_q_heads,
                                   num_kv_heads, head_dim, weight_scale=None, *, yarn: YarnParams | None = None,
-                                  positions: torch.Tensor | None = None):
+                                  positions: torch.Tensor | None = None, norm_scale: torch.Tensor | None = None,
+                                  norm_eps: float = 1e-5):
     """Fused decode step: projection + bias + rotary; the rotated k and the raw v of the
     new token are written into the KV cache at slot ``offset``; q ``[B,1,Hq*D]`` is returned
     (a borrowed pool buffer). ``offset`` is an int64 device tensor of shape (1,) and is read
-    on the device, so the call can be replayed from a HIP graph."""
-    _on_gpu(hidden, weight, bias, cache_k, cache_v, offset, positions)
+    on the device, so the call can be replayed from a HIP graph. With ``norm_scale`` the
+    block's input RMSNorm (model.py:476) runs inside the same kernel on the raw ``hidden``."""
+    _on_gpu(hidden, weight, bias, cache_k, cache_v, offset, positions, norm_scale)
     if weight_scale is not None:
         raise NotImplementedError("fp8 weights with per-row scales are not implemented in the HIP path")
     batch, num_tokens, hidden_size = hidden.shape
@@ -301,7 +330,8 @@ def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_le
     keep: list = []
     desc = _rope_desc(cos, sin, yarn, positions, offset, 1, max_context_length, keep)
     _launch_qkv("decode", x2, weight, bias, q, cache_k, cache_v, num_q_heads * head_dim, cache_k.stride(0), cache_v.stride(0),
-                cache_k.stride(1), num_q_heads, num_kv_heads, head_dim, desc)
+                cache_k.stride(1), num_q_heads, num_kv_heads, head_dim, desc,
+                norm=None if norm_scale is None else (norm_scale, norm_eps))
     return q.reshape(batch, 1, num_q_heads * head_dim)
 
 
