@@ -262,18 +262,25 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   bf16x8 sc16 = {};
   if constexpr (NORM == 1) sc32 = reinterpret_cast<const f32x4*>(a.norm_scale)[wave * (SPW * 8) + (lane < SPW * 8 ? lane : SPW * 8 - 1)];
   if constexpr (NORM == 2) sc16 = reinterpret_cast<const bf16x8*>(a.norm_scale)[wave * (SPW * 4) + (lane < SPW * 4 ? lane : SPW * 4 - 1)];
+  auto load_x = [&]() {
 #pragma unroll
-  for (int j = 0; j < NCH; ++j) {
+    for (int j = 0; j < NCH; ++j) {
 #pragma unroll
-    for (int i = 0; i < XL; ++i) {          // patch chunk e -> activation row e / CPR, chunk e % CPR
-      int e = i * 64 + lane;
-      e = e < XR * CPR ? e : XR * CPR - 1;
-      int r = e / CPR;
-      const int kc = e - r * CPR;
-      r = r < nvalid ? r : nvalid - 1;
-      xr[j * XL + i] = xg[r * KV + j * CPR + kc];
+      for (int i = 0; i < XL; ++i) {          // patch chunk e -> activation row e / CPR, chunk e % CPR
+        int e = i * 64 + lane;
+        e = e < XR * CPR ? e : XR * CPR - 1;
+        int r = e / CPR;
+        const int kc = e - r * CPR;
+        r = r < nvalid ? r : nvalid - 1;
+        xr[j * XL + i] = xg[r * KV + j * CPR + kc];
+      }
     }
-  }
+  };
+  // Order of the requests. All 256 workgroups read the same few activation rows, which the L2s can only hand
+  // out at their own pace (32 CUs per L2 asking for the same lines), while the weight stream has the whole
+  // HBM latency ahead of it: without the norm the weight requests go first and the activations follow in
+  // their shadow. With the fused norm the activations are needed first (see below).
+  if constexpr (NORM != 0) load_x();
   auto load_w = [&](int idx) {               // weight load idx: patch j = idx / WL, chunk slot i = idx % WL
     const int j = idx / WL, i = idx % WL;
     int e = i * 64 + lane;                    // patch chunk e -> weight row e / CPR: the ten low rows, then their partners
@@ -294,6 +301,7 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   if constexpr (NORM != 0) __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int idx = 0; idx < NEARLY; ++idx) load_w(idx);
+  if constexpr (NORM == 0) load_x();
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- cos/sin of this thread's (pair, row) while the weights are in flight.

@@ -12,14 +12,21 @@
 // cannot be padded; instead the chunk order inside each row is XOR-swizzled with the row index --
 // applied by choosing which *global* chunk a lane fetches -- and the fragment reads undo it, which
 // keeps the 128-bit fragment reads of 16 consecutive rows conflict-free.
-// With one tile per CU nothing but the kernel's own schedule hides memory latency:
-//   * the one barrier per slice sits before the slice's last MFMA group, and the loads of the slice
-//     after next are issued right behind it, so their latency overlaps a whole slice of MFMAs and
-//     both fragment prefetches (rest of this slice, head of the next) overlap MFMAs too;
+// With one tile per CU (one wavefront per SIMD) nothing but the kernel's own schedule overlaps anything:
+//   * the one barrier per slice sits before the slice's last k16 step; the stage just finished is handed to
+//     the slice after next, whose loads go out one per MFMA behind that step and the next (never fourteen
+//     in a row: a CU's load queue is bounded and a wavefront that overflows it stalls, MFMAs included);
+//   * the fragment reads of the next k16 step are pinned between the MFMAs of the current one
+//     (sched_group_barrier): hoisted to the top of the iteration, as the compiler does by itself, the four
+//     wavefronts read their 112 KB per slice in one burst with no MFMA running;
 //   * an L2 miss still costs more than a slice of MFMAs and LDS has no room for a third stage, so
 //     three slices ahead every workgroup touches (one dword per line) its share of the lines its
 //     XCD's tiles are going to need, which pulls them into that XCD's L2 in time;
-//   * measured: the loop is bound by the L2->LDS feed (57 KB per slice per CU), not by the MFMAs.
+//   * measured with per-slice cycle stamps: the waits for loads and at the barrier are ~10 % of a slice; the
+//     rest is the MFMA / LDS phase itself at ~1.5x the 1280 MFMA cycles. LDS is the binding resource: per
+//     slice 112 KB of fragment reads plus 57 KB of incoming tile data against 128 B/clk is 1320 cycles at
+//     best, i.e. this tiling cannot run the MFMAs much above two thirds busy, and the clock under this
+//     load is ~1.85-1.9 GHz rather than the 2.4 GHz of the published peak.
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
@@ -201,13 +208,34 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
 #pragma unroll
     for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(st + fb_off[kk][nb]);
   };
-  auto mfma_group = [&](const bf16x8 (&fa)[2], const bf16x8 (&fb)[5]) {
+  auto issue_load = [&](int it, int j) {                // one load instruction of slice `it`
+    unsigned char* dst = smem + (it % NS) * STAGE + wave * (LPW * 1024);
+    const int itc = it < n_iter ? it : n_iter - 1;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + itc * CHUNKS),
+                                     (__attribute__((address_space(3))) void*)(dst + blk_off[j]), 16, 0, 0);
+  };
+  // One k16 step: ten MFMAs on the fragments in buffer `cur`. Behind MFMA m goes the LDS read of fragment m of
+  // the next step (seven of them, into buffer cur ^ 1) and, for m < n, one global->LDS load instruction
+  // (j0 + m) of slice `lit`. The interleaving is pinned with sched_group_barrier, for two reasons:
+  //   * left alone, the compiler hoists all 28 fragment reads of a slice to the top of the iteration; the four
+  //     wavefronts then read 112 KB from LDS in one burst (~900 cycles with no MFMA running) and do their 40
+  //     MFMAs afterwards -- the two costs add up instead of overlapping;
+  //   * a CU takes only so many loads into its queue and a wavefront that issues one more stalls, MFMAs
+  //     included (there is one wavefront per SIMD), until the queue has drained that far; fourteen loads in a
+  //     row do exactly that. Handed out one per MFMA (32 cycles) they never find the queue full.
+  bf16x8 fa[2][2], fb[2][5];
+  auto step = [&](int cur, const unsigned char* nst, int nkk, int lit, int j0, int n) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int nb = 0; nb < 5; ++nb) {
-        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nb], fa[mb], acc[mb][nb], 0, 0, 0);   // weights on M, tokens on N
-      }
+    for (int m = 0; m < 10; ++m) {
+      const int mb = m / 5, nb = m % 5;
+      acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][nb], fa[cur][mb], acc[mb][nb], 0, 0, 0);   // weights on M, tokens on N
+      if (m < 2) fa[cur ^ 1][m] = *reinterpret_cast<const bf16x8*>(nst + fa_off[nkk][m]);
+      else if (m < 7) fb[cur ^ 1][m - 2] = *reinterpret_cast<const bf16x8*>(nst + fb_off[nkk][m - 2]);
+      if (m < n) issue_load(lit, j0 + m);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // one MFMA
+      if (m < 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // one LDS read
+      if (m < n) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // one VMEM read
+    }
   };
 
   // prologue: slices 0..NS-2 in flight, slice 0 landed
@@ -235,29 +263,34 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   }
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPW) : "memory");
   __syncthreads();
-  bf16x8 fa[2][2], fb[2][5];
   load_frags(smem, 0, fa[0], fb[0]);
 
   // Steady state: slices it+1 .. it+NS-1 are in flight or landed while slice it is multiplied. The one
-  // barrier per slice sits before the slice's last MFMA group; right behind it the stage being finished
-  // is handed to slice it+NS (all reads of it have been issued), so the next loads start a whole MFMA
-  // group before the iteration ends and their latency overlaps the following slice's MFMAs.
+  // barrier per slice sits before the slice's last k16 step; from there on the stage of slice `it` is free
+  // (all reads of it have been issued) and is handed to slice it+NS, whose loads go out behind the MFMAs of
+  // this last step (ten of them) and of the next slice's first step (the other four) -- a whole slice of
+  // MFMAs before they are needed.
   issue_loads(NS - 1);
   issue_touch(kTouchDist);
   for (int it = 0; it < n_iter; ++it) {
     const unsigned char* st = smem + (it % NS) * STAGE;
+    const unsigned char* nx = smem + ((it + 1) % NS) * STAGE;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) {
       if (kk + 1 < KS) {
-        load_frags(st, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+        if (kk == 0 && it > 0) {
+          step(kk & 1, st, kk + 1, it + NS - 1, 10, LPW - 10);
+          issue_touch(it + kTouchDist);             // youngest in the queue: the wait below leaves it outstanding
+        } else {
+          step(kk & 1, st, kk + 1, 0, 0, 0);
+        }
       } else {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * (LPW + kTouch) + kTouch) : "memory");   // slice it+1 has landed (this wavefront's share)
-        __syncthreads();                                // ... everyone's share; and everyone has issued its last reads of slice it
-        issue_loads(it + NS);
-        issue_touch(it + 1 + kTouchDist);          // youngest in the queue: the wait above leaves it outstanding
-        load_frags(smem + ((it + 1) % NS) * STAGE, 0, fa[0], fb[0]);
+        // Slice it+1 has landed (this wavefront's share; the touch stays in flight), then the barrier: everyone's
+        // share has, and everyone has issued its last reads of slice it. Spelled out, because __syncthreads()
+        // carries a fence that drains every load in flight, the look-ahead ones included.
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * (LPW + kTouch) + kTouch) : "memory");
+        step(kk & 1, nx, 0, it + NS, 0, 10);
       }
-      mfma_group(fa[kk & 1], fb[kk & 1]);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch_sink)::"memory");   // drain the look-ahead loads before LDS is reused
