@@ -49,6 +49,9 @@ def algorithmic_bytes():
         "swiglu": lambda m: m * (2 * HIDDEN * 2 + HIDDEN * 2),
         "qkv": lambda r: w + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
         "norm_qkv": lambda r: w + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
+        # fp8 weight: one byte per element + one fp32 scale per output row
+        "qkv_w8": lambda r: w // 2 + QKV_DIM * 4 + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
+        "norm_qkv_w8": lambda r: w // 2 + QKV_DIM * 4 + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
     }
 
 
@@ -58,17 +61,20 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
     kind, _, size = name.rpartition("_")
     n = int(size[1:])
     flops = nbytes = None
-    if kind in ("qkv_rope_prefill", "qkv_rope_decode", "norm_qkv_rope_decode"):
+    if kind in ("qkv_rope_prefill", "qkv_rope_decode", "norm_qkv_rope_decode", "qkv_rope_decode_w8", "norm_qkv_rope_decode_w8"):
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         pp = torch.arange(n, dtype=torch.int64, device=dev) if kind.endswith("prefill") else \
             torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
         qo = (torch.empty(n, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev),
               torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev))
         mode = "prefill" if kind.endswith("prefill") else "decode"
-        fused = kind.startswith("norm_")
-        fn = lambda i: T.qkv_rope_forward(xp, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn, positions=pp,
-                                          mode=mode, out=qo, norm_scale=scales[i % N_LAYERS] if fused else None)
-        flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of["norm_qkv" if fused else "qkv"](n)
+        fused, w8 = kind.startswith("norm_"), kind.endswith("_w8")
+        wq = [T.quantize_fp8_rows(w) for w in weights] if w8 else None
+        fn = lambda i: T.qkv_rope_forward(xp, wq[i % N_LAYERS][0] if w8 else weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
+                                          yarn=yarn, positions=pp, mode=mode, out=qo,
+                                          norm_scale=scales[i % N_LAYERS] if fused else None,
+                                          weight_scale=wq[i % N_LAYERS][1] if w8 else None)
+        flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of[("norm_qkv" if fused else "qkv") + ("_w8" if w8 else "")](n)
     elif kind == "rmsnorm":
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         to = torch.empty_like(xp)
@@ -270,6 +276,26 @@ def main() -> int:
                                                                            yarn=yarn, positions=pr, mode="decode", out=qo,
                                                                            norm_scale=scales[i % N_LAYERS]),
                          bytes_of["norm_qkv"](r), n=240)
+        # the same stream with the weight quantised to fp8 e4m3 + per-row scales (the reference's ATTN_FP8 option)
+        wq = [T.quantize_fp8_rows(w) for w in weights]
+        for r in (1, 8, 32):
+            xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
+            pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
+            qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),
+                  torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev))
+            bench_kernel(f"qkv_rope_decode_w8_B{r}",
+                         lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, wq[i % N_LAYERS][0], biases[i % N_LAYERS], NQ, NKV, HD,
+                                                                           yarn=yarn, positions=pr, mode="decode", out=qo,
+                                                                           weight_scale=wq[i % N_LAYERS][1]),
+                         bytes_of["qkv_w8"](r), n=240)
+            if r == 8:
+                bench_kernel("norm_qkv_rope_decode_w8_B8",
+                             lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, wq[i % N_LAYERS][0], biases[i % N_LAYERS], NQ, NKV, HD,
+                                                                               yarn=yarn, positions=pr, mode="decode", out=qo,
+                                                                               norm_scale=scales[i % N_LAYERS],
+                                                                               weight_scale=wq[i % N_LAYERS][1]),
+                             bytes_of["norm_qkv_w8"](r), n=240)
+        del wq
         # prefill sizes
         for tt in (2048, 8192):
             xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)

@@ -154,6 +154,19 @@ int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int sc
                                    int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
                                    const TllmRope* rope, void* stream);
 
+/* The decode projection with an fp8 weight: W8 is [n_heads*64, hidden] OCP e4m3 bytes, w_scale one fp32
+ * per output row, W[n][k] = fp8(W8[n][k]) * w_scale[n] (the reference's per-row quantisation,
+ * triton_kernels.py:261-268; its use in the fused decode kernel, :927-940 and :963-965, argument
+ * weight_scale of qkv_rope_cache_decode_forward :1109). Half the bytes of the bf16 kernel; activations stay
+ * bf16, accumulation fp32. norm_scale may be NULL (no fused RMSNorm) or as in tllm_norm_qkv_rope_decode_bf16.
+ * Exists for hidden == 2880, head_dim == 64 (TLLM_E_SHAPE otherwise). */
+int tllm_qkv_rope_decode_w8_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps,
+                                 const void* W8, const float* w_scale, const void* b, void* q, void* k, void* v,
+                                 int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                                 int64_t kv_slot_stride,
+                                 int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
+                                 const TllmRope* rope, void* stream);
+
 int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const void* b,
                                void* q, void* k, void* v,
                                int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,

@@ -31,6 +31,8 @@ force and special cases -- in ``tests/test_oracle_pins.py``:
     qkv_rope_ref                      composition of the above, v slice un-rotated
     swiglu_ref                        float64 brute force, edge grid, l=-1 => 0,
                                       interleaved == chunked under permutation
+    quantize_fp8_rows_ref /           all 256 e4m3 codes against the OCP bit formula, row maxima map to
+    dequant_fp8_ref                   +-448, round-trip error within half a step of the format
 
 The third-party arithmetic underneath (torch.cos/sin/pow/rsqrt, F.linear) is
 PyTorch's, un-pinned by the reference (its README leaves torch unversioned);
@@ -134,6 +136,24 @@ def linear_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None)
     if bias is not None:
         out = out + bias.to(torch.float32)
     return out
+
+
+def quantize_fp8_rows_ref(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """triton_kernels.py:261-268 (``_quantize_unembed_fp8``): per-row e4m3 quantisation.
+
+    scale[n] = max_k |W[n,k]| / 448 (fp32, floor 1e-12); W8 = fp8_e4m3fn(W / scale). Returns
+    (W8 ``[n, k]`` float8_e4m3fn, scale ``[n]`` fp32)."""
+    w = weight.to(torch.float32)
+    max_fp8 = torch.finfo(torch.float8_e4m3fn).max
+    amax = w.abs().max(dim=1, keepdim=True).values.clamp(min=1e-12)
+    scale = (amax / max_fp8).squeeze(1).to(torch.float32)
+    w8 = (w / scale[:, None].clamp(min=1e-12)).to(torch.float8_e4m3fn)
+    return w8, scale
+
+
+def dequant_fp8_ref(w8: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """triton_kernels.py:963-965: the weight the fp8 kernels multiply with, ``fp32(W8) * scale[row]``. fp32."""
+    return w8.to(torch.float32) * scale.to(torch.float32)[:, None]
 
 
 def rope_rotate_ref(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:

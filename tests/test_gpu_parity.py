@@ -266,6 +266,59 @@ def test_norm_qkv_fused_entry_point_beyond_16_rows(gpu, yarn, rows, monkeypatch)
     close(v, vr)
 
 
+@pytest.mark.parametrize("rows", [1, 8, 13, 16, 32, 40])
+@pytest.mark.parametrize("with_norm", [False, True])
+def test_qkv_fp8_weight_decode_parity(gpu, yarn, rows, with_norm):
+    """fp8 e4m3 weight + per-row scale (triton_kernels.py:261-268, 927-965): the kernel must equal the oracle's
+    projection with the dequantised weight fp32(W8) * scale; the quantiser must equal the oracle's bit for bit."""
+    d = O.make_inputs(rows, seed=500 + rows)
+    w8_ref, s_ref = O.quantize_fp8_rows_ref(d["w"])
+    w8, s = T.quantize_fp8_rows(d["w"].to(gpu))
+    # the quantiser is torch arithmetic on the GPU: same scales to the last bits, same codes except where the GPU's
+    # division rounds a quotient to the other side of an fp8 tie
+    torch.testing.assert_close(s.cpu(), s_ref, rtol=1e-6, atol=0)
+    assert (w8.cpu().view(torch.uint8) != w8_ref.view(torch.uint8)).float().mean().item() < 1e-3
+    w8_ref, s_ref = w8.cpu(), s.cpu()          # the kernel is checked on exactly the bytes it was given
+    kw = dict(norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5) if with_norm else {}
+    q, k, v = T.qkv_rope_forward(d["x"].to(gpu), w8, d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu),
+                                 mode="decode", weight_scale=s, **kw)
+    xin = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16() if with_norm else d["x"]
+    qr, kr, vr = O.qkv_rope_ref(xin, O.dequant_fp8_ref(w8_ref, s_ref), d["b"], d["positions"])
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+
+
+def test_qkv_fp8_weight_cache_form_module_and_refusals(gpu, yarn, monkeypatch):
+    d = O.make_inputs(8, seed=51)
+    monkeypatch.setenv("ATTN_FP8", "1")
+    qkv = T.QKV(2880, 5120, device=gpu)
+    with torch.no_grad():
+        qkv.weight.copy_(d["w"])
+        qkv.bias.copy_(d["b"])
+    w8, ws = qkv._fp8_weight
+    assert w8.dtype == torch.float8_e4m3fn and ws.shape == (5120,) and qkv._fp8_weight[0] is w8      # quantised once
+    rope = T.RotaryEmbedding(64, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=gpu)
+    slot = 5
+    cache_k = torch.zeros(8, 16, 8, 64, dtype=torch.bfloat16, device=gpu)
+    cache_v = torch.zeros_like(cache_k)
+    q = T.qkv_rope_cache_decode_forward(d["x"].view(8, 1, 2880).to(gpu), w8, qkv.bias, rope.sin, rope.cos, rope.max_context_length,
+                                        cache_k, cache_v, torch.tensor([slot], device=gpu), 64, 8, 64, ws)
+    qr, kr, vr = O.qkv_rope_ref(d["x"], O.dequant_fp8_ref(w8.cpu(), ws.cpu()), d["b"], torch.full((8,), slot, dtype=torch.int64))
+    close(q.view(8, 4096), qr)
+    close(cache_k[:, slot].reshape(8, 512), kr)
+    close(cache_v[:, slot].reshape(8, 512), vr)
+    monkeypatch.delenv("ATTN_FP8")
+    assert T.QKV(2880, 5120, device=gpu)._fp8_weight == (None, None)
+    with pytest.raises(AssertionError):      # an fp8 weight without its scales
+        T.qkv_rope_forward(d["x"].to(gpu), w8, d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu))
+    with pytest.raises(NotImplementedError): # prefill sizes keep the bf16 weight
+        T.qkv_rope_forward(d["x"].to(gpu), w8, d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), mode="prefill",
+                           weight_scale=ws)
+    with pytest.raises(AssertionError):
+        T.qkv_decode_forward(d["x"].view(8, 1, 2880).to(gpu), w8, d["b"].to(gpu), 4096, 512)
+
+
 def test_norm_qkv_composed_when_not_fusable_and_cache_form(gpu, yarn):
     """norm_scale on shapes the decode kernel does not fuse (prefill rows, other hidden sizes) runs rmsnorm first;
     the cache-writing decode call takes it too."""
@@ -415,7 +468,7 @@ def test_reference_signatures_decode_with_cache(gpu):
     close(qf.reshape(300, 4096), qr)
     close(kf.reshape(300, 512), kr)
     close(vf.reshape(300, 512), vr)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(AssertionError):      # a scale without an fp8 weight
         T.qkv_rope_cache_decode_forward(t, qkv.weight, qkv.bias, rope.sin, rope.cos, rope.max_context_length, cache_k, cache_v,
                                         offset, 64, 8, 64, weight_scale=torch.ones(5120, device=gpu))
     with pytest.raises(AssertionError):

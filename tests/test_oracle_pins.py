@@ -230,3 +230,32 @@ def test_eager_twins_within_tolerance_of_upcast_oracle():
     qr, kr, vr = O.qkv_rope_ref(d["x"], d["w"], d["b"], d["positions"])
     torch.testing.assert_close(q.float(), qr, rtol=5e-2, atol=5e-2)
     torch.testing.assert_close(v.float(), vr, rtol=1.6e-2, atol=1e-2)
+
+
+def test_fp8_rows_quantisation_pins():
+    """e4m3fn decode against the OCP bit formula for all 256 codes; the row maximum lands on +-448; the round trip
+    stays within half a step of the format (3 mantissa bits: relative 2^-4 for normals)."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    dec = codes.view(torch.float8_e4m3fn).to(torch.float32)
+    for c in range(256):
+        s, e, m = c >> 7, (c >> 3) & 15, c & 7
+        if e == 15 and m == 7:
+            assert math.isnan(dec[c].item())
+            continue
+        val = (m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+        assert dec[c].item() == (-val if s else val), c
+    g = torch.Generator().manual_seed(5)
+    w = (0.02 * torch.randn(64, 256, generator=g)).bfloat16()
+    w[3] = 0                                                    # an all-zero row must not divide by zero
+    w8, scale = O.quantize_fp8_rows_ref(w)
+    assert w8.dtype == torch.float8_e4m3fn and scale.dtype == torch.float32 and scale.shape == (64,)
+    amax = w.float().abs().max(dim=1).values
+    torch.testing.assert_close(scale[amax > 0], (amax / 448.0)[amax > 0], rtol=1e-6, atol=0)
+    assert scale[3].item() == pytest.approx(1e-12 / 448.0, rel=1e-5)
+    assert torch.all(w8.float().abs().max(dim=1).values[amax > 0] == 448.0)
+    deq = O.dequant_fp8_ref(w8, scale)
+    assert torch.all(deq[3] == 0)
+    err = (deq - w.float()).abs()
+    # half a step: normals 2^-4 relative; below 2^-6 (in units of scale) the step is fixed at 2^-9
+    bound = torch.maximum(w.float().abs() * 2.0 ** -4, scale[:, None] * 2.0 ** -10) * 1.0001
+    assert torch.all(err <= bound)

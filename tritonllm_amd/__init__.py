@@ -9,6 +9,7 @@ from .ops import (
     qkv_decode_forward,
     qkv_rope_cache_decode_forward,
     qkv_rope_forward,
+    quantize_fp8_rows,
     rmsnorm_forward,
     rope_forward,
     swiglu,
@@ -18,5 +19,5 @@ from .yarn import YarnParams, gpt_oss_yarn
 __all__ = [
     "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
     "embedding_forward", "linear_qkv_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
-    "qkv_rope_forward", "rmsnorm_forward", "rope_forward", "swiglu",
+    "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu",
 ]

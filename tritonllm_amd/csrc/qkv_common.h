@@ -21,6 +21,7 @@ struct QkvArgs {
   int has_rope;
   const void* norm_scale;     // fused RMSNorm prologue (decode fast path only): scale [hidden], fp32 or bf16
   float norm_eps;
+  const float* w_scale;        // fp8 weight (decode fast path only): one fp32 scale per output row
 };
 
 // KV-cache slot the new token goes to (0 when the outputs are plain tensors). A global load: call it early.

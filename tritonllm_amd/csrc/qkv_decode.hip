@@ -54,6 +54,7 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
   a->has_rope = rope != nullptr;
   a->norm_scale = nullptr;
   a->norm_eps = 0.f;
+  a->w_scale = nullptr;
   return TLLM_OK;
 }
 
@@ -204,13 +205,19 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 // are summed by 16 x XR threads, one (pair, activation row) each, which also add the bias, rotate
 // with cos/sin they computed while the loads were in flight, round once and store.
 // NORM: 0 = x is used as it is; 1 / 2 = x is first RMS-normalised with an fp32 / bf16 scale (fused prologue).
-template <int XR, int CH, int NORM>
+// W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row, W[n][k] = fp8[n][k] * w_scale[n]
+// (triton_kernels.py:261-268, 927-940, 963-965). Half the bytes to stream; the values are widened to bf16 (exact)
+// on their way into the LDS patch, so the MFMAs and the fp32 accumulation are those of the bf16 kernel, and the
+// row scale multiplies the finished sum.
+template <int XR, int CH, int NORM, bool W8>
 __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   constexpr int NW = 15, SPW = 6, NCH = SPW / CH, PAIRS = 10;
-  constexpr int KV = 360;                 // 16-byte vectors per row (hidden 2880)
+  constexpr int KV = 360;                 // 16-byte vectors per activation row (hidden 2880)
+  constexpr int KVW = W8 ? 180 : 360;     // ... per weight row
   constexpr int WROW = CH * 64 + 16;      // padded patch row, bytes
-  constexpr int CPR = CH * 4;             // 16-byte chunks per row per patch
-  constexpr int WL = (2 * PAIRS * CPR + 63) / 64;   // weight load instructions per patch
+  constexpr int CPR = CH * 4;             // 16-byte chunks per row per patch (bf16)
+  constexpr int CPRW = W8 ? CPR / 2 : CPR;            // ... of the weight as it lies in memory
+  constexpr int WL = (2 * PAIRS * CPRW + 63) / 64;    // weight load instructions per patch
   constexpr int XL = (XR * CPR + 63) / 64;          // activation load instructions per patch
   constexpr int PATCH = (32 + XR) * WROW;
   constexpr int RED = XR * 32;            // floats per wavefront in the reduction buffer
@@ -252,10 +259,15 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
     b_hi = bias_ptr[ehead * 64 + 32 + ed];
   }
   const float freq = fr.v[ed];
+  float ws_lo = 1.f, ws_hi = 1.f;
+  if constexpr (W8) {
+    ws_lo = a.w_scale[ehead * 64 + ed];
+    ws_hi = a.w_scale[ehead * 64 + 32 + ed];
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   const bf16x8* xg = reinterpret_cast<const bf16x8*>(a.x) + row0 * KV + wave * (SPW * 4);
-  const bf16x8* wg = reinterpret_cast<const bf16x8*>(a.W) + wave * (SPW * 4);
+  const bf16x8* wg = reinterpret_cast<const bf16x8*>(a.W) + wave * (W8 ? SPW * 2 : SPW * 4);   // 16-byte units either way
   bf16x8 xr[NCH * XL], wr[NCH * WL];
   // The norm scale of this wavefront's K slice (SPW * 32 values): one load per wavefront, parked in LDS later.
   f32x4 sc32 = {};
@@ -283,13 +295,13 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   if constexpr (NORM != 0) load_x();
   auto load_w = [&](int idx) {               // weight load idx: patch j = idx / WL, chunk slot i = idx % WL
     const int j = idx / WL, i = idx % WL;
-    int e = i * 64 + lane;                    // patch chunk e -> weight row e / CPR: the ten low rows, then their partners
-    e = e < 2 * PAIRS * CPR ? e : 2 * PAIRS * CPR - 1;
-    const int r = e / CPR, kc = e - r * CPR;
+    int e = i * 64 + lane;                    // patch chunk e -> weight row e / CPRW: the ten low rows, then their partners
+    e = e < 2 * PAIRS * CPRW ? e : 2 * PAIRS * CPRW - 1;
+    const int r = e / CPRW, kc = e - r * CPRW;
     int gp = pair0 + (r < PAIRS ? r : r - PAIRS);
     gp = gp < total_pairs ? gp : total_pairs - 1;
     const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + (r < PAIRS ? 0u : 32u);
-    wr[idx] = __builtin_nontemporal_load(wg + wrow * static_cast<unsigned>(KV) + j * CPR + kc);
+    wr[idx] = __builtin_nontemporal_load(wg + wrow * static_cast<unsigned>(KVW) + j * CPRW + kc);
   };
   // A CU holds a bounded number of loads in flight and a wavefront stalls when it issues one beyond that. With
   // the fused norm every wavefront must see its activations, and meet the others at a barrier, before any MFMA
@@ -437,9 +449,30 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 #pragma unroll
     for (int i = 0; i < WL; ++i) {
       const int e = i * 64 + lane;
-      const int r = e / CPR, kc = e - r * CPR;
+      const int r = e / CPRW, kc = e - r * CPRW;
       const int trow = r < PAIRS ? r : r - PAIRS + 16;
-      if (e < 2 * PAIRS * CPR) *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 16) = wr[j * WL + i];
+      if constexpr (W8) {
+        // sixteen fp8 -> sixteen bf16 (exact: e4m3 fits), two chunks of the patch row
+        typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
+        typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+        const i32x4 raw = __builtin_bit_cast(i32x4, wr[j * WL + i]);
+        bf16x8 w0, w1;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[d], false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[d], true);
+          bf16x8& dst = d < 2 ? w0 : w1;
+          dst[4 * (d & 1) + 0] = static_cast<bf16>(p0[0]);
+          dst[4 * (d & 1) + 1] = static_cast<bf16>(p0[1]);
+          dst[4 * (d & 1) + 2] = static_cast<bf16>(p1[0]);
+          dst[4 * (d & 1) + 3] = static_cast<bf16>(p1[1]);
+        }
+        if (e < 2 * PAIRS * CPRW) {
+          *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 32) = w0;
+          *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 32 + 16) = w1;
+        }
+      } else {
+        if (e < 2 * PAIRS * CPRW) *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 16) = wr[j * WL + i];
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -471,6 +504,10 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
     lo += red[w * RED + es * XR + en];
     hi += red[w * RED + (16 + es) * XR + en];
   }
+  if constexpr (W8) {
+    lo *= ws_lo;
+    hi *= ws_hi;
+  }
   if (a.bias) {
     lo += __uint_as_float(static_cast<unsigned>(b_lo) << 16);
     hi += __uint_as_float(static_cast<unsigned>(b_hi) << 16);
@@ -489,45 +526,80 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 
 using namespace tllm;
 
-static void launch_cu(int xr, int norm, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
-#define TLLM_CU(XR, CH)                                                                                      \
-  do {                                                                                                       \
-    if (norm == 0) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, 0>), grid, dim3(960), 0, st, a, ra, fr);      \
-    else if (norm == 1) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, 1>), grid, dim3(960), 0, st, a, ra, fr); \
-    else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, 2>), grid, dim3(960), 0, st, a, ra, fr);                \
+static void launch_cu(int xr, int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+#define TLLM_CU1(XR, CH, NORM)                                                                                  \
+  do {                                                                                                          \
+    if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, true>), grid, dim3(960), 0, st, a, ra, fr);  \
+    else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, false>), grid, dim3(960), 0, st, a, ra, fr);    \
+  } while (0)
+#define TLLM_CU(XR, CH)                \
+  do {                                 \
+    if (norm == 0) TLLM_CU1(XR, CH, 0); \
+    else if (norm == 1) TLLM_CU1(XR, CH, 1); \
+    else TLLM_CU1(XR, CH, 2);          \
   } while (0)
   if (xr == 8) TLLM_CU(8, 3);
   else if (xr == 16) TLLM_CU(16, 3);
   else TLLM_CU(32, 2);
 #undef TLLM_CU
+#undef TLLM_CU1
+}
+
+// Shared tail of the hidden-2880 decode entry points: row-count -> kernel variant and grid.
+static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, int norm, bool w8, int64_t rows,
+                              int heads, hipStream_t st) {
+  TLLM_REQUIRE(static_cast<int64_t>(heads) * 64 * 2880 < (1ll << 31), TLLM_E_SHAPE, "%s: weight too large", what);
+  const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
+  const int64_t chunks = (rows + xr - 1) / xr;
+  TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
+  launch_cu(xr, norm, w8, dim3((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks), st, a, ra, fr);
+  return check_launch(what);
+}
+
+// Common body of the two entry points that exist for the gpt-oss shape only (fused norm and/or fp8 weight).
+static int decode_2880_entry(const char* what, const void* x, const void* norm_scale, int scale_is_bf16, float eps, const void* W,
+                             const float* w_scale, bool w8, const void* b, void* q, void* k, void* v, int64_t q_row_stride,
+                             int64_t k_row_stride, int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows, int64_t hidden,
+                             int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope, void* stream) {
+  QkvArgs a;
+  RopeArgs ra;
+  YarnFreqs fr;
+  int rc = qkv_validate(what, x, W, q, k, v, q_row_stride, k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads,
+                        n_kv_heads, head_dim, rope, &a, &ra, &fr);
+  if (rc != TLLM_OK) return rc;
+  TLLM_REQUIRE(hidden == 2880 && head_dim == 64, TLLM_E_SHAPE,
+               "%s: this kernel exists for hidden 2880 / head_dim 64 only (got %lld / %d)", what, (long long)hidden, head_dim);
+  TLLM_REQUIRE(aligned16(x) && aligned16(W) && aligned16(norm_scale), TLLM_E_ALIGN, "%s: x, W and norm_scale must be 16-byte aligned", what);
+  TLLM_REQUIRE(!w8 || (w_scale != nullptr && reinterpret_cast<uintptr_t>(w_scale) % 4 == 0), TLLM_E_ARG,
+               "%s: w_scale must be a 4-byte aligned device pointer", what);
+  a.bias = (const bf16*)b;
+  a.norm_scale = norm_scale;
+  a.norm_eps = eps;
+  a.w_scale = w_scale;
+  if (rows == 0) return TLLM_OK;
+  return launch_decode_2880(what, a, ra, fr, norm_scale ? (scale_is_bf16 ? 2 : 1) : 0, w8, rows, n_q_heads + 2 * n_kv_heads,
+                            static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps, const void* W,
                                               const void* b, void* q, void* k, void* v, int64_t q_row_stride, int64_t k_row_stride,
                                               int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows, int64_t hidden, int n_q_heads,
                                               int n_kv_heads, int head_dim, const TllmRope* rope, void* stream) {
-  QkvArgs a;
-  RopeArgs ra;
-  YarnFreqs fr;
-  int rc = qkv_validate("norm_qkv_rope_decode", x, W, q, k, v, q_row_stride, k_row_stride, v_row_stride, kv_slot_stride, rows, hidden,
-                        n_q_heads, n_kv_heads, head_dim, rope, &a, &ra, &fr);
-  if (rc != TLLM_OK) return rc;
-  TLLM_REQUIRE(norm_scale != nullptr, TLLM_E_ARG, "norm_qkv_rope_decode: norm_scale is NULL");
-  TLLM_REQUIRE(hidden == 2880 && head_dim == 64, TLLM_E_SHAPE,
-               "norm_qkv_rope_decode: the fused kernel exists for hidden 2880 / head_dim 64 only (got %lld / %d); "
-               "call tllm_rmsnorm_bf16 and tllm_qkv_rope_decode_bf16", (long long)hidden, head_dim);
-  TLLM_REQUIRE(aligned16(x) && aligned16(W) && aligned16(norm_scale), TLLM_E_ALIGN, "norm_qkv_rope_decode: x, W and norm_scale must be 16-byte aligned");
-  a.bias = (const bf16*)b;
-  a.norm_scale = norm_scale;
-  a.norm_eps = eps;
-  if (rows == 0) return TLLM_OK;
-  const int heads = n_q_heads + 2 * n_kv_heads;
-  TLLM_REQUIRE(static_cast<int64_t>(heads) * 64 * hidden < (1ll << 31), TLLM_E_SHAPE, "norm_qkv_rope_decode: weight too large");
-  const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
-  const int64_t chunks = (rows + xr - 1) / xr;
-  TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "norm_qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
-  launch_cu(xr, scale_is_bf16 ? 2 : 1, dim3((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks), static_cast<hipStream_t>(stream), a, ra, fr);
-  return check_launch("norm_qkv_rope_decode");
+  if (norm_scale == nullptr) {
+    set_error("norm_qkv_rope_decode: norm_scale is NULL");
+    return TLLM_E_ARG;
+  }
+  return decode_2880_entry("norm_qkv_rope_decode", x, norm_scale, scale_is_bf16, eps, W, nullptr, false, b, q, k, v, q_row_stride,
+                           k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads, n_kv_heads, head_dim, rope, stream);
+}
+
+extern "C" int tllm_qkv_rope_decode_w8_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps, const void* W8,
+                                            const float* w_scale, const void* b, void* q, void* k, void* v, int64_t q_row_stride,
+                                            int64_t k_row_stride, int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows,
+                                            int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope,
+                                            void* stream) {
+  return decode_2880_entry("qkv_rope_decode_w8", x, norm_scale, scale_is_bf16, eps, W8, w_scale, true, b, q, k, v, q_row_stride,
+                           k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads, n_kv_heads, head_dim, rope, stream);
 }
 
 extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const void* b, void* q, void* k, void* v, int64_t q_row_stride,
@@ -547,12 +619,7 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
   const bool mfma_ok = head_dim == 64 && hidden % 32 == 0 && aligned16(x) && aligned16(W);
   if (mfma_ok && hidden == 2880 && aligned16(b) && static_cast<int64_t>(heads) * 64 * hidden < (1ll << 31)) {
     // 32-bit element offsets inside W and x are enough here; outputs are written element-wise, any alignment
-    const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
-    const int64_t chunks = (rows + xr - 1) / xr;
-    TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
-    dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
-    launch_cu(xr, 0, grid, st, a, ra, fr);
-    return check_launch("qkv_rope_decode");
+    return launch_decode_2880("qkv_rope_decode", a, ra, fr, 0, false, rows, heads, st);
   }
   const bool out4 = (reinterpret_cast<uintptr_t>(q) % 4 == 0) && (reinterpret_cast<uintptr_t>(k) % 4 == 0) &&
                     (reinterpret_cast<uintptr_t>(v) % 4 == 0) && q_row_stride % 2 == 0 && k_row_stride % 2 == 0 &&

@@ -9,6 +9,7 @@ tensors on the GPU, and the HIP library must be present.
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import torch
 
@@ -33,6 +34,19 @@ class QKV(torch.nn.Module):
         super().__init__()
         self.weight = torch.nn.Parameter(torch.empty((qkv_dim, hidden_size), device=device, dtype=torch.bfloat16))
         self.bias = torch.nn.Parameter(torch.empty((qkv_dim), device=device, dtype=torch.bfloat16))
+        # model.py:130-134: ATTN_FP8 switches the decode path to a per-row quantised fp8 copy of the weight
+        self._use_fp8 = os.getenv("ATTN_FP8", "0").strip().lower() not in {"0", "false", "no", "off"}
+        self._weight_fp8: torch.Tensor | None = None
+        self._weight_scale: torch.Tensor | None = None
+
+    @property
+    def _fp8_weight(self):
+        """``(weight_fp8, weight_scale)``, quantised on first use (model.py:160-167); ``(None, None)`` unless ATTN_FP8 is set."""
+        if not self._use_fp8:
+            return None, None
+        if self._weight_fp8 is None:
+            self._weight_fp8, self._weight_scale = ops.quantize_fp8_rows(self.weight.detach())
+        return self._weight_fp8, self._weight_scale
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """``F.linear(x, weight, bias)``: one dense ``[..., qkv_dim]`` tensor."""

@@ -191,33 +191,62 @@ def _norm_fusable(kind: str, rows: int, hidden: int, hd: int) -> bool:
     return kind == "decode" and hidden == 2880 and hd == 64 and rows <= 16
 
 
-def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_stride, n_q, n_kv, hd, desc, norm=None):
+def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_stride, n_q, n_kv, hd, desc, norm=None, w_scale=None):
     """``norm = (scale, eps)``: x2 is the raw hidden state and is RMS-normalised first -- inside
-    the decode kernel where it can, by a preceding rmsnorm launch otherwise."""
+    the decode kernel where it can, by a preceding rmsnorm launch otherwise.
+    ``w_scale``: ``weight`` is fp8 e4m3 with one fp32 scale per output row (decode kernel, gpt-oss shape only)."""
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    rope = C.byref(desc) if desc is not None else None
     if norm is not None:
         scale, eps = norm
         assert scale.dtype in (torch.float32, _BF16) and scale.shape == (x2.shape[1],)
         if not scale.is_contiguous():
             scale = scale.contiguous()
-        if _norm_fusable(kind, x2.shape[0], x2.shape[1], hd):
+        if w_scale is None and _norm_fusable(kind, x2.shape[0], x2.shape[1], hd):
             rc = lib().tllm_norm_qkv_rope_decode_bf16(
-                x2.data_ptr(), scale.data_ptr(), int(scale.dtype == _BF16), float(eps), weight.data_ptr(),
-                bias.data_ptr() if bias is not None else None, q.data_ptr() if q is not None else None,
-                k.data_ptr() if k is not None else None, v.data_ptr() if v is not None else None, q_rs, k_rs, v_rs,
-                kv_slot_stride, x2.shape[0], x2.shape[1], n_q, n_kv, hd, C.byref(desc) if desc is not None else None, _stream())
+                x2.data_ptr(), scale.data_ptr(), int(scale.dtype == _BF16), float(eps), weight.data_ptr(), ptr(bias), ptr(q), ptr(k),
+                ptr(v), q_rs, k_rs, v_rs, kv_slot_stride, x2.shape[0], x2.shape[1], n_q, n_kv, hd, rope, _stream())
             check(rc, "norm_qkv_rope_decode")
             return
-        x2 = rmsnorm_forward(x2, scale, eps)
+        if w_scale is None or not _norm_fusable(kind, x2.shape[0], x2.shape[1], hd):
+            x2 = rmsnorm_forward(x2, scale, eps)
+            norm = None
+    if w_scale is not None:
+        if not (kind == "decode" and x2.shape[1] == 2880 and hd == 64):
+            raise NotImplementedError("fp8 weights with per-row scales: the HIP path has the decode kernel for hidden 2880 / head_dim 64 only")
+        scale, eps = norm if norm is not None else (None, 0.0)
+        rc = lib().tllm_qkv_rope_decode_w8_bf16(
+            x2.data_ptr(), ptr(scale), int(scale is not None and scale.dtype == _BF16), float(eps), weight.data_ptr(),
+            w_scale.data_ptr(), ptr(bias), ptr(q), ptr(k), ptr(v), q_rs, k_rs, v_rs, kv_slot_stride, x2.shape[0], x2.shape[1], n_q,
+            n_kv, hd, rope, _stream())
+        check(rc, "qkv_rope_decode_w8")
+        return
     fn = lib().tllm_qkv_rope_decode_bf16 if kind == "decode" else lib().tllm_qkv_rope_prefill_bf16
-    rc = fn(x2.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
-            q.data_ptr() if q is not None else None, k.data_ptr() if k is not None else None,
-            v.data_ptr() if v is not None else None, q_rs, k_rs, v_rs, kv_slot_stride, x2.shape[0], x2.shape[1], n_q, n_kv, hd,
-            C.byref(desc) if desc is not None else None, _stream())
+    rc = fn(x2.data_ptr(), weight.data_ptr(), ptr(bias), ptr(q), ptr(k), ptr(v), q_rs, k_rs, v_rs, kv_slot_stride, x2.shape[0],
+            x2.shape[1], n_q, n_kv, hd, rope, _stream())
     check(rc, f"qkv_rope_{kind}")
 
 
+_FP8 = torch.float8_e4m3fn
+
+
+def quantize_fp8_rows(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-row fp8 e4m3 quantisation of a bf16 weight, as ``_quantize_unembed_fp8`` (triton_kernels.py:261-268):
+    returns ``(weight_fp8 [n, k] float8_e4m3fn, scale [n] float32)`` on the weight's device."""
+    w = weight.to(torch.float32)
+    amax = w.abs().max(dim=1, keepdim=True).values.clamp(min=1e-12)
+    scale = (amax / torch.finfo(_FP8).max).squeeze(1).to(torch.float32)
+    return (w / scale[:, None].clamp(min=1e-12)).to(_FP8), scale
+
+
+def _prep_weight_scale(weight, weight_scale):
+    assert weight.dtype == _FP8, "weight_scale goes with a float8_e4m3fn weight"
+    assert weight_scale.dtype == torch.float32 and weight_scale.shape == (weight.shape[0],)
+    return weight_scale if weight_scale.is_contiguous() else weight_scale.contiguous()
+
+
 def _prep_linear(hidden2, weight, bias):
-    assert hidden2.dtype == _BF16 and weight.dtype == _BF16 and (bias is None or bias.dtype == _BF16)
+    assert hidden2.dtype == _BF16 and weight.dtype in (_BF16, _FP8) and (bias is None or bias.dtype == _BF16)
     if not hidden2.is_contiguous():
         hidden2 = hidden2.contiguous()
     if not weight.is_contiguous():
@@ -232,18 +261,20 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
                      sin: torch.Tensor | None = None, positions: torch.Tensor | None = None, offset: torch.Tensor | None = None,
                      tokens_per_batch: int | None = None, max_context_length: int = 131072, rotate: bool = True,
                      mode: str = "auto", out: tuple | None = None, norm_scale: torch.Tensor | None = None,
-                     norm_eps: float = 1e-5):
+                     norm_eps: float = 1e-5, weight_scale: torch.Tensor | None = None):
     """RMS-normed activations ``x [rows, hidden]`` -> ``(q [rows, Hq*D], k [rows, Hkv*D], v [rows, Hkv*D])``.
 
     With ``norm_scale`` given, ``x`` is the raw hidden state and the call also performs the
     ``RMSNorm(x)`` of model.py:476 (inside the same kernel for decode-sized gpt-oss shapes).
+    With ``weight_scale`` the weight is float8_e4m3fn with per-row scales (see ``quantize_fp8_rows``).
 
     One fused kernel: projection, bias, rotary on q/k (fp32 accumulator, one rounding),
     outputs written to three dense tensors. ``mode``: "decode" (weight streaming),
     "prefill" (MFMA GEMM) or "auto" (by row count). No reference twin as a single call:
     it is F.linear + split + contiguous + rope_forward of model.py:506-522 in one launch."""
-    _on_gpu(x, weight, bias, positions, offset, cos, sin, norm_scale)
+    _on_gpu(x, weight, bias, positions, offset, cos, sin, norm_scale, weight_scale)
     assert x.ndim == 2
+    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
     rows, hidden = x.shape
     total_out, hidden_w = weight.shape
     assert hidden == hidden_w
@@ -268,7 +299,8 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
         mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
     assert mode in ("decode", "prefill")
     _launch_qkv(mode, x, weight, bias, q, k, v, q.stride(0), k.stride(0), v.stride(0), 0, num_q_heads, num_kv_heads, head_dim, desc,
-                norm=None if norm_scale is None else (norm_scale, norm_eps))
+                norm=None if norm_scale is None else (norm_scale, norm_eps),
+                w_scale=None if weight_scale is None else _prep_weight_scale(weight, weight_scale))
     return q, k, v
 
 
@@ -290,6 +322,7 @@ def qkv_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias: torch.T
     assert hidden_size == hidden_size_weight
     assert bias.shape == (total_out,)
     assert total_out == q_dim + 2 * kv_dim
+    assert weight.dtype == _BF16
     x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
     hd = _split_head_dim(q_dim, kv_dim)
     q = scratch_pool.get((batch, q_dim), hidden.dtype, hidden.device)
@@ -308,9 +341,8 @@ def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_le
     (a borrowed pool buffer). ``offset`` is an int64 device tensor of shape (1,) and is read
     on the device, so the call can be replayed from a HIP graph. With ``norm_scale`` the
     block's input RMSNorm (model.py:476) runs inside the same kernel on the raw ``hidden``."""
-    _on_gpu(hidden, weight, bias, cache_k, cache_v, offset, positions, norm_scale)
-    if weight_scale is not None:
-        raise NotImplementedError("fp8 weights with per-row scales are not implemented in the HIP path")
+    _on_gpu(hidden, weight, bias, cache_k, cache_v, offset, positions, norm_scale, weight_scale)
+    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
     batch, num_tokens, hidden_size = hidden.shape
     total_out, hidden_size_weight = weight.shape
     assert num_tokens == 1
@@ -331,7 +363,8 @@ def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_le
     desc = _rope_desc(cos, sin, yarn, positions, offset, 1, max_context_length, keep)
     _launch_qkv("decode", x2, weight, bias, q, cache_k, cache_v, num_q_heads * head_dim, cache_k.stride(0), cache_v.stride(0),
                 cache_k.stride(1), num_q_heads, num_kv_heads, head_dim, desc,
-                norm=None if norm_scale is None else (norm_scale, norm_eps))
+                norm=None if norm_scale is None else (norm_scale, norm_eps),
+                w_scale=None if weight_scale is None else _prep_weight_scale(weight, weight_scale))
     return q.reshape(batch, 1, num_q_heads * head_dim)
 
 
@@ -340,7 +373,7 @@ def linear_qkv_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     through the MFMA kernel (or the streaming kernel for few rows), writing one dense output."""
     _on_gpu(x, weight, bias)
     total_out, hidden = weight.shape
-    assert x.shape[-1] == hidden
+    assert x.shape[-1] == hidden and weight.dtype == _BF16
     x2, weight, bias = _prep_linear(x.reshape(-1, hidden), weight, bias)
     rows = x2.shape[0]
     hd = 64 if total_out % 64 == 0 else 2
