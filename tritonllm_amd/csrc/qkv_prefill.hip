@@ -22,11 +22,15 @@
 //   * an L2 miss still costs more than a slice of MFMAs and LDS has no room for a third stage, so
 //     three slices ahead every workgroup touches (one dword per line) its share of the lines its
 //     XCD's tiles are going to need, which pulls them into that XCD's L2 in time;
-//   * measured with per-slice cycle stamps: the waits for loads and at the barrier are ~10 % of a slice; the
-//     rest is the MFMA / LDS phase itself at ~1.5x the 1280 MFMA cycles. LDS is the binding resource: per
-//     slice 112 KB of fragment reads plus 57 KB of incoming tile data against 128 B/clk is 1320 cycles at
-//     best, i.e. this tiling cannot run the MFMAs much above two thirds busy, and the clock under this
-//     load is ~1.85-1.9 GHz rather than the 2.4 GHz of the published peak.
+//   * measured with cycle stamps per k16 step (one build with the stamps compiled in), per slice of 64:
+//     the two steps that only multiply take ~375 cycles each (320 of MFMAs); the two that also carry load
+//     instructions take 590 and 715 -- every load instruction holds the wavefront 35-50 cycles, because the
+//     CU's one address unit serves the four wavefronts' 1 KB loads at ~16 cycles apiece and they all come at
+//     once; waits for the look-ahead loads and at the barrier add ~180. 2240 cycles for 1280 of MFMAs, at a
+//     shader clock of 1.83-1.92 GHz under this load (the published peak assumes 2.4 GHz).
+//     LDS is not the limit (a microbenchmark reads > 400 B/clk/CU with 128-bit reads). Tried and measured, no
+//     better: four extra wavefronts that only load (the multipliers then wait at the barrier for data that is
+//     requested in one burst, 71-75 us), and the same with K slices of 32 in a four-stage ring (77 us).
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
