@@ -51,6 +51,9 @@ def algorithmic_bytes():
         "norm_qkv": lambda r: w + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
         # fp8 weight: one byte per element + one fp32 scale per output row
         "qkv_w8": lambda r: w // 2 + QKV_DIM * 4 + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
+        # attention out-projection [2880, 4096] + bias + residual: weight, bias, x row, residual row in, output row out
+        "out": lambda r: HIDDEN * 4096 * 2 + HIDDEN * 2 + r * (4096 * 2 + 2 * HIDDEN * 2),
+        "out_w8": lambda r: HIDDEN * 4096 + HIDDEN * 4 + HIDDEN * 2 + r * (4096 * 2 + 2 * HIDDEN * 2),
         "norm_qkv_w8": lambda r: w // 2 + QKV_DIM * 4 + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
     }
 
@@ -75,6 +78,17 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
                                           norm_scale=scales[i % N_LAYERS] if fused else None,
                                           weight_scale=wq[i % N_LAYERS][1] if w8 else None)
         flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of[("norm_qkv" if fused else "qkv") + ("_w8" if w8 else "")](n)
+    elif kind in ("out_residual_decode", "out_residual_decode_w8"):
+        w8 = kind.endswith("_w8")
+        ow = [torch.empty(HIDDEN, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
+        if w8:
+            ow = [T.quantize_fp8_rows(w) for w in ow]
+        ob = torch.empty(HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
+        ox = torch.empty(n, 1, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        ores = torch.zeros(n, 1, HIDDEN, dtype=torch.bfloat16, device=dev)
+        fn = (lambda i: T.out_residual_decode_forward(ox, ow[i % N_LAYERS][0], ob, ores, weight_scale=ow[i % N_LAYERS][1])) if w8 else \
+             (lambda i: T.out_residual_decode_forward(ox, ow[i % N_LAYERS], ob, ores))
+        nbytes = bytes_of["out_w8" if w8 else "out"](n)
     elif kind == "rmsnorm":
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         to = torch.empty_like(xp)
@@ -296,6 +310,21 @@ def main() -> int:
                                                                                weight_scale=wq[i % N_LAYERS][1]),
                              bytes_of["norm_qkv_w8"](r), n=240)
         del wq
+        # attention out-projection + bias + residual (decode), bf16 and fp8 weight
+        ow = [torch.empty(HIDDEN, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
+        ow8 = [T.quantize_fp8_rows(w) for w in ow]
+        ob = torch.empty(HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
+        for r in (1, 8, 32):
+            ox = torch.empty(r, 1, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            ores = torch.zeros(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev)
+            bench_kernel(f"out_residual_decode_B{r}", lambda i, ox=ox, ores=ores: T.out_residual_decode_forward(ox, ow[i % N_LAYERS], ob, ores),
+                         bytes_of["out"](r), n=240)
+            if r == 8:
+                bench_kernel("out_residual_decode_w8_B8",
+                             lambda i, ox=ox, ores=ores: T.out_residual_decode_forward(ox, ow8[i % N_LAYERS][0], ob, ores,
+                                                                                       weight_scale=ow8[i % N_LAYERS][1]),
+                             bytes_of["out_w8"](r), n=240)
+        del ow, ow8
         # prefill sizes
         for tt in (2048, 8192):
             xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)

@@ -174,6 +174,19 @@ int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const void* b,
                                int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
                                const TllmRope* rope, void* stream);
 
+/* Decode-size attention out-projection with bias and residual,
+ *   out[r, n] = sum_k x[r, k] * W[n, k] + bias[n] + residual[r, n]        (fp32 accumulate, one RNE to bf16),
+ * replaces out_residual_decode_forward(hidden, weight, bias, residual, weight_scale=None),
+ * triton_kernels.py:1470-1517 (its split-K kernel :1340-1416 and reduce kernel :1419-1467, in one launch
+ * and without the partial-sum buffer). x [rows, in_dim] bf16 dense; W [out_dim, in_dim] bf16 dense, or fp8
+ * e4m3 bytes when w_scale (one fp32 per output row) is not NULL; bias [out_dim] or NULL; residual
+ * [rows, out_dim] with res_row_stride elements between rows, or NULL; out likewise and MAY BE the residual
+ * buffer (the reference writes its result into it). The weight-streaming kernel serves in_dim == 4096
+ * with out_dim a multiple of 12 (gpt-oss: 2880 x 4096); other shapes take a plain kernel. */
+int tllm_out_residual_decode_bf16(const void* x, const void* W, const float* w_scale, const void* bias,
+                                  const void* residual, void* out, int64_t res_row_stride, int64_t out_row_stride,
+                                  int64_t rows, int64_t in_dim, int64_t out_dim, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,7 @@ force and special cases -- in ``tests/test_oracle_pins.py``:
     qkv_rope_ref                      composition of the above, v slice un-rotated
     swiglu_ref                        float64 brute force, edge grid, l=-1 => 0,
                                       interleaved == chunked under permutation
+    out_residual_ref                  linear_ref + an fp32 add; float64 brute force
     quantize_fp8_rows_ref /           all 256 e4m3 codes against the OCP bit formula, row maxima map to
     dequant_fp8_ref                   +-448, round-trip error within half a step of the format
 
@@ -135,6 +136,15 @@ def linear_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None)
     out = x.to(torch.float32) @ weight.to(torch.float32).t()
     if bias is not None:
         out = out + bias.to(torch.float32)
+    return out
+
+
+def out_residual_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, residual: torch.Tensor | None) -> torch.Tensor:
+    """triton_kernels.py:1470-1517 (kernel :1340-1416, reduce :1419-1467): ``x @ W.T + bias + residual`` with every
+    operand upcast to fp32 (pass the dequantised weight for the fp8 form). Returns fp32."""
+    out = linear_ref(x, weight, bias)
+    if residual is not None:
+        out = out + residual.to(torch.float32)
     return out
 
 

@@ -511,3 +511,56 @@ def test_graph_replay_reads_positions_from_device(gpu, yarn):
         qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], torch.full((8,), p, dtype=torch.int64))
         close(outs["q"], qr, rtol=3e-2, atol=2e-2)   # t_ref is the oracle's rounding of the norm, the GPU's may differ by one bf16 ulp
         close(outs["k"], kr, rtol=3e-2, atol=2e-2)
+
+
+# ----------------------------------------------------------------------------------- out-projection (decode)
+def _out_inputs(rows, seed, in_dim=4096, out_dim=2880):
+    g = torch.Generator().manual_seed(seed)
+    return dict(x=torch.randn(rows, in_dim, generator=g).bfloat16(), w=(0.02 * torch.randn(out_dim, in_dim, generator=g)).bfloat16(),
+                b=(0.02 * torch.randn(out_dim, generator=g)).bfloat16(), r=torch.randn(rows, out_dim, generator=g).bfloat16())
+
+
+@pytest.mark.parametrize("rows", [1, 8, 11, 16, 17, 32, 45])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_out_residual_decode_parity(gpu, rows, fp8):
+    d = _out_inputs(rows, 600 + rows)
+    res = d["r"].view(rows, 1, 2880).to(gpu)
+    res_before = res.clone()
+    if fp8:
+        w8, ws = T.quantize_fp8_rows(d["w"].to(gpu))
+        out = T.out_residual_decode_forward(d["x"].view(rows, 1, 4096).to(gpu), w8, d["b"].to(gpu), res, weight_scale=ws)
+        want = O.out_residual_ref(d["x"], O.dequant_fp8_ref(w8.cpu(), ws.cpu()), d["b"], d["r"])
+    else:
+        out = T.out_residual_decode_forward(d["x"].view(rows, 1, 4096).to(gpu), d["w"].to(gpu), d["b"].to(gpu), res)
+        want = O.out_residual_ref(d["x"], d["w"], d["b"], d["r"])
+    assert out.shape == (rows, 1, 2880) and out.data_ptr() == res.data_ptr()          # written into the residual, as the reference does
+    assert not torch.equal(res, res_before)
+    close(out.view(rows, 2880), want)
+
+
+def test_out_residual_other_shapes_module_and_errors(gpu, monkeypatch):
+    # a shape the streaming kernel does not serve (in_dim != 4096): the plain kernel, bf16 and fp8
+    d = _out_inputs(5, 61, in_dim=320, out_dim=100)
+    res = d["r"].view(5, 1, 100).to(gpu)
+    out = T.out_residual_decode_forward(d["x"].view(5, 1, 320).to(gpu), d["w"].to(gpu), d["b"].to(gpu), res)
+    close(out.view(5, 100), O.out_residual_ref(d["x"], d["w"], d["b"], d["r"]))
+    w8, ws = T.quantize_fp8_rows(d["w"].to(gpu))
+    out = T.out_residual_decode_forward(d["x"].view(5, 1, 320).to(gpu), w8, d["b"].to(gpu), d["r"].view(5, 1, 100).to(gpu), weight_scale=ws)
+    close(out.view(5, 100), O.out_residual_ref(d["x"], O.dequant_fp8_ref(w8.cpu(), ws.cpu()), d["b"], d["r"]))
+    # the module, plain and under ATTN_FP8 (model.py:170-216)
+    d = _out_inputs(8, 62)
+    for env in ("0", "1"):
+        monkeypatch.setenv("ATTN_FP8", env)
+        mod = T.OUT(4096, 2880, device=gpu)
+        with torch.no_grad():
+            mod.weight.copy_(d["w"])
+            mod.bias.copy_(d["b"])
+        y = mod.decode_residual(d["x"].view(8, 1, 4096).to(gpu), d["r"].view(8, 1, 2880).to(gpu))
+        w_used = O.dequant_fp8_ref(*[t.cpu() for t in mod._fp8_weight]) if env == "1" else d["w"]
+        close(y.view(8, 2880), O.out_residual_ref(d["x"], w_used, d["b"], d["r"]))
+    with pytest.raises(AssertionError):
+        T.out_residual_decode_forward(torch.zeros(8, 2, 4096, dtype=torch.bfloat16, device=gpu), mod.weight, mod.bias,
+                                      torch.zeros(8, 1, 2880, dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(AssertionError):
+        T.out_residual_decode_forward(torch.zeros(8, 1, 4096, dtype=torch.bfloat16, device=gpu), mod.weight, mod.bias,
+                                      torch.zeros(8, 1, 2881, dtype=torch.bfloat16, device=gpu))

@@ -259,3 +259,17 @@ def test_fp8_rows_quantisation_pins():
     # half a step: normals 2^-4 relative; below 2^-6 (in units of scale) the step is fixed at 2^-9
     bound = torch.maximum(w.float().abs() * 2.0 ** -4, scale[:, None] * 2.0 ** -10) * 1.0001
     assert torch.all(err <= bound)
+
+
+def test_out_residual_ref_brute_force():
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(3, 40, generator=g).bfloat16()
+    w = (0.1 * torch.randn(7, 40, generator=g)).bfloat16()
+    b = (0.1 * torch.randn(7, generator=g)).bfloat16()
+    r = torch.randn(3, 7, generator=g).bfloat16()
+    want = torch.zeros(3, 7, dtype=torch.float64)
+    for i in range(3):
+        for n in range(7):
+            want[i, n] = sum(float(x[i, k]) * float(w[n, k]) for k in range(40)) + float(b[n]) + float(r[i, n])
+    torch.testing.assert_close(O.out_residual_ref(x, w, b, r).double(), want, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(O.out_residual_ref(x, w, None, None), O.linear_ref(x, w, None))

@@ -2,10 +2,11 @@
 clamped SwiGLU and the token-embedding gather, as hand-written HIP for gfx950 behind a
 C ABI (``include/tllm_hip.h``) with the reference model's Python call signatures on top."""
 from . import scratch_pool
-from .modules import QKV, Embedding, RMSNorm, RotaryEmbedding
+from .modules import OUT, QKV, Embedding, RMSNorm, RotaryEmbedding
 from .ops import (
     embedding_forward,
     linear_qkv_forward,
+    out_residual_decode_forward,
     qkv_decode_forward,
     qkv_rope_cache_decode_forward,
     qkv_rope_forward,
@@ -17,7 +18,7 @@ from .ops import (
 from .yarn import YarnParams, gpt_oss_yarn
 
 __all__ = [
-    "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
-    "embedding_forward", "linear_qkv_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
+    "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
+    "embedding_forward", "linear_qkv_forward", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
     "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu",
 ]

@@ -1,5 +1,5 @@
 """Leaf modules with the constructor and forward signatures of the reference's
-``gpt_oss/triton/model.py``: ``RMSNorm`` (:55-68), ``QKV`` (:119-167),
+``gpt_oss/triton/model.py``: ``RMSNorm`` (:55-68), ``QKV`` (:119-167), ``OUT`` (:170-216),
 ``RotaryEmbedding`` (:218-337) and the token ``Embedding`` (``torch.nn.Embedding``
 at :906-908). A model file written against the reference can import these instead.
 
@@ -66,6 +66,37 @@ class QKV(torch.nn.Module):
                                        positions=positions, offset=offset, tokens_per_batch=t,
                                        max_context_length=rope.max_context_length)
         return q.view(b, t, num_q_heads, d), k.view(b, t, num_kv_heads, d), v.view(b, t, num_kv_heads, d)
+
+
+class OUT(torch.nn.Module):
+    """Attention out-projection (model.py:170-216): ``weight [hidden_size, out_dim]``, ``bias [hidden_size]``.
+    ``decode_residual`` is the HIP kernel; ``forward`` is, as in the reference, the library GEMM."""
+
+    def __init__(self, out_dim: int, hidden_size: int, device: torch.device | None = None):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.empty((hidden_size, out_dim), device=device, dtype=torch.bfloat16))
+        self.bias = torch.nn.Parameter(torch.empty((hidden_size), device=device, dtype=torch.bfloat16))
+        self._use_fp8 = os.getenv("ATTN_FP8", "0").strip().lower() not in {"0", "false", "no", "off"}
+        self._weight_fp8: torch.Tensor | None = None
+        self._weight_scale: torch.Tensor | None = None
+
+    @property
+    def _fp8_weight(self):
+        if not self._use_fp8:
+            return None, None
+        if self._weight_fp8 is None:
+            self._weight_fp8, self._weight_scale = ops.quantize_fp8_rows(self.weight.detach())
+        return self._weight_fp8, self._weight_scale
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return torch.nn.functional.linear(x, self.weight, self.bias)
+
+    def decode_residual(self, x: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        """``residual + x @ W.T + b`` for ``x [B,1,out_dim]``, written into ``residual`` (model.py:199-216)."""
+        if self._use_fp8:
+            w_fp8, w_scale = self._fp8_weight
+            return ops.out_residual_decode_forward(x, w_fp8, self.bias, residual, weight_scale=w_scale)
+        return ops.out_residual_decode_forward(x, self.weight, self.bias, residual)
 
 
 class RotaryEmbedding(torch.nn.Module):

@@ -384,3 +384,39 @@ def linear_qkv_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     # all columns as "q heads" of one dense output row
     _launch_qkv(mode, x2, weight, bias, o2, None, None, total_out, 0, 0, 0, total_out // hd, 0, hd, None)
     return out
+
+
+# --------------------------------------------------------------------------------------- out-projection (decode)
+def out_residual_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, residual: torch.Tensor,
+                                weight_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """``residual + hidden @ weight.T + bias`` for one token per batch row (triton_kernels.py:1470-1517):
+    ``hidden [B,1,out_dim]``, ``weight [hidden_size, out_dim]`` (bf16, or float8_e4m3fn with ``weight_scale
+    [hidden_size]``), ``bias [hidden_size]``, ``residual [B,1,hidden_size]``. Like the reference the result is
+    written into ``residual``'s storage (when its last dimension is dense) and returned as ``[B,1,hidden_size]``."""
+    _on_gpu(hidden, weight, bias, residual, weight_scale)
+    batch, num_tokens, out_dim_hidden = hidden.shape
+    hidden_size, out_dim_weight = weight.shape
+    assert num_tokens == 1
+    assert out_dim_hidden == out_dim_weight
+    assert bias.shape == (hidden_size,)
+    assert residual.shape == (batch, 1, hidden_size)
+    assert hidden.dtype == _BF16 and bias.dtype == _BF16 and residual.dtype == _BF16
+    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
+    assert weight.dtype in (_BF16, _FP8)
+    x2 = hidden.reshape(batch, out_dim_hidden)
+    res2 = residual.reshape(batch, hidden_size)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    if not weight.is_contiguous():
+        weight = weight.contiguous()
+    if not bias.is_contiguous():
+        bias = bias.contiguous()
+    if res2.stride(-1) != 1:
+        res2 = res2.contiguous()
+    ws = None if weight_scale is None else _prep_weight_scale(weight, weight_scale)
+    out = res2
+    rc = lib().tllm_out_residual_decode_bf16(x2.data_ptr(), weight.data_ptr(), ws.data_ptr() if ws is not None else None, bias.data_ptr(),
+                                             res2.data_ptr(), out.data_ptr(), res2.stride(0), out.stride(0), batch, out_dim_hidden,
+                                             hidden_size, _stream())
+    check(rc, "out_residual_decode_forward")
+    return out[:, None, :]
