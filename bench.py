@@ -54,6 +54,10 @@ def algorithmic_bytes():
         # attention out-projection [2880, 4096] + bias + residual: weight, bias, x row, residual row in, output row out
         "out": lambda r: HIDDEN * 4096 * 2 + HIDDEN * 2 + r * (4096 * 2 + 2 * HIDDEN * 2),
         "out_w8": lambda r: HIDDEN * 4096 + HIDDEN * 4 + HIDDEN * 2 + r * (4096 * 2 + 2 * HIDDEN * 2),
+        # unembedding [201088, 2880]: weight + x rows in, bf16 logits out (argmax form: no logits)
+        "unembed": lambda r: VOCAB_BENCH * HIDDEN * 2 + r * (HIDDEN * 2 + VOCAB_BENCH * 2),
+        "unembed_argmax": lambda r: VOCAB_BENCH * HIDDEN * 2 + r * (HIDDEN * 2 + 4),
+        "unembed_w8": lambda r: VOCAB_BENCH * HIDDEN + VOCAB_BENCH * 4 + r * (HIDDEN * 2 + VOCAB_BENCH * 2),
         "norm_qkv_w8": lambda r: w // 2 + QKV_DIM * 4 + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
     }
 
@@ -89,6 +93,18 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         fn = (lambda i: T.out_residual_decode_forward(ox, ow[i % N_LAYERS][0], ob, ores, weight_scale=ow[i % N_LAYERS][1])) if w8 else \
              (lambda i: T.out_residual_decode_forward(ox, ow[i % N_LAYERS], ob, ores))
         nbytes = bytes_of["out_w8" if w8 else "out"](n)
+    elif kind in ("unembedding_decode", "unembedding_argmax", "unembedding_decode_w8"):
+        ux = torch.empty(n, 1, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        if kind.endswith("_w8"):
+            uw8, uws = T.quantize_fp8_rows(table)
+            fn = lambda i: T.unembedding_decode_forward(ux, uw8, uws)
+            nbytes = bytes_of["unembed_w8"](n)
+        elif kind == "unembedding_argmax":
+            fn = lambda i: T.unembedding_decode_argmax_forward(ux, table)
+            nbytes = bytes_of["unembed_argmax"](n)
+        else:
+            fn = lambda i: T.unembedding_decode_forward(ux, table)
+            nbytes = bytes_of["unembed"](n)
     elif kind == "rmsnorm":
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         to = torch.empty_like(xp)
@@ -325,6 +341,15 @@ def main() -> int:
                                                                                        weight_scale=ow8[i % N_LAYERS][1]),
                              bytes_of["out_w8"](r), n=240)
         del ow, ow8
+        # unembedding over the full vocabulary (the embedding table doubles as the [201088, 2880] weight: 1.16 GB per launch)
+        for r in (1, 8):
+            ux = torch.empty(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            bench_kernel(f"unembedding_decode_B{r}", lambda i, ux=ux: T.unembedding_decode_forward(ux, table), bytes_of["unembed"](r), n=10)
+            bench_kernel(f"unembedding_argmax_B{r}", lambda i, ux=ux: T.unembedding_decode_argmax_forward(ux, table),
+                         bytes_of["unembed_argmax"](r), n=10)
+        uw8, uws = T.quantize_fp8_rows(table)
+        bench_kernel("unembedding_decode_w8_B8", lambda i, ux=ux: T.unembedding_decode_forward(ux, uw8, uws), bytes_of["unembed_w8"](8), n=10)
+        del uw8, uws
         # prefill sizes
         for tt in (2048, 8192):
             xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)

@@ -187,6 +187,24 @@ int tllm_out_residual_decode_bf16(const void* x, const void* W, const float* w_s
                                   const void* residual, void* out, int64_t res_row_stride, int64_t out_row_stride,
                                   int64_t rows, int64_t in_dim, int64_t out_dim, void* stream);
 
+/* Decode-size unembedding over the whole vocabulary, logits[r, v] = sum_k x[r, k] * W[v, k] (fp32 accumulate, one
+ * RNE to bf16); replaces unembedding_decode_forward(hidden, weight), triton_kernels.py:163-197 (kernel :111-160),
+ * and with w_scale != NULL unembedding_decode_fp8_forward :271-302 (W = fp8 e4m3 bytes, one fp32 scale per
+ * vocabulary row, as quantised by :261-268). x [rows, hidden] bf16 dense, W [vocab, hidden] dense, logits
+ * [rows, vocab] with logits_row_stride elements between rows. hidden must be a multiple of 64. */
+int tllm_unembedding_decode_bf16(const void* x, const void* W, const float* w_scale, void* logits,
+                                 int64_t logits_row_stride, int64_t rows, int64_t hidden, int64_t vocab, void* stream);
+
+/* Greedy sampling fused into the same stream: token_ids[r] = argmax_v of the fp32 sums above (lowest index on a
+ * tie), no logits written; replaces unembedding_decode_argmax_forward, triton_kernels.py:363-401 (kernel
+ * :305-360 + the torch argmax over tiles), and its fp8 twin :470-512. The per-wavefront candidates pass through
+ * `workspace` (device memory, 4-byte aligned, at least tllm_unembedding_argmax_workspace_bytes(rows) bytes; the
+ * reference takes its partial_max / partial_idx from its scratch pool the same way). token_ids: int32 [rows]. */
+int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows);
+int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_scale, void* workspace,
+                                 int64_t workspace_bytes, int32_t* token_ids, int64_t rows, int64_t hidden,
+                                 int64_t vocab, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -564,3 +564,75 @@ def test_out_residual_other_shapes_module_and_errors(gpu, monkeypatch):
     with pytest.raises(AssertionError):
         T.out_residual_decode_forward(torch.zeros(8, 1, 4096, dtype=torch.bfloat16, device=gpu), mod.weight, mod.bias,
                                       torch.zeros(8, 1, 2881, dtype=torch.bfloat16, device=gpu))
+
+
+# ----------------------------------------------------------------------------------- unembedding (decode)
+def _argmax_ok(ids, logits_ref):
+    """The chosen token must be an argmax of the fp32 oracle logits up to summation noise: its oracle logit within
+    1e-3 of the oracle maximum; and where the oracle's winner is clear (margin > 1e-2) it must be that very token."""
+    ids = ids.cpu().long()
+    top2 = logits_ref.topk(2, dim=-1)
+    chosen = logits_ref.gather(1, ids[:, None])[:, 0]
+    assert torch.all(chosen >= top2.values[:, 0] - 1e-3), (chosen, top2.values[:, 0])
+    clear = (top2.values[:, 0] - top2.values[:, 1]) > 1e-2
+    assert torch.equal(ids[clear], top2.indices[clear, 0])
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 4096), (8, 5000), (13, 4097), (16, 20000), (20, 3001)])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_unembedding_decode_parity_small_vocab(gpu, rows, vocab, fp8):
+    g = torch.Generator().manual_seed(700 + rows)
+    x = torch.randn(rows, 2880, generator=g).bfloat16()
+    w = (0.02 * torch.randn(vocab, 2880, generator=g)).bfloat16()
+    xg = x.view(rows, 1, 2880).to(gpu)
+    if fp8:
+        w8, ws = T.quantize_fp8_rows(w.to(gpu))
+        want = O.linear_ref(x, O.dequant_fp8_ref(w8.cpu(), ws.cpu()), None)
+        logits = T.unembedding_decode_fp8_forward(xg, w8, ws).clone()
+        ids = T.unembedding_decode_fp8_argmax_forward(xg, w8, ws)
+    else:
+        want = O.linear_ref(x, w, None)
+        logits = T.unembedding_decode_forward(xg, w.to(gpu)).clone()
+        ids = T.unembedding_decode_argmax_forward(xg, w.to(gpu))
+    assert logits.shape == (rows, 1, vocab) and ids.shape == (rows,) and ids.dtype == torch.int32
+    close(logits.view(rows, vocab), want)
+    _argmax_ok(ids, want)
+
+
+def test_unembedding_full_vocabulary_and_module(gpu, monkeypatch):
+    """The real size: [201088, 2880]. Logits against the oracle on a sample of columns (the full fp32 product on
+    the CPU would take minutes), argmax against a planted winner, and the module's dispatch."""
+    monkeypatch.delenv("UNEMBED_FP8", raising=False)
+    vocab, rows = 201088, 8
+    gg = torch.Generator(device=gpu).manual_seed(3)
+    mod = T.UnEmbedding(2880, vocab, device=gpu)
+    with torch.no_grad():
+        mod.weight.normal_(0, 0.02, generator=gg)
+    g = torch.Generator().manual_seed(71)
+    x = torch.randn(rows, 2880, generator=g).bfloat16()
+    planted = torch.tensor([0, 31, 32, 100000, 201087, 77777, 12345, 201056])
+    with torch.no_grad():
+        for r in range(rows):                                  # row r of x points at weight row planted[r]
+            mod.weight[planted[r]] = (x[r].float() * 0.05).bfloat16().to(gpu)
+    xg = x.view(rows, 1, 2880).to(gpu)
+    logits = mod(xg).clone()
+    assert logits.shape == (rows, 1, vocab)
+    cols = torch.cat([torch.arange(0, 64), torch.arange(100000, 100064), torch.arange(vocab - 64, vocab), planted])
+    close(logits.view(rows, vocab)[:, cols.to(gpu)], O.linear_ref(x, mod.weight.detach()[cols.to(gpu)].cpu(), None))
+    ids = mod.forward_argmax(xg)
+    assert torch.equal(ids.cpu().long(), planted)
+    assert torch.equal(logits.view(rows, vocab).float().argmax(dim=-1).cpu(), planted)
+    # prefill-shaped input goes to the library GEMM like the reference's module
+    y = mod(torch.zeros(1, 3, 2880, dtype=torch.bfloat16, device=gpu))
+    assert y.shape == (1, 3, vocab)
+    # fp8 copy under UNEMBED_FP8
+    monkeypatch.setenv("UNEMBED_FP8", "1")
+    mod8 = T.UnEmbedding(2880, vocab, device=gpu)
+    with torch.no_grad():
+        mod8.weight.copy_(mod.weight)
+    assert torch.equal(mod8.forward_argmax(xg).cpu().long(), planted)
+    w8, ws = mod8._fp8()
+    l8 = mod8(xg)
+    close(l8.view(rows, vocab)[:, cols.to(gpu)], O.linear_ref(x, O.dequant_fp8_ref(w8[cols.to(gpu)].cpu(), ws[cols.to(gpu)].cpu()), None))
+    with pytest.raises(AssertionError):
+        T.unembedding_decode_forward(torch.zeros(2, 2, 2880, dtype=torch.bfloat16, device=gpu), mod.weight)

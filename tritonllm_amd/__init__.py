@@ -2,7 +2,7 @@
 clamped SwiGLU and the token-embedding gather, as hand-written HIP for gfx950 behind a
 C ABI (``include/tllm_hip.h``) with the reference model's Python call signatures on top."""
 from . import scratch_pool
-from .modules import OUT, QKV, Embedding, RMSNorm, RotaryEmbedding
+from .modules import OUT, QKV, Embedding, RMSNorm, RotaryEmbedding, UnEmbedding
 from .ops import (
     embedding_forward,
     linear_qkv_forward,
@@ -14,11 +14,16 @@ from .ops import (
     rmsnorm_forward,
     rope_forward,
     swiglu,
+    unembedding_decode_argmax_forward,
+    unembedding_decode_forward,
+    unembedding_decode_fp8_argmax_forward,
+    unembedding_decode_fp8_forward,
 )
 from .yarn import YarnParams, gpt_oss_yarn
 
 __all__ = [
     "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
     "embedding_forward", "linear_qkv_forward", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
-    "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu",
+    "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu", "UnEmbedding", "unembedding_decode_forward", "unembedding_decode_argmax_forward",
+    "unembedding_decode_fp8_forward", "unembedding_decode_fp8_argmax_forward",
 ]

@@ -1,0 +1,356 @@
+// Decode-size unembedding: logits[r, v] = sum_k x[r, k] * W[v, k] over the whole vocabulary, and its fused
+// greedy-sampling form that returns argmax_v instead of the logits
+// (unembedding_decode_forward triton_kernels.py:111-197, unembedding_decode_argmax_forward :305-401, the fp8-weight
+// twins :200-302 and :404-512). With W = [201088, 2880] bf16 this is a 1.16 GB stream per token -- the largest
+// single read of a decode step -- so the kernel is built around keeping HBM busy and nothing else:
+//
+//   * one workgroup of sixteen (eight) wavefronts per CU, alive for the whole launch; the few activation rows sit in LDS,
+//     read once per workgroup;
+//   * a wavefront owns whole 32-row vocabulary tiles (dealt round-robin, so every CU gets the same share +-1) and
+//     walks K in steps of 64: four 1 KB loads per step, each lane fetching 16 bytes so that eight lanes cover one
+//     128-byte line of one row (fully coalesced), four steps (16 KB per wavefront, 128 KB per CU) always in
+//     flight, the stream running on across tile boundaries;
+//   * a step's 32 x 64 block goes through a wavefront-private LDS patch into MFMA operand layout:
+//     v_mfma_f32_32x32x16_bf16 with the activations on M and the vocabulary rows on N, so a lane owns one
+//     vocabulary row and the logits of one batch row leave as 64-byte runs;
+//   * no wavefront ever waits for another: no barrier after the prologue, no cross-wavefront reduction.
+//
+// ARGMAX: instead of storing logits every lane keeps the best (value, index) it has seen per batch row (fp32
+// accumulator values, as the reference compares them); one shuffle reduction per wavefront at the end, one
+// (value, index) pair per wavefront and batch row into a small workspace, and a second tiny kernel picks the
+// winner. Ties go to the lowest index.
+//
+// W8: fp8 (OCP e4m3) weight with one fp32 scale per vocabulary row (triton_kernels.py:261-268): widened to bf16
+// on the way into the patch, the row scale multiplies the finished sum. Half the bytes.
+#include "common.h"
+
+namespace tllm {
+
+struct UnembedArgs {
+  const bf16* x;          // [rows, hidden]
+  const void* W;          // [vocab, hidden] bf16, or fp8 bytes when w_scale != null
+  const float* w_scale;   // [vocab] or null
+  bf16* logits;           // [rows, vocab] with row stride ld (logits form)
+  int64_t ld;
+  float* part_max;        // [gridDim.y][gridDim.x * UNW][XR] (argmax form)
+  int* part_idx;
+  int64_t rows;
+  int hidden, vocab;
+};
+
+namespace {
+constexpr int UD = 4;              // K steps in flight per wavefront
+constexpr int UPROW = 128 + 16;    // patch row: 64 bf16 + padding, bytes
+constexpr int UPATCH = 32 * UPROW;
+}  // namespace
+
+__host__ __device__ constexpr int unembed_xrow(int hidden) { return hidden * 2 + 16; }   // activation row in LDS, bytes
+
+// UNW wavefronts per workgroup: sixteen where LDS allows (up to 8 batch rows: measured 6.3 against 6.0 TB/s with eight),
+// eight with 16 batch rows resident.
+template <int XR, int UNW, bool W8, bool ARGMAX>
+__global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int xrow_b = unembed_xrow(a.hidden);
+  unsigned char* xs = smem;                                   // [XR][xrow_b]
+  unsigned char* patch = smem + XR * xrow_b + wave * UPATCH;  // this wavefront's [32][UPROW]
+  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
+  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+  const int kvec = a.hidden >> 3;                             // 16-byte chunks per activation row
+  const int nsteps = a.hidden >> 6;                           // K steps of 64
+
+  // ---- prologue: the activation rows into LDS (rows past the end repeat the last one; never stored)
+  for (int c = tid; c < XR * kvec; c += UNW * 64) {
+    int r = c / kvec;
+    const int kc = c - r * kvec;
+    const int rs = r < nvalid ? r : nvalid - 1;
+    *reinterpret_cast<bf16x8*>(xs + r * xrow_b + kc * 16) = reinterpret_cast<const bf16x8*>(a.x)[(row0 + rs) * kvec + kc];
+  }
+  __syncthreads();
+
+  // ---- this wavefront's tiles: t = gw, gw + G, gw + 2G, ...
+  const int gw = blockIdx.x * UNW + wave, G = gridDim.x * UNW;
+  const int ntiles = (a.vocab + 31) >> 5;
+  const int my_tiles = gw < ntiles ? (ntiles - gw + G - 1) / G : 0;
+  const int total = my_tiles * nsteps;                        // steps of the whole stream
+
+  // Weight bytes per row per K step: 128 (bf16) or 64 (fp8). One load instruction moves 1 KB: eight (sixteen)
+  // rows of one step; lane -> (row within the group, 16-byte chunk of the row's segment).
+  constexpr int LPS = W8 ? 2 : 4;                             // load instructions per step
+  constexpr int RPL = 32 / LPS;                               // rows per load instruction
+  constexpr int CPS = 64 / RPL;                               // 16-byte chunks per row per step
+  const int64_t wrow_vec = W8 ? (a.hidden >> 4) : (a.hidden >> 3);   // 16-byte chunks per weight row
+  const bf16x8* wv = reinterpret_cast<const bf16x8*>(a.W);
+  auto row_base = [&](int tile, int i) -> const bf16x8* {    // first chunk this lane fetches of load i in tile `tile`
+    int v = tile * 32 + i * RPL + lane / CPS;
+    v = v < a.vocab ? v : a.vocab - 1;                        // ragged last tile: repeat the last row (never stored)
+    return wv + static_cast<int64_t>(v) * wrow_vec + (lane % CPS);
+  };
+
+  bf16x8 buf[UD][LPS];
+  const bf16x8* lp[LPS];                                      // load cursor: row bases of the tile being requested
+  int l_tile = gw, l_step = 0, l_count = 0;
+#pragma unroll
+  for (int i = 0; i < LPS; ++i) lp[i] = row_base(my_tiles > 0 ? l_tile : 0, i);
+  // Unconditional on purpose (a load under a branch makes the compiler wait for it where the paths join): past
+  // the end of the stream the cursor simply stays on the last step and re-requests it.
+  auto issue = [&](int d) {                                   // request the next step of the stream into buf[d]
+#pragma unroll
+    for (int i = 0; i < LPS; ++i) buf[d][i] = __builtin_nontemporal_load(lp[i] + l_step * CPS);
+    if (l_count + 1 < total) {
+      ++l_count;
+      if (++l_step == nsteps) {
+        l_step = 0;
+        l_tile += G;
+#pragma unroll
+        for (int i = 0; i < LPS; ++i) lp[i] = row_base(l_tile < ntiles ? l_tile : ntiles - 1, i);
+      }
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < UD; ++d) issue(d);
+
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  constexpr int NB = XR / 2;                                  // accumulator registers that carry batch rows: row(v) = 8*(v>>2) + 4*h + (v&3)
+  float best[NB];
+  int best_i[NB];
+#pragma unroll
+  for (int v = 0; v < NB; ++v) {
+    best[v] = -3.0e38f;
+    best_i[v] = 0x7fffffff;
+  }
+
+  const unsigned char* xfrag = xs + (m & (XR - 1)) * xrow_b + h * 16;   // activations on M: tile rows >= XR repeat, never stored
+  const unsigned char* wfrag = patch + m * UPROW + h * 16;              // vocabulary rows on N
+  int c_tile = gw, c_step = 0;
+  for (int g0 = 0; g0 < total; g0 += UD) {
+#pragma unroll
+    for (int d = 0; d < UD; ++d) {
+      if (g0 + d < total) {                                   // uniform
+        // step (c_tile, c_step) is in buf[d]: into the patch, then four k16 MFMAs
+#pragma unroll
+        for (int i = 0; i < LPS; ++i) {
+          const int r = i * RPL + lane / CPS, kc = lane % CPS;
+          if constexpr (W8) {
+            typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
+            typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+            const i32x4 raw = __builtin_bit_cast(i32x4, buf[d][i]);
+            bf16x8 w0, w1;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[q], false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[q], true);
+              bf16x8& dst = q < 2 ? w0 : w1;
+              dst[4 * (q & 1) + 0] = static_cast<bf16>(p0[0]);
+              dst[4 * (q & 1) + 1] = static_cast<bf16>(p0[1]);
+              dst[4 * (q & 1) + 2] = static_cast<bf16>(p1[0]);
+              dst[4 * (q & 1) + 3] = static_cast<bf16>(p1[1]);
+            }
+            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32) = w0;
+            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32 + 16) = w1;
+          } else {
+            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 16) = buf[d][i];
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + c_step * 128 + t * 32);
+          const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        issue(d);                                             // buf[d] is free again: the step UD ahead
+        if (++c_step == nsteps) {                             // tile finished: lane owns vocabulary row c_tile*32 + m
+          const int v = c_tile * 32 + m;
+          float sc = 1.f;
+          if constexpr (W8) sc = a.w_scale[v < a.vocab ? v : a.vocab - 1];
+#pragma unroll
+          for (int r = 0; r < NB; ++r) {
+            const int brow = 8 * (r >> 2) + 4 * h + (r & 3);
+            const float val = acc[r] * sc;
+            if constexpr (ARGMAX) {
+              if (v < a.vocab && val > best[r]) {             // tiles come in ascending order: '>' keeps the lowest index
+                best[r] = val;
+                best_i[r] = v;
+              }
+            } else {
+              if (v < a.vocab && brow < nvalid) a.logits[(row0 + brow) * a.ld + v] = static_cast<bf16>(val);
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+          c_step = 0;
+          c_tile += G;
+        }
+      }
+    }
+  }
+
+  if constexpr (ARGMAX) {
+    // best of the wavefront per batch row: the 32 lanes of a half hold the same batch rows, different vocabulary rows
+#pragma unroll
+    for (int r = 0; r < NB; ++r) {
+      float bv = best[r];
+      int bi = best_i[r];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (m == 0) {
+        const int brow = 8 * (r >> 2) + 4 * h + (r & 3);
+        const int64_t slot = (static_cast<int64_t>(blockIdx.y) * G + gw) * XR + brow;
+        a.part_max[slot] = bv;
+        a.part_idx[slot] = bi;
+      }
+    }
+  }
+}
+
+// One workgroup per batch row: the winner among the per-wavefront candidates. Lowest index wins a tie.
+__global__ __launch_bounds__(256) void unembed_argmax_reduce_kernel(const float* part_max, const int* part_idx, int* token_ids, int n_part,
+                                                                    int xr) {
+  __shared__ float s_v[256];
+  __shared__ int s_i[256];
+  const int row = blockIdx.x;
+  const int chunk = row / xr, brow = row - chunk * xr;
+  float bv = -3.0e38f;
+  int bi = 0x7fffffff;
+  for (int p = threadIdx.x; p < n_part; p += 256) {
+    const int64_t slot = (static_cast<int64_t>(chunk) * n_part + p) * xr + brow;
+    const float v = part_max[slot];
+    const int i = part_idx[slot];
+    if (v > bv || (v == bv && i < bi)) {
+      bv = v;
+      bi = i;
+    }
+  }
+  s_v[threadIdx.x] = bv;
+  s_i[threadIdx.x] = bi;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (threadIdx.x < o) {
+      const float v = s_v[threadIdx.x + o];
+      const int i = s_i[threadIdx.x + o];
+      if (v > s_v[threadIdx.x] || (v == s_v[threadIdx.x] && i < s_i[threadIdx.x])) {
+        s_v[threadIdx.x] = v;
+        s_i[threadIdx.x] = i;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) token_ids[row] = s_i[0];
+}
+
+}  // namespace tllm
+
+using namespace tllm;
+
+namespace {
+constexpr int kUnembedGrid = 256;      // one workgroup per CU
+
+int unembed_xr(int64_t rows) { return rows <= 8 ? 8 : 16; }
+
+int unembed_nw(int xr) { return xr == 8 ? 16 : 8; }
+
+size_t unembed_smem(int xr, int64_t hidden) { return static_cast<size_t>(xr) * unembed_xrow((int)hidden) + unembed_nw(xr) * UPATCH; }
+
+int unembed_xr(int64_t rows);
+size_t unembed_smem(int xr, int64_t hidden);
+int unembed_check(const char* who, const void* x, const void* W, int64_t rows, int64_t hidden, int64_t vocab) {
+  TLLM_REQUIRE(rows >= 0 && hidden >= 1 && vocab >= 1 && vocab < (1ll << 31) && hidden < (1ll << 24), TLLM_E_SHAPE,
+               "%s: rows %lld, hidden %lld, vocab %lld", who, (long long)rows, (long long)hidden, (long long)vocab);
+  if (rows == 0) return TLLM_OK;
+  TLLM_REQUIRE(x && W, TLLM_E_ARG, "%s: x and W must not be NULL", who);
+  TLLM_REQUIRE(hidden % 64 == 0, TLLM_E_SHAPE, "%s: hidden %lld must be a multiple of 64", who, (long long)hidden);
+  TLLM_REQUIRE(unembed_smem(unembed_xr(rows), hidden) <= 160 * 1024, TLLM_E_SHAPE, "%s: hidden %lld too large for the LDS-resident activations", who,
+               (long long)hidden);
+  TLLM_REQUIRE(aligned16(x) && aligned16(W), TLLM_E_ALIGN, "%s: x and W must be 16-byte aligned", who);
+  TLLM_REQUIRE((rows + 15) / 16 <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many", who, (long long)rows);
+  return TLLM_OK;
+}
+
+template <bool ARGMAX>
+int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t st) {
+  const int xr = unembed_xr(a.rows);
+  const size_t smem = unembed_smem(xr, a.hidden);
+  const dim3 grid(kUnembedGrid, (unsigned)((a.rows + xr - 1) / xr));
+#define TLLM_UNEMBED(XR, W8F)                                                                                               \
+  do {                                                                                                                      \
+    auto kern = unembed_kernel<XR, (XR == 8 ? 16 : 8), W8F, ARGMAX>;                                                                            \
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+    TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "%s: cannot raise LDS limit: %s", who, hipGetErrorString(e));              \
+    hipLaunchKernelGGL(kern, grid, dim3(unembed_nw(XR) * 64), smem, st, a);                                                                 \
+  } while (0)
+  if (xr == 8) {
+    if (w8) TLLM_UNEMBED(8, true);
+    else TLLM_UNEMBED(8, false);
+  } else {
+    if (w8) TLLM_UNEMBED(16, true);
+    else TLLM_UNEMBED(16, false);
+  }
+#undef TLLM_UNEMBED
+  return check_launch(who);
+}
+}  // namespace
+
+extern "C" int tllm_unembedding_decode_bf16(const void* x, const void* W, const float* w_scale, void* logits, int64_t logits_row_stride,
+                                            int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
+  int rc = unembed_check("unembedding_decode", x, W, rows, hidden, vocab);
+  if (rc != TLLM_OK || rows == 0) return rc;
+  TLLM_REQUIRE(logits != nullptr && logits_row_stride >= vocab, TLLM_E_ARG, "unembedding_decode: logits NULL or row stride < vocab");
+  UnembedArgs a{};
+  a.x = (const bf16*)x;
+  a.W = W;
+  a.w_scale = w_scale;
+  a.logits = (bf16*)logits;
+  a.ld = logits_row_stride;
+  a.rows = rows;
+  a.hidden = (int)hidden;
+  a.vocab = (int)vocab;
+  return unembed_launch<false>("unembedding_decode", a, w_scale != nullptr, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows) {
+  if (rows <= 0) return 0;
+  const int xr = unembed_xr(rows);
+  const int64_t chunks = (rows + xr - 1) / xr;
+  return chunks * kUnembedGrid * unembed_nw(xr) * xr * 8;      // one (float, int) pair per wavefront and batch-row slot
+}
+
+extern "C" int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_scale, void* workspace, int64_t workspace_bytes,
+                                            int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
+  int rc = unembed_check("unembedding_argmax", x, W, rows, hidden, vocab);
+  if (rc != TLLM_OK || rows == 0) return rc;
+  const int64_t need = tllm_unembedding_argmax_workspace_bytes(rows);
+  TLLM_REQUIRE(token_ids != nullptr, TLLM_E_ARG, "unembedding_argmax: token_ids is NULL");
+  TLLM_REQUIRE(workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 4 == 0, TLLM_E_ARG,
+               "unembedding_argmax: workspace of %lld bytes needed (tllm_unembedding_argmax_workspace_bytes), got %lld", (long long)need,
+               (long long)workspace_bytes);
+  const int xr = unembed_xr(rows);
+  UnembedArgs a{};
+  a.x = (const bf16*)x;
+  a.W = W;
+  a.w_scale = w_scale;
+  a.part_max = static_cast<float*>(workspace);
+  a.part_idx = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) + need / 2);
+  a.rows = rows;
+  a.hidden = (int)hidden;
+  a.vocab = (int)vocab;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  rc = unembed_launch<true>("unembedding_argmax", a, w_scale != nullptr, st);
+  if (rc != TLLM_OK) return rc;
+  hipLaunchKernelGGL(unembed_argmax_reduce_kernel, dim3((unsigned)rows), dim3(256), 0, st, a.part_max, a.part_idx, token_ids,
+                     kUnembedGrid * unembed_nw(xr), xr);
+  return check_launch("unembedding_argmax(reduce)");
+}

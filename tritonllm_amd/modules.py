@@ -1,5 +1,5 @@
 """Leaf modules with the constructor and forward signatures of the reference's
-``gpt_oss/triton/model.py``: ``RMSNorm`` (:55-68), ``QKV`` (:119-167), ``OUT`` (:170-216),
+``gpt_oss/triton/model.py``: ``RMSNorm`` (:55-68), ``QKV`` (:119-167), ``OUT`` (:170-216), ``UnEmbedding`` (:70-117),
 ``RotaryEmbedding`` (:218-337) and the token ``Embedding`` (``torch.nn.Embedding``
 at :906-908). A model file written against the reference can import these instead.
 
@@ -97,6 +97,38 @@ class OUT(torch.nn.Module):
             w_fp8, w_scale = self._fp8_weight
             return ops.out_residual_decode_forward(x, w_fp8, self.bias, residual, weight_scale=w_scale)
         return ops.out_residual_decode_forward(x, self.weight, self.bias, residual)
+
+
+class UnEmbedding(torch.nn.Module):
+    """Output projection onto the vocabulary (model.py:70-117): ``weight [vocab_size, hidden_size]`` bf16.
+    One token per batch row goes through the HIP stream kernels (fp8 copy of the weight under ``UNEMBED_FP8``);
+    anything else is, as in the reference, the library GEMM."""
+
+    def __init__(self, hidden_size: int, vocab_size: int, device: torch.device | None = None):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.empty((vocab_size, hidden_size), device=device, dtype=torch.bfloat16))
+        self._use_fp8 = os.getenv("UNEMBED_FP8", "0").strip().lower() not in {"0", "false", "no", "off"}
+        self._weight_fp8: torch.Tensor | None = None
+        self._weight_scale: torch.Tensor | None = None
+
+    def _fp8(self):
+        if self._weight_fp8 is None:
+            self._weight_fp8, self._weight_scale = ops.quantize_fp8_rows(self.weight.detach())
+        return self._weight_fp8, self._weight_scale
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.is_cuda and x.ndim == 3 and x.shape[1] == 1 and x.dtype == torch.bfloat16:
+            if self._use_fp8:
+                return ops.unembedding_decode_forward(x, *self._fp8())
+            return ops.unembedding_decode_forward(x, self.weight)
+        return torch.nn.functional.linear(x, self.weight, bias=None)
+
+    def forward_argmax(self, x: torch.Tensor) -> torch.Tensor:
+        if x.is_cuda and x.ndim == 3 and x.shape[1] == 1 and x.dtype == torch.bfloat16:
+            if self._use_fp8:
+                return ops.unembedding_decode_argmax_forward(x, *self._fp8())
+            return ops.unembedding_decode_argmax_forward(x, self.weight)
+        return self.forward(x)[-1].argmax(dim=-1)
 
 
 class RotaryEmbedding(torch.nn.Module):

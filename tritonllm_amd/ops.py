@@ -420,3 +420,56 @@ def out_residual_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias
                                              hidden_size, _stream())
     check(rc, "out_residual_decode_forward")
     return out[:, None, :]
+
+
+# --------------------------------------------------------------------------------------- unembedding (decode)
+def _unembed_prep(hidden, weight, weight_scale):
+    _on_gpu(hidden, weight, weight_scale)
+    batch, num_tokens, hidden_size = hidden.shape
+    vocab_size, hidden_size_weight = weight.shape
+    assert num_tokens == 1
+    assert hidden_size == hidden_size_weight
+    assert hidden.dtype == _BF16
+    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
+    assert weight.dtype in (_BF16, _FP8)
+    x2 = hidden.reshape(batch, hidden_size)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    if not weight.is_contiguous():
+        weight = weight.contiguous()
+    ws = None if weight_scale is None else _prep_weight_scale(weight, weight_scale)
+    return x2, weight, ws, batch, hidden_size, vocab_size
+
+
+def unembedding_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """``hidden [B,1,H] @ weight[V,H].T -> logits [B,1,V]`` (a borrowed pool buffer), triton_kernels.py:163-197;
+    with ``weight_scale`` the fp8 form :271-302."""
+    x2, weight, ws, batch, hidden_size, vocab_size = _unembed_prep(hidden, weight, weight_scale)
+    logits = scratch_pool.get((batch, vocab_size), hidden.dtype, hidden.device)
+    rc = lib().tllm_unembedding_decode_bf16(x2.data_ptr(), weight.data_ptr(), ws.data_ptr() if ws is not None else None,
+                                            logits.data_ptr(), logits.stride(0), batch, hidden_size, vocab_size, _stream())
+    check(rc, "unembedding_decode_forward")
+    return logits[:, None, :]
+
+
+def unembedding_decode_fp8_forward(hidden, weight_fp8, weight_scale):
+    """triton_kernels.py:271-302."""
+    return unembedding_decode_forward(hidden, weight_fp8, weight_scale)
+
+
+def unembedding_decode_argmax_forward(hidden: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """Greedy token per batch row without materialising the logits: ``int32 [B]`` (triton_kernels.py:363-401;
+    with ``weight_scale`` :470-512). The candidates of the wavefronts travel through a pooled workspace."""
+    x2, weight, ws, batch, hidden_size, vocab_size = _unembed_prep(hidden, weight, weight_scale)
+    nbytes = lib().tllm_unembedding_argmax_workspace_bytes(batch)
+    work = scratch_pool.get((max(nbytes // 4, 1),), torch.float32, hidden.device)
+    ids = scratch_pool.get((batch,), torch.int32, hidden.device)
+    rc = lib().tllm_unembedding_argmax_bf16(x2.data_ptr(), weight.data_ptr(), ws.data_ptr() if ws is not None else None, work.data_ptr(),
+                                            work.numel() * 4, ids.data_ptr(), batch, hidden_size, vocab_size, _stream())
+    check(rc, "unembedding_decode_argmax_forward")
+    return ids
+
+
+def unembedding_decode_fp8_argmax_forward(hidden, weight_fp8, weight_scale):
+    """triton_kernels.py:470-512."""
+    return unembedding_decode_argmax_forward(hidden, weight_fp8, weight_scale)
