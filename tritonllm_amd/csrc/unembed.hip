@@ -38,28 +38,25 @@ struct UnembedArgs {
   int hidden, vocab;
 };
 
-namespace {
-constexpr int UD = 4;              // K steps in flight per wavefront
-constexpr int UPROW = 128 + 16;    // patch row: 64 bf16 + padding, bytes
-constexpr int UPATCH = 32 * UPROW;
-}  // namespace
+__host__ __device__ constexpr int unembed_patch(int ks) { return 32 * (ks * 2 + 16); }   // wavefront patch: 32 rows of KS bf16 + padding
 
 __host__ __device__ constexpr int unembed_xrow(int hidden) { return hidden * 2 + 16; }   // activation row in LDS, bytes
 
 // UNW wavefronts per workgroup: sixteen where LDS allows (up to 8 batch rows: measured 6.3 against 6.0 TB/s with eight),
 // eight with 16 batch rows resident.
-template <int XR, int UNW, bool W8, bool ARGMAX>
+template <int XR, int UNW, int KS, int UD, bool W8, bool ARGMAX>
 __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 31, h = lane >> 5;
   const int xrow_b = unembed_xrow(a.hidden);
   unsigned char* xs = smem;                                   // [XR][xrow_b]
+  constexpr int UPROW = KS * 2 + 16, UPATCH = unembed_patch(KS);
   unsigned char* patch = smem + XR * xrow_b + wave * UPATCH;  // this wavefront's [32][UPROW]
   const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
   const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
   const int kvec = a.hidden >> 3;                             // 16-byte chunks per activation row
-  const int nsteps = a.hidden >> 6;                           // K steps of 64
+  const int nsteps = a.hidden / KS;                           // K steps
 
   // ---- prologue: the activation rows into LDS (rows past the end repeat the last one; never stored)
   for (int c = tid; c < XR * kvec; c += UNW * 64) {
@@ -76,17 +73,18 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   const int my_tiles = gw < ntiles ? (ntiles - gw + G - 1) / G : 0;
   const int total = my_tiles * nsteps;                        // steps of the whole stream
 
-  // Weight bytes per row per K step: 128 (bf16) or 64 (fp8). One load instruction moves 1 KB: eight (sixteen)
-  // rows of one step; lane -> (row within the group, 16-byte chunk of the row's segment).
-  constexpr int LPS = W8 ? 2 : 4;                             // load instructions per step
-  constexpr int RPL = 32 / LPS;                               // rows per load instruction
-  constexpr int CPS = 64 / RPL;                               // 16-byte chunks per row per step
+  // One load instruction moves 1 KB; the 32 x (KS elements) block of a step is dealt to the lanes as 16-byte
+  // chunks in row-major order, so consecutive lanes cover consecutive bytes of a row (KS = 64: eight lanes per
+  // 128-byte line; KS = 192: 24 lanes per 384-byte run).
+  constexpr int CPS = (W8 ? KS : KS * 2) / 16;                // 16-byte chunks per row per step, as the weight lies in memory
+  constexpr int LPS = 32 * CPS / 64;                          // load instructions per step
   const int64_t wrow_vec = W8 ? (a.hidden >> 4) : (a.hidden >> 3);   // 16-byte chunks per weight row
   const bf16x8* wv = reinterpret_cast<const bf16x8*>(a.W);
   auto row_base = [&](int tile, int i) -> const bf16x8* {    // first chunk this lane fetches of load i in tile `tile`
-    int v = tile * 32 + i * RPL + lane / CPS;
+    const int c = i * 64 + lane;
+    int v = tile * 32 + c / CPS;
     v = v < a.vocab ? v : a.vocab - 1;                        // ragged last tile: repeat the last row (never stored)
-    return wv + static_cast<int64_t>(v) * wrow_vec + (lane % CPS);
+    return wv + static_cast<int64_t>(v) * wrow_vec + (c % CPS);
   };
 
   bf16x8 buf[UD][LPS];
@@ -131,10 +129,10 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
 #pragma unroll
     for (int d = 0; d < UD; ++d) {
       if (g0 + d < total) {                                   // uniform
-        // step (c_tile, c_step) is in buf[d]: into the patch, then four k16 MFMAs
+        // step (c_tile, c_step) is in buf[d]: into the patch, then KS / 16 MFMAs
 #pragma unroll
         for (int i = 0; i < LPS; ++i) {
-          const int r = i * RPL + lane / CPS, kc = lane % CPS;
+          const int r = (i * 64 + lane) / CPS, kc = (i * 64 + lane) % CPS;
           if constexpr (W8) {
             typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
             typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
@@ -158,8 +156,8 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + c_step * 128 + t * 32);
+        for (int t = 0; t < KS / 16; ++t) {
+          const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + c_step * (KS * 2) + t * 32);
           const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
           acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
         }
@@ -261,19 +259,26 @@ constexpr int kUnembedGrid = 256;      // one workgroup per CU
 
 int unembed_xr(int64_t rows) { return rows <= 8 ? 8 : 16; }
 
-int unembed_nw(int xr) { return xr == 8 ? 16 : 8; }
-
-size_t unembed_smem(int xr, int64_t hidden) { return static_cast<size_t>(xr) * unembed_xrow((int)hidden) + unembed_nw(xr) * UPATCH; }
+// (wavefronts, K step, steps in flight), measured at B = 8 on the full vocabulary:
+//   bf16, up to 8 rows : 16 wavefronts, K step 64 (whole 128-byte lines), 4 in flight   185 us (8 wavefronts: 194)
+//   fp8,  up to 8 rows :  8 wavefronts, K step 192, 2 in flight                          133 us (16 x 64 x 4: 167)
+//   16 rows            :  8 wavefronts (LDS holds the 16 activation rows), K step 64, 4 in flight
+// K steps that split 128-byte lines (96 elements of bf16, 32) cost 25-50 %.
+int unembed_nw(int xr, bool w8) { return (xr == 8 && !w8) ? 16 : 8; }
+int unembed_ks(int xr, bool w8, int64_t hidden) { return (xr == 8 && w8 && hidden % 192 == 0) ? 192 : 64; }
+size_t unembed_smem(int xr, bool w8, int64_t hidden) {
+  return static_cast<size_t>(xr) * unembed_xrow((int)hidden) + unembed_nw(xr, w8) * unembed_patch(unembed_ks(xr, w8, hidden));
+}
 
 int unembed_xr(int64_t rows);
-size_t unembed_smem(int xr, int64_t hidden);
-int unembed_check(const char* who, const void* x, const void* W, int64_t rows, int64_t hidden, int64_t vocab) {
+size_t unembed_smem(int xr, bool w8, int64_t hidden);
+int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_t rows, int64_t hidden, int64_t vocab) {
   TLLM_REQUIRE(rows >= 0 && hidden >= 1 && vocab >= 1 && vocab < (1ll << 31) && hidden < (1ll << 24), TLLM_E_SHAPE,
                "%s: rows %lld, hidden %lld, vocab %lld", who, (long long)rows, (long long)hidden, (long long)vocab);
   if (rows == 0) return TLLM_OK;
   TLLM_REQUIRE(x && W, TLLM_E_ARG, "%s: x and W must not be NULL", who);
   TLLM_REQUIRE(hidden % 64 == 0, TLLM_E_SHAPE, "%s: hidden %lld must be a multiple of 64", who, (long long)hidden);
-  TLLM_REQUIRE(unembed_smem(unembed_xr(rows), hidden) <= 160 * 1024, TLLM_E_SHAPE, "%s: hidden %lld too large for the LDS-resident activations", who,
+  TLLM_REQUIRE(unembed_smem(unembed_xr(rows), w8, hidden) <= 160 * 1024, TLLM_E_SHAPE, "%s: hidden %lld too large for the LDS-resident activations", who,
                (long long)hidden);
   TLLM_REQUIRE(aligned16(x) && aligned16(W), TLLM_E_ALIGN, "%s: x and W must be 16-byte aligned", who);
   TLLM_REQUIRE((rows + 15) / 16 <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many", who, (long long)rows);
@@ -283,22 +288,20 @@ int unembed_check(const char* who, const void* x, const void* W, int64_t rows, i
 template <bool ARGMAX>
 int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t st) {
   const int xr = unembed_xr(a.rows);
-  const size_t smem = unembed_smem(xr, a.hidden);
+  const size_t smem = unembed_smem(xr, w8, a.hidden);
   const dim3 grid(kUnembedGrid, (unsigned)((a.rows + xr - 1) / xr));
-#define TLLM_UNEMBED(XR, W8F)                                                                                               \
+#define TLLM_UNEMBED(XR, NW, KS, UD, W8F)                                                                                   \
   do {                                                                                                                      \
-    auto kern = unembed_kernel<XR, (XR == 8 ? 16 : 8), W8F, ARGMAX>;                                                                            \
+    auto kern = unembed_kernel<XR, NW, KS, UD, W8F, ARGMAX>;                                                                \
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "%s: cannot raise LDS limit: %s", who, hipGetErrorString(e));              \
-    hipLaunchKernelGGL(kern, grid, dim3(unembed_nw(XR) * 64), smem, st, a);                                                                 \
+    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, a);                                                             \
   } while (0)
-  if (xr == 8) {
-    if (w8) TLLM_UNEMBED(8, true);
-    else TLLM_UNEMBED(8, false);
-  } else {
-    if (w8) TLLM_UNEMBED(16, true);
-    else TLLM_UNEMBED(16, false);
-  }
+  if (xr == 8 && !w8) TLLM_UNEMBED(8, 16, 64, 4, false);
+  else if (xr == 8 && unembed_ks(8, true, a.hidden) == 192) TLLM_UNEMBED(8, 8, 192, 2, true);
+  else if (xr == 8) TLLM_UNEMBED(8, 8, 64, 4, true);
+  else if (w8) TLLM_UNEMBED(16, 8, 64, 4, true);
+  else TLLM_UNEMBED(16, 8, 64, 4, false);
 #undef TLLM_UNEMBED
   return check_launch(who);
 }
@@ -306,7 +309,7 @@ int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t s
 
 extern "C" int tllm_unembedding_decode_bf16(const void* x, const void* W, const float* w_scale, void* logits, int64_t logits_row_stride,
                                             int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
-  int rc = unembed_check("unembedding_decode", x, W, rows, hidden, vocab);
+  int rc = unembed_check("unembedding_decode", x, W, w_scale != nullptr, rows, hidden, vocab);
   if (rc != TLLM_OK || rows == 0) return rc;
   TLLM_REQUIRE(logits != nullptr && logits_row_stride >= vocab, TLLM_E_ARG, "unembedding_decode: logits NULL or row stride < vocab");
   UnembedArgs a{};
@@ -325,12 +328,12 @@ extern "C" int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows) {
   if (rows <= 0) return 0;
   const int xr = unembed_xr(rows);
   const int64_t chunks = (rows + xr - 1) / xr;
-  return chunks * kUnembedGrid * unembed_nw(xr) * xr * 8;      // one (float, int) pair per wavefront and batch-row slot
+  return chunks * kUnembedGrid * 16 * xr * 8;      // one (float, int) pair per wavefront (at most 16 per workgroup) and batch-row slot
 }
 
 extern "C" int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_scale, void* workspace, int64_t workspace_bytes,
                                             int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
-  int rc = unembed_check("unembedding_argmax", x, W, rows, hidden, vocab);
+  int rc = unembed_check("unembedding_argmax", x, W, w_scale != nullptr, rows, hidden, vocab);
   if (rc != TLLM_OK || rows == 0) return rc;
   const int64_t need = tllm_unembedding_argmax_workspace_bytes(rows);
   TLLM_REQUIRE(token_ids != nullptr, TLLM_E_ARG, "unembedding_argmax: token_ids is NULL");
@@ -351,6 +354,6 @@ extern "C" int tllm_unembedding_argmax_bf16(const void* x, const void* W, const 
   rc = unembed_launch<true>("unembedding_argmax", a, w_scale != nullptr, st);
   if (rc != TLLM_OK) return rc;
   hipLaunchKernelGGL(unembed_argmax_reduce_kernel, dim3((unsigned)rows), dim3(256), 0, st, a.part_max, a.part_idx, token_ids,
-                     kUnembedGrid * unembed_nw(xr), xr);
+                     kUnembedGrid * unembed_nw(xr, w_scale != nullptr), xr);
   return check_launch("unembedding_argmax(reduce)");
 }
