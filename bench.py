@@ -105,6 +105,18 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         else:
             fn = lambda i: T.unembedding_decode_forward(ux, table)
             nbytes = bytes_of["unembed"](n)
+    elif kind.startswith("attention_decode_"):
+        # attention_decode_ctx<L>_B<n> (full causal context of L keys) or attention_decode_win<L>_B<n> (window 128 inside a cache of L)
+        mode, ctx = kind[len("attention_decode_"):][:3], int(kind[len("attention_decode_") + 3:])
+        aq = torch.empty(n, 1, NKV, NQ // NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        ak = [torch.empty(n, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
+        av = [torch.empty(n, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
+        asink = torch.empty(NQ, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        astart = torch.tensor([ctx - 1], dtype=torch.int64, device=dev)
+        win = 128 if mode == "win" else None
+        fn = lambda i: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart)
+        keys = min(ctx, 128) if win else ctx
+        nbytes = n * NKV * keys * HD * 2 * 2 + n * NQ * HD * 2 * 2
     elif kind == "rmsnorm":
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         to = torch.empty_like(xp)
@@ -341,6 +353,18 @@ def main() -> int:
                                                                                        weight_scale=ow8[i % N_LAYERS][1]),
                              bytes_of["out_w8"](r), n=240)
         del ow, ow8
+        # decode attention: full causal context and the sliding-window layers, 4 rotating KV caches
+        for ctx, win, r in ((4096, None, 8), (4096, 128, 8), (4096, None, 1), (32768, None, 8)):
+            aq = torch.empty(r, 1, NKV, NQ // NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            ak = [torch.empty(r, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
+            av = [torch.empty(r, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
+            asink = torch.empty(NQ, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            astart = torch.tensor([ctx - 1], dtype=torch.int64, device=dev)
+            keys = min(ctx, win) if win else ctx
+            bench_kernel(f"attention_decode_{'win' if win else 'ctx'}{ctx}_B{r}",
+                         lambda i, aq=aq, ak=ak, av=av, asink=asink, astart=astart, win=win: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart),
+                         r * NKV * keys * HD * 2 * 2 + r * NQ * HD * 2 * 2, n=96)
+            del ak, av
         # unembedding over the full vocabulary (the embedding table doubles as the [201088, 2880] weight: 1.16 GB per launch)
         for r in (1, 8):
             ux = torch.empty(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)

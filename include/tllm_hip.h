@@ -205,6 +205,26 @@ int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_sc
                                  int64_t workspace_bytes, int32_t* token_ids, int64_t rows, int64_t hidden,
                                  int64_t vocab, void* stream);
 
+/* Decode attention with learned sinks and an optional sliding window: one new token per batch row against the KV
+ * cache; replaces attention_decode(q, k, v, sinks, sm_scale, bandwidth, start_q), attention_tt_decode.py:290-408
+ * (kernels :9-287), whose definition is attention_ref.py:4-42:
+ *   keys lo..hi-1, hi = min(start_q + 1, n_kv_ctx), lo = window ? max(0, start_q - window + 1) : 0;
+ *   out[h] = softmax over {sm_scale <q[h], k[n]>} U {sink[h]} applied to v (the sink has no value row).
+ * q, out: [batch, n_kv_heads * group * 64] bf16 (head h = kv_head * group + g), row strides in elements;
+ * k, v: [batch, n_kv_ctx, n_kv_heads, 64] bf16 with the given batch and token strides (the heads of a token
+ * dense); sinks: [n_kv_heads * group] bf16 or NULL (then every head has a sink of logit 0, as in the reference);
+ * start_q: DEVICE scalar, int32 or int64 (start_q_is_i64), read by the kernel; window 0 = none.
+ * Long contexts are split over workgroups: tllm_attention_decode_workspace_bytes(...) says how much device
+ * scratch (4-byte aligned) that needs for the same arguments -- 0 for short contexts; the reference allocates its
+ * acc/m/l partials per call (:343-345). head_dim must be 64, group <= 16. */
+int tllm_attention_decode_splits(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window);
+int64_t tllm_attention_decode_workspace_bytes(int64_t batch, int n_q_heads, int n_kv_heads, int64_t n_kv_ctx, int window);
+int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, const void* sinks, void* out,
+                               int64_t q_row_stride, int64_t out_row_stride, int64_t kv_batch_stride,
+                               int64_t kv_token_stride, int64_t batch, int64_t n_kv_ctx, int n_kv_heads, int group,
+                               int head_dim, float sm_scale, int window, const void* start_q, int start_q_is_i64,
+                               void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

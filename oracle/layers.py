@@ -31,6 +31,8 @@ force and special cases -- in ``tests/test_oracle_pins.py``:
     qkv_rope_ref                      composition of the above, v slice un-rotated
     swiglu_ref                        float64 brute force, edge grid, l=-1 => 0,
                                       interleaved == chunked under permutation
+    attention_decode_ref              float64 brute force per head, causal / window key ranges, sink limits
+                                      (-> -inf: plain softmax; -> +inf: zero output), equal keys => mean of values
     out_residual_ref                  linear_ref + an fp32 add; float64 brute force
     quantize_fp8_rows_ref /           all 256 e4m3 codes against the OCP bit formula, row maxima map to
     dequant_fp8_ref                   +-448, round-trip error within half a step of the format
@@ -146,6 +148,32 @@ def out_residual_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     if residual is not None:
         out = out + residual.to(torch.float32)
     return out
+
+
+def attention_decode_ref(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, sinks: torch.Tensor | None, sm_scale: float = 0.125,
+                         sliding_window: int | None = None, start_q: int = 0) -> torch.Tensor:
+    """attention_ref.py:4-42 for one query position (the decode case), fp32, returned as fp32 ``[bs, 1, heads*hd]``.
+
+    query ``[bs, 1, kv_heads, groups, hd]``, key/value ``[bs, n_keys, kv_heads, hd]``, sinks ``[kv_heads*groups]``
+    (``None``: logit 0 for every head, attention_tt_decode.py:55-58). Keys after position ``start_q`` are masked
+    (:20-23), keys older than ``start_q - sliding_window + 1`` too (:25-27); the sink joins the softmax
+    denominator but contributes no value (:32-37)."""
+    bs, nq, n_kv, groups, hd = query.shape
+    n_keys = key.shape[1]
+    assert nq == 1
+    sink = torch.zeros(n_kv * groups) if sinks is None else sinks.to(torch.float32)
+    sink = sink.view(1, n_kv, groups, 1)
+    pos = torch.arange(n_keys)
+    masked = pos > start_q
+    if sliding_window:
+        masked = masked | (pos < start_q - sliding_window + 1)
+    logits = torch.einsum("bhmd,bkhd->bhmk", query[:, 0].to(torch.float32), key.to(torch.float32)) * sm_scale
+    logits = logits.masked_fill(masked[None, None, None, :], float("-inf"))
+    top = torch.maximum(sink, logits.max(dim=-1, keepdim=True).values)
+    w = torch.exp(logits - top)
+    z = w.sum(dim=-1, keepdim=True) + torch.exp(sink - top)
+    out = torch.einsum("bhmk,bkhd->bhmd", w / z, value.to(torch.float32))
+    return out.reshape(bs, 1, n_kv * groups * hd)
 
 
 def quantize_fp8_rows_ref(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

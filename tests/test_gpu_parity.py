@@ -636,3 +636,57 @@ def test_unembedding_full_vocabulary_and_module(gpu, monkeypatch):
     close(l8.view(rows, vocab)[:, cols.to(gpu)], O.linear_ref(x, O.dequant_fp8_ref(w8[cols.to(gpu)].cpu(), ws[cols.to(gpu)].cpu()), None))
     with pytest.raises(AssertionError):
         T.unembedding_decode_forward(torch.zeros(2, 2, 2880, dtype=torch.bfloat16, device=gpu), mod.weight)
+
+
+# ----------------------------------------------------------------------------------- decode attention
+def _attn_case(gpu, batch_size, num_keys, sliding_window, start_q, start_dtype=torch.int32, seed=0, with_sinks=True, groups=8):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(batch_size, 1, 8, groups, 64, generator=g).bfloat16()
+    k = torch.randn(batch_size, num_keys, 8, 64, generator=g).bfloat16()
+    v = torch.randn(batch_size, num_keys, 8, 64, generator=g).bfloat16()
+    sinks = torch.randn(8 * groups, generator=g).bfloat16() if with_sinks else None
+    o1 = T.attention_decode(q.to(gpu), k.to(gpu), v.to(gpu), sinks.to(gpu) if with_sinks else None, 0.125, sliding_window,
+                            torch.tensor([start_q], dtype=start_dtype, device=gpu))
+    o2 = O.attention_decode_ref(q, k, v, sinks, 0.125, sliding_window, start_q)
+    assert o1.shape == (batch_size, 1, 8 * groups * 64) and o1.dtype == torch.bfloat16
+    # the reference's own bar (attention_tt_decode.py:429, 454) ...
+    torch.testing.assert_close(o1.float().cpu(), o2.bfloat16().float(), atol=1e-2, rtol=1e-1)
+    # ... and the tolerance of the other bf16 outputs of this library
+    close(o1, o2)
+
+
+@pytest.mark.parametrize("batch_size", [1, 2])
+@pytest.mark.parametrize("num_keys", [128, 1024])
+@pytest.mark.parametrize("sliding_window", [None, 128])
+@pytest.mark.parametrize("start_q", [0, 5, 63])
+def test_attention_decode_eq(gpu, batch_size, num_keys, sliding_window, start_q):
+    """The reference's test_decode_eq (attention_tt_decode.py:413-429), same parameter grid."""
+    _attn_case(gpu, batch_size, num_keys, sliding_window, start_q, seed=start_q + num_keys)
+
+
+@pytest.mark.parametrize("batch_size", [1, 2])
+@pytest.mark.parametrize("num_keys", [2048, 4096])
+@pytest.mark.parametrize("sliding_window", [None, 2048])
+@pytest.mark.parametrize("start_q", [0, 1023, 2047])
+def test_attention_decode_splitk(gpu, batch_size, num_keys, sliding_window, start_q):
+    """The reference's test_decode_splitk (attention_tt_decode.py:432-454): long contexts, split over workgroups."""
+    _attn_case(gpu, batch_size, num_keys, sliding_window, start_q, seed=start_q + num_keys)
+
+
+def test_attention_decode_edges(gpu):
+    _attn_case(gpu, 8, 4096, None, 4095, start_dtype=torch.int64, seed=1)       # full cache, int64 offset as the model passes it
+    _attn_case(gpu, 3, 4096, 128, 3000, start_dtype=torch.int64, seed=2)        # sliding window deep into a long cache
+    _attn_case(gpu, 1, 777, None, 776, seed=3)                                  # ragged last block
+    _attn_case(gpu, 2, 300, 128, 299, seed=4, with_sinks=False)                 # sinks=None -> logit 0 (attention_tt_decode.py:55-58)
+    _attn_case(gpu, 2, 256, None, 10000, seed=5)                                # start_q beyond the cache: every key is visible
+    _attn_case(gpu, 2, 200, None, 150, seed=6, groups=4)                        # another group size
+    # strided cache views (a cache allocated for more tokens than are handed over)
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(2, 1, 8, 8, 64, generator=g).bfloat16()
+    kc = torch.randn(2, 512, 8, 64, generator=g).bfloat16()
+    vc = torch.randn(2, 512, 8, 64, generator=g).bfloat16()
+    sinks = torch.randn(64, generator=g).bfloat16()
+    o1 = T.attention_decode(q.to(gpu), kc.to(gpu)[:, :300], vc.to(gpu)[:, :300], sinks.to(gpu), 0.125, None, torch.tensor([299], device=gpu))
+    close(o1, O.attention_decode_ref(q, kc[:, :300], vc[:, :300], sinks, 0.125, None, 299))
+    with pytest.raises(AssertionError):
+        T.attention_decode(q.to(gpu).expand(-1, 2, -1, -1, -1), kc.to(gpu), vc.to(gpu), sinks.to(gpu), 0.125, None, torch.tensor([1], device=gpu))

@@ -273,3 +273,35 @@ def test_out_residual_ref_brute_force():
             want[i, n] = sum(float(x[i, k]) * float(w[n, k]) for k in range(40)) + float(b[n]) + float(r[i, n])
     torch.testing.assert_close(O.out_residual_ref(x, w, b, r).double(), want, rtol=1e-5, atol=1e-5)
     torch.testing.assert_close(O.out_residual_ref(x, w, None, None), O.linear_ref(x, w, None))
+
+
+def test_attention_decode_ref_pins():
+    g = torch.Generator().manual_seed(11)
+    bs, n_keys, n_kv, groups, hd = 2, 40, 2, 3, 16
+    q = torch.randn(bs, 1, n_kv, groups, hd, generator=g).bfloat16()
+    k = torch.randn(bs, n_keys, n_kv, hd, generator=g).bfloat16()
+    v = torch.randn(bs, n_keys, n_kv, hd, generator=g).bfloat16()
+    sinks = torch.randn(n_kv * groups, generator=g).bfloat16()
+    for window, start in ((None, 39), (None, 7), (8, 20), (8, 3), (100, 25)):
+        got = O.attention_decode_ref(q, k, v, sinks, 0.25, window, start).view(bs, n_kv, groups, hd)
+        lo = max(0, start - window + 1) if window else 0
+        for b in range(bs):
+            for h in range(n_kv):
+                for m in range(groups):
+                    s = [0.25 * sum(float(q[b, 0, h, m, d]) * float(k[b, n, h, d]) for d in range(hd)) for n in range(lo, start + 1)]
+                    sk = float(sinks[h * groups + m])
+                    top = max(max(s), sk)
+                    wts = [math.exp(x - top) for x in s]
+                    z = sum(wts) + math.exp(sk - top)
+                    want = [sum(wts[i] * float(v[b, lo + i, h, d]) for i in range(len(s))) / z for d in range(hd)]
+                    torch.testing.assert_close(got[b, h, m].double(), torch.tensor(want, dtype=torch.float64), rtol=1e-4, atol=1e-5)
+    # sink -> -inf: plain causal softmax; sink -> +inf: nothing is left for the values; no sinks = logit 0
+    plain = O.attention_decode_ref(q, k, v, torch.full((6,), -1e4), 0.25, None, 39).view(bs, n_kv, groups, hd)
+    sm = torch.softmax(torch.einsum("bhmd,bkhd->bhmk", q[:, 0].float(), k.float()) * 0.25, dim=-1)
+    torch.testing.assert_close(plain, torch.einsum("bhmk,bkhd->bhmd", sm, v.float()), rtol=1e-5, atol=1e-6)
+    assert O.attention_decode_ref(q, k, v, torch.full((6,), 1e4), 0.25, None, 39).abs().max() < 1e-6
+    torch.testing.assert_close(O.attention_decode_ref(q, k, v, None, 0.25, None, 39), O.attention_decode_ref(q, k, v, torch.zeros(6), 0.25, None, 39))
+    # all keys equal: every weight is the same, output = mean of the values times the non-sink share
+    ke = k[:, :1].expand(-1, n_keys, -1, -1)
+    out = O.attention_decode_ref(q, ke, v, torch.full((6,), -1e4), 0.25, None, 39).view(bs, n_kv, groups, hd)
+    torch.testing.assert_close(out, v.float().mean(dim=1)[:, :, None, :].expand(-1, -1, groups, -1), rtol=1e-5, atol=1e-6)

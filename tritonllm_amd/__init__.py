@@ -4,6 +4,7 @@ C ABI (``include/tllm_hip.h``) with the reference model's Python call signatures
 from . import scratch_pool
 from .modules import OUT, QKV, Embedding, RMSNorm, RotaryEmbedding, UnEmbedding
 from .ops import (
+    attention_decode,
     embedding_forward,
     linear_qkv_forward,
     out_residual_decode_forward,
@@ -23,7 +24,7 @@ from .yarn import YarnParams, gpt_oss_yarn
 
 __all__ = [
     "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
-    "embedding_forward", "linear_qkv_forward", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
+    "attention_decode", "embedding_forward", "linear_qkv_forward", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
     "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu", "UnEmbedding", "unembedding_decode_forward", "unembedding_decode_argmax_forward",
     "unembedding_decode_fp8_forward", "unembedding_decode_fp8_argmax_forward",
 ]

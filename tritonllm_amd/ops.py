@@ -473,3 +473,49 @@ def unembedding_decode_argmax_forward(hidden: torch.Tensor, weight: torch.Tensor
 def unembedding_decode_fp8_argmax_forward(hidden, weight_fp8, weight_scale):
     """triton_kernels.py:470-512."""
     return unembedding_decode_argmax_forward(hidden, weight_fp8, weight_scale)
+
+
+# --------------------------------------------------------------------------------------- decode attention
+def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Tensor | None, sm_scale: float,
+                     bandwidth: int | None, start_q: torch.Tensor) -> torch.Tensor:
+    """One new token per batch row against the KV cache, with sinks and an optional sliding window
+    (attention_tt_decode.py:290-408): ``q [bs, 1, n_kv_heads, repeat_kv, 64]``, ``k, v [bs, n_kv_ctx, n_kv_heads, 64]``,
+    ``sinks [n_kv_heads * repeat_kv]`` bf16, ``start_q`` a device tensor of one int32/int64 element (read on the
+    device), ``bandwidth`` the sliding window (``None`` / 0: none). Returns ``[bs, 1, n_heads * 64]`` (pooled)."""
+    _on_gpu(q, k, v, sinks, start_q)
+    assert len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64)
+    bs, n_ctx, n_kv_heads, repeat_kv, head_dim_q = q.shape
+    bs_k, n_kv_ctx, n_kv_heads_k, head_dim_k = k.shape
+    bs_v, n_kv_ctx_v, n_kv_heads_v, head_dim_v = v.shape
+    assert n_ctx == 1
+    assert bs == bs_k == bs_v and n_kv_ctx == n_kv_ctx_v
+    assert n_kv_heads == n_kv_heads_k == n_kv_heads_v
+    assert head_dim_q == head_dim_k == head_dim_v
+    assert head_dim_q in {16, 32, 64, 128, 256}
+    if head_dim_q != 64 or repeat_kv > 16:
+        raise NotImplementedError("attention_decode: the HIP kernel is built for head_dim 64 and up to 16 query heads per KV head")
+    assert q.dtype == _BF16 and k.dtype == _BF16 and v.dtype == _BF16 and (sinks is None or sinks.dtype == _BF16)
+    n_heads = n_kv_heads * repeat_kv
+    q2 = q[:, 0].reshape(bs, n_heads * 64)
+    if not q2.is_contiguous():
+        q2 = q2.contiguous()
+
+    def dense_heads(t):
+        return t if (t.stride(3) == 1 and t.stride(2) == 64 and t.stride(1) % 8 == 0 and t.stride(0) % 8 == 0) else t.contiguous()
+
+    k, v = dense_heads(k), dense_heads(v)
+    if k.stride() != v.stride():
+        k, v = k.contiguous(), v.contiguous()
+    if sinks is not None:
+        assert sinks.shape == (n_heads,)
+        sinks = sinks if sinks.is_contiguous() else sinks.contiguous()
+    window = int(bandwidth) if bandwidth else 0
+    o = scratch_pool.get((bs, n_heads * 64), q.dtype, q.device)
+    nbytes = lib().tllm_attention_decode_workspace_bytes(bs, n_heads, n_kv_heads, n_kv_ctx, window)
+    work = scratch_pool.get((max(nbytes // 4, 1),), torch.float32, q.device) if nbytes else None
+    rc = lib().tllm_attention_decode_bf16(q2.data_ptr(), k.data_ptr(), v.data_ptr(), sinks.data_ptr() if sinks is not None else None,
+                                          o.data_ptr(), q2.stride(0), o.stride(0), k.stride(0), k.stride(1), bs, n_kv_ctx, n_kv_heads,
+                                          repeat_kv, 64, float(sm_scale), window, start_q.data_ptr(), int(start_q.dtype == torch.int64),
+                                          work.data_ptr() if work is not None else None, nbytes, _stream())
+    check(rc, "attention_decode")
+    return o.view(bs, 1, n_heads * 64)
