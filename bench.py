@@ -429,6 +429,37 @@ def main() -> int:
             stack[f"B{r}"] = {"us_per_token_step": round(sec * 1e6, 2), "tokens/s": round(r / sec, 1), "launches": launches,
                               "weight_GB/s": round(N_LAYERS * QKV_DIM * HIDDEN * 2 / sec / 1e9, 1)}
 
+    # ---------------------------------------------------------------- attention blocks of a 24-layer decode step
+    # per layer: RMSNorm + QKV + bias + RoPE with the KV-cache write (one launch), attention over the cache (sliding
+    # window 128 on even layers, model.py:448), out-projection + bias + residual. Context 4096, one graph replay per token.
+    attn_stack = {}
+    if not args.no_kernel_table:
+        rope = T.RotaryEmbedding(HD, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=dev)
+        ow = [torch.empty(HIDDEN, NQ * HD, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
+        ob = torch.empty(HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
+        asink = torch.empty(NQ, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        ctx = 4096
+        off = torch.tensor([ctx - 1], dtype=torch.int64, device=dev)
+        for r in (1, 8):
+            ck = [torch.empty(r, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(N_LAYERS)]
+            cv = [torch.empty(r, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(N_LAYERS)]
+            xr = torch.randn(r, 1, HIDDEN, generator=g).bfloat16().to(dev)
+
+            def attn_step(_i, r=r, ck=ck, cv=cv, xr=xr):
+                for l in range(N_LAYERS):
+                    qh = T.qkv_rope_cache_decode_forward(xr, weights[l], biases[l], rope.sin, rope.cos, rope.max_context_length, ck[l], cv[l],
+                                                         off, NQ, NKV, HD, norm_scale=scales[l], norm_eps=1e-5)
+                    th = T.attention_decode(qh.view(r, 1, NKV, NQ // NKV, HD), ck[l], cv[l], asink, 0.125, 128 if l % 2 == 0 else None, off)
+                    T.out_residual_decode_forward(th, ow[l], ob, xr)
+
+            attn_step(0)
+            gr = graph_of(attn_step, 2)
+            gr.replay()
+            sec = min(time_graph(gr) for _ in range(5)) / 2
+            attn_stack[f"B{r}_ctx{ctx}"] = {"us_per_token_step": round(sec * 1e6, 2), "us_per_layer": round(sec * 1e6 / N_LAYERS, 2),
+                                            "tokens/s": round(r / sec, 1)}
+            del ck, cv
+
     # ---------------------------------------------------------------- CPU baseline (reported only)
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -471,7 +502,7 @@ def main() -> int:
                                "clamped SwiGLU[32,5760]; 24 rotating weight sets; HIP-graph replay of all steps",
                    "batch": B, "layers_rotated": N_LAYERS,
                    "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel"},
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack,
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "attention_blocks24": attn_stack,
         "wall_s_timed_region": round(wall, 4),
     }
     print(json.dumps(out))

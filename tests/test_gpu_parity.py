@@ -690,3 +690,36 @@ def test_attention_decode_edges(gpu):
     close(o1, O.attention_decode_ref(q, kc[:, :300], vc[:, :300], sinks, 0.125, None, 299))
     with pytest.raises(AssertionError):
         T.attention_decode(q.to(gpu).expand(-1, 2, -1, -1, -1), kc.to(gpu), vc.to(gpu), sinks.to(gpu), 0.125, None, torch.tensor([1], device=gpu))
+
+
+def test_attention_block_decode_chain(gpu):
+    """The whole attention block of a decode step as model.py:471-573 strings it together -- RMSNorm, QKV + bias + RoPE
+    with the new k/v written into the cache at `offset`, attention over the cache with sinks (full and windowed),
+    out-projection + bias + residual -- every stage on the HIP kernels, against the oracle chain."""
+    bs, n_ctx, slot = 4, 300, 207
+    d = O.make_inputs(bs, seed=81)
+    g = torch.Generator().manual_seed(82)
+    cache_k = torch.randn(bs, n_ctx, 8, 64, generator=g).bfloat16()
+    cache_v = torch.randn(bs, n_ctx, 8, 64, generator=g).bfloat16()
+    sinks = torch.randn(64, generator=g).bfloat16()
+    w_out = (0.02 * torch.randn(2880, 4096, generator=g)).bfloat16()
+    b_out = (0.02 * torch.randn(2880, generator=g)).bfloat16()
+    rope = T.RotaryEmbedding(64, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=gpu)
+    offset = torch.tensor([slot], dtype=torch.int64, device=gpu)
+    for window in (None, 128):
+        ck, cv = cache_k.to(gpu), cache_v.to(gpu)
+        x = d["x"].view(bs, 1, 2880).to(gpu)
+        q = T.qkv_rope_cache_decode_forward(x, d["w"].to(gpu), d["b"].to(gpu), rope.sin, rope.cos, rope.max_context_length, ck, cv, offset,
+                                            64, 8, 64, norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+        t = T.attention_decode(q.view(bs, 1, 8, 8, 64), ck, cv, sinks.to(gpu), 0.125, window, offset)
+        y = T.out_residual_decode_forward(t, w_out.to(gpu), b_out.to(gpu), x.clone())
+        # oracle chain, rounding to bf16 wherever a tensor crosses from one reference kernel to the next
+        tn = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16()
+        qr, kr, vr = O.qkv_rope_ref(tn, d["w"], d["b"], torch.full((bs,), slot, dtype=torch.int64))
+        rk, rv = cache_k.clone(), cache_v.clone()
+        rk[:, slot] = kr.bfloat16().view(bs, 8, 64)
+        rv[:, slot] = vr.bfloat16().view(bs, 8, 64)
+        tr = O.attention_decode_ref(qr.bfloat16().view(bs, 1, 8, 8, 64), rk, rv, sinks, 0.125, window, slot).bfloat16()
+        yr = O.out_residual_ref(tr.view(bs, 4096), w_out, b_out, d["x"])
+        close(t, tr.float())
+        close(y.view(bs, 2880), yr)
