@@ -2,8 +2,8 @@
 //
 // Pure streaming (17 280 bytes per gpt-oss row): each lane loads 32 bytes of input
 // (eight gate/linear pairs when interleaved), computes in fp32 and stores one 128-bit
-// vector of eight bf16 outputs. The grid-stride loop runs over output vectors of the
-// whole [rows, n_out] matrix, so small and large row counts use the same kernel.
+// vector of eight bf16 outputs. The grid runs over the output vectors of the
+// whole [rows, n_out] matrix, one per thread, so small and large row counts use the same kernel.
 #include "common.h"
 
 namespace tllm {
@@ -14,42 +14,46 @@ __device__ __forceinline__ float swiglu1(float g, float l, float alpha, float li
     l = l > limit ? limit : l;                 // linear: both sides
     l = l < -limit ? -limit : l;
   }
-  const float s = g / (1.0f + __expf(-alpha * g));   // g * sigmoid(alpha * g)
+  // g * sigmoid(alpha * g). The quotient goes through the hardware reciprocal (1 ulp): an IEEE division is ten more
+  // instructions per element and this kernel has eight elements per 48 bytes of traffic to get through.
+  const float s = g * __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * g));
   return fmaf(s, l, s);                              // s * (l + 1)
 }
 
+// One output vector per thread, workgroups in memory order: the grid then sweeps the input like one contiguous
+// read (measured at [32768, 5760]: 87 us = 6.5 TB/s; a grid-stride loop over 32 workgroups per CU 94 us, with two
+// or four vectors per thread and iteration 99 / 112 us).
 template <bool kInterleaved>
 __global__ __launch_bounds__(256) void swiglu_vec_kernel(const bf16x8* __restrict__ x, bf16x8* __restrict__ out, int64_t rows,
                                                          int nvec_out, int64_t x_row_stride_vec, float alpha, float limit,
                                                          int has_limit) {
   const int64_t total = rows * nvec_out;
-  const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < total; v += step) {
-    const int64_t row = v / nvec_out;
-    const int c = static_cast<int>(v - row * nvec_out);
-    const bf16x8* xr = x + row * x_row_stride_vec;
-    bf16x8 a, b;
-    if constexpr (kInterleaved) {
-      a = xr[2 * c];
-      b = xr[2 * c + 1];
-    } else {
-      a = xr[c];
-      b = xr[nvec_out + c];
-    }
-    bf16x8 o;
-    if constexpr (kInterleaved) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        o[j] = static_cast<bf16>(swiglu1(static_cast<float>(a[2 * j]), static_cast<float>(a[2 * j + 1]), alpha, limit, has_limit));
-        o[4 + j] = static_cast<bf16>(swiglu1(static_cast<float>(b[2 * j]), static_cast<float>(b[2 * j + 1]), alpha, limit, has_limit));
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        o[j] = static_cast<bf16>(swiglu1(static_cast<float>(a[j]), static_cast<float>(b[j]), alpha, limit, has_limit));
-    }
-    out[v] = o;
+  const int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (v >= total) return;
+  const int64_t row = v / nvec_out;
+  const int c = static_cast<int>(v - row * nvec_out);
+  const bf16x8* xr = x + row * x_row_stride_vec;
+  bf16x8 a, b;
+  if constexpr (kInterleaved) {
+    a = __builtin_nontemporal_load(xr + 2 * c);
+    b = __builtin_nontemporal_load(xr + 2 * c + 1);
+  } else {
+    a = __builtin_nontemporal_load(xr + c);
+    b = __builtin_nontemporal_load(xr + nvec_out + c);
   }
+  bf16x8 o;
+  if constexpr (kInterleaved) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[j] = static_cast<bf16>(swiglu1(static_cast<float>(a[2 * j]), static_cast<float>(a[2 * j + 1]), alpha, limit, has_limit));
+      o[4 + j] = static_cast<bf16>(swiglu1(static_cast<float>(b[2 * j]), static_cast<float>(b[2 * j + 1]), alpha, limit, has_limit));
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      o[j] = static_cast<bf16>(swiglu1(static_cast<float>(a[j]), static_cast<float>(b[j]), alpha, limit, has_limit));
+  }
+  __builtin_nontemporal_store(o, out + v);
 }
 
 __global__ __launch_bounds__(256) void swiglu_scalar_kernel(const bf16* __restrict__ x, bf16* __restrict__ out, int64_t rows,
@@ -80,8 +84,8 @@ extern "C" int tllm_swiglu_bf16(const void* x, void* out, int64_t rows, int64_t 
   const bool vec_ok = n_out % 8 == 0 && x_row_stride % 8 == 0 && aligned16(x) && aligned16(out) && n_out / 8 < (1ll << 31);
   if (vec_ok) {
     const int64_t total = rows * (n_out / 8);
-    int64_t blocks = (total + 255) / 256;
-    if (blocks > 256 * 32) blocks = 256 * 32;
+    const int64_t blocks = (total + 255) / 256;
+    TLLM_REQUIRE(blocks < (1ll << 31), TLLM_E_SHAPE, "swiglu: %lld output vectors are too many for one launch", (long long)total);
     dim3 grid(static_cast<unsigned>(blocks)), block(256);
     if (interleaved)
       hipLaunchKernelGGL(swiglu_vec_kernel<true>, grid, block, 0, st, (const bf16x8*)x, (bf16x8*)out, rows, (int)(n_out / 8),
