@@ -470,6 +470,13 @@ def unembedding_decode_argmax_forward(hidden: torch.Tensor, weight: torch.Tensor
     return ids
 
 
+def unembedding_forward(hidden: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """triton_kernels.py:515-525: the stream kernel for one bf16 token per batch row on the GPU, the library GEMM otherwise."""
+    if hidden.is_cuda and hidden.ndim == 3 and hidden.shape[1] == 1 and hidden.dtype == _BF16 and weight.dtype == _BF16:
+        return unembedding_decode_forward(hidden, weight)
+    return torch.nn.functional.linear(hidden, weight, bias=None)
+
+
 def unembedding_decode_fp8_argmax_forward(hidden, weight_fp8, weight_scale):
     """triton_kernels.py:470-512."""
     return unembedding_decode_argmax_forward(hidden, weight_fp8, weight_scale)
