@@ -47,6 +47,7 @@ def algorithmic_bytes():
         "rmsnorm": lambda r: r * 2 * HIDDEN * 2 + HIDDEN * 2,
         "embedding": lambda t: t * (2 * HIDDEN * 2 + 4),
         "swiglu": lambda m: m * (2 * HIDDEN * 2 + HIDDEN * 2),
+        "mxfp4": lambda blocks: blocks * (16 + 1 + 64),
         "qkv": lambda r: w + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
         "norm_qkv": lambda r: w + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
         # fp8 weight: one byte per element + one fp32 scale per output row
@@ -132,6 +133,13 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         hp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev)
         fn = lambda i: T.embedding_forward(idp, table, out=hp)
         nbytes = bytes_of["embedding"](n)
+    elif kind == "mxfp4_dequant":
+        # mxfp4_dequant_E<n>: the mlp1 weight of n experts, [n, 5760, 2880] from [n, 5760, 90, 16] blocks
+        mb = torch.randint(0, 256, (n, 2 * HIDDEN, HIDDEN // 32, 16), dtype=torch.uint8, device=dev, generator=gg)
+        ms = torch.randint(110, 130, (n, 2 * HIDDEN, HIDDEN // 32), dtype=torch.uint8, device=dev, generator=gg)
+        mo = torch.empty(n, 2 * HIDDEN, HIDDEN, dtype=torch.bfloat16, device=dev)
+        fn = lambda i: T.mxfp4_dequant(mb, ms, out=mo)
+        nbytes = bytes_of["mxfp4"](ms.numel())
     else:
         print(f"bench.py: unknown --only target {name}", file=sys.stderr)
         return 2
@@ -395,6 +403,11 @@ def main() -> int:
         so = torch.empty(32768, HIDDEN, dtype=torch.bfloat16, device=dev)
         bench_kernel("swiglu_M32768", lambda i: T.swiglu(sx, out=so), bytes_of["swiglu"](32768), n=48)
         del sx, so
+        mb = torch.randint(0, 256, (32, 2 * HIDDEN, HIDDEN // 32, 16), dtype=torch.uint8, device=dev, generator=gg)
+        ms = torch.randint(110, 130, (32, 2 * HIDDEN, HIDDEN // 32), dtype=torch.uint8, device=dev, generator=gg)
+        mo = torch.empty(32, 2 * HIDDEN, HIDDEN, dtype=torch.bfloat16, device=dev)
+        bench_kernel("mxfp4_dequant_E32", lambda i: T.mxfp4_dequant(mb, ms, out=mo), bytes_of["mxfp4"](ms.numel()), n=12)
+        del mb, ms, mo
 
     # ---------------------------------------------------------------- 24-layer per-token stack (one graph replay = one token step)
     stack = {}

@@ -225,6 +225,12 @@ int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, cons
                                int head_dim, float sm_scale, int window, const void* start_q, int start_q_is_i64,
                                void* workspace, int64_t workspace_bytes, void* stream);
 
+/* MXFP4 -> bf16 expansion of checkpoint tensors (Checkpoint._get_mxfp4_tensor, weights.py:68-117): blocks
+ * [n_blocks][16] bytes, 32 e2m1 values per block with the low nibble first (table weights.py:11-14); scales [n_blocks]
+ * e8m0 bytes (bias 127); out [n_blocks][32] bf16 = FP4[nibble] * 2^(scale - 127), formed in fp32 and rounded once, as
+ * torch.ldexp does on the reference's bf16 tensor. Bit-exact. */
+int tllm_mxfp4_dequant_bf16(const void* blocks, const void* scales, void* out, int64_t n_blocks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

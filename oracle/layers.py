@@ -36,6 +36,9 @@ force and special cases -- in ``tests/test_oracle_pins.py``:
     out_residual_ref                  linear_ref + an fp32 add; float64 brute force
     quantize_fp8_rows_ref /           all 256 e4m3 codes against the OCP bit formula, row maxima map to
     dequant_fp8_ref                   +-448, round-trip error within half a step of the format
+    mxfp4_dequant_ref                 every (byte, scale) pair against the e2m1 bit formula times an exact power of
+                                      two in float64, torch.ldexp on the looked-up bf16 table, nibble order by
+                                      planted bytes, the reference's second formulation (stack + view interleave)
 
 The third-party arithmetic underneath (torch.cos/sin/pow/rsqrt, F.linear) is
 PyTorch's, un-pinned by the reference (its README leaves torch unversioned);
@@ -333,3 +336,27 @@ def make_inputs(rows: int, swiglu_rows: int = 0, seed: int = 0, hidden: int = HI
     if swiglu_rows:
         d["swiglu_x"] = (2.0 * torch.randn(swiglu_rows, 2 * hidden, generator=g)).bfloat16()
     return d
+
+
+# ---- MXFP4 checkpoint expansion (weights.py:11-14, 68-117) ----------------------------------------------------------
+
+FP4_VALUES = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0)
+
+
+def mxfp4_dequant_ref(blocks: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """Checkpoint._get_mxfp4_tensor (weights.py:68-117): blocks uint8 [..., G, B], scales uint8 [..., G] ->
+    bf16 [..., G * B * 2]. Byte k of a block gives element 2k from its low nibble and 2k+1 from its high nibble
+    (weights.py:105-110); each element is table[nibble] * 2^(scale - 127) (weights.py:86, 112). The reference forms
+    the product with torch.ldexp on a bf16 tensor, which multiplies by pow(2.0, e) in fp32 and rounds once to bf16;
+    the same two steps are written out here."""
+    assert blocks.dtype == torch.uint8 and scales.dtype == torch.uint8
+    assert blocks.shape[:-1] == scales.shape
+    *prefix, G, B = blocks.shape
+    lut = torch.tensor(FP4_VALUES, dtype=torch.float32)
+    b = blocks.reshape(-1, B).to(torch.int64)
+    vals = torch.empty(b.shape[0], 2 * B, dtype=torch.float32)
+    vals[:, 0::2] = lut[b & 0x0F]
+    vals[:, 1::2] = lut[b >> 4]
+    e = scales.reshape(-1, 1).to(torch.int32) - 127
+    p = torch.pow(torch.tensor(2.0, dtype=torch.float32), e.to(torch.float32))   # fp32: denormal below -126, inf at 128
+    return (vals * p).to(torch.bfloat16).reshape(*prefix, G * B * 2)

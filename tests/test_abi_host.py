@@ -110,3 +110,49 @@ def test_scratch_pool_returns_same_buffer():
     assert a.data_ptr() == b.data_ptr() and a.data_ptr() != c.data_ptr()
     assert scratch_pool.stats()["num_buffers"] == 2
     scratch_pool.clear()
+
+
+def test_checkpoint_names_and_plain_tensors(tmp_path):
+    """Host logic of the checkpoint reader (reference weights.py:17-66): key discovery over several files, the MoE
+    name mapping, plain tensors on the CPU, and no CPU expansion of MXFP4 data."""
+    from safetensors.torch import save_file
+
+    from tritonllm_amd.weights import Checkpoint, _param_names
+
+    assert _param_names("block.0.mlp.mlp1_weight") == ("block.0.mlp.mlp1_weight.blocks", "block.0.mlp.mlp1_weight.scales")
+    assert _param_names("block.35.mlp.mlp2_weight") == ("block.35.mlp.mlp2_weight.blocks", "block.35.mlp.mlp2_weight.scales")
+    assert _param_names("block.36.mlp.mlp2_weight") == "block.36.mlp.mlp2_weight"       # the reference maps 36 blocks
+    assert _param_names("block.3.mlp.mlp1_bias") == "block.3.mlp.mlp1_bias"
+    assert _param_names("block.3.attn.qkv.weight") == "block.3.attn.qkv.weight"
+    assert _param_names("embedding.weight") == "embedding.weight"
+
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(4, 8, generator=g).bfloat16()
+    b = torch.randn(3, generator=g)
+    save_file({"embedding.weight": a}, str(tmp_path / "one.safetensors"))
+    save_file({"block.0.mlp.mlp1_bias": b,
+               "block.0.mlp.mlp1_weight.blocks": torch.zeros(2, 4, 3, 16, dtype=torch.uint8),
+               "block.0.mlp.mlp1_weight.scales": torch.full((2, 4, 3), 127, dtype=torch.uint8)}, str(tmp_path / "two.safetensors"))
+    (tmp_path / "ignored.txt").write_text("not a tensor file")
+    ck = Checkpoint(str(tmp_path), torch.device("cpu"))
+    assert sorted(ck.tensor_name_to_file) == ["block.0.mlp.mlp1_bias", "block.0.mlp.mlp1_weight.blocks", "block.0.mlp.mlp1_weight.scales",
+                                              "embedding.weight"]
+    assert torch.equal(ck.get("embedding.weight"), a)
+    assert torch.equal(ck.get("block.0.mlp.mlp1_bias"), b)
+    dst = torch.empty(3)
+    assert ck.get("block.0.mlp.mlp1_bias", out=dst) is dst and torch.equal(dst, b)
+    with pytest.raises(AssertionError, match="not found"):
+        ck.get("block.1.mlp.mlp1_bias")
+    with pytest.raises(AssertionError, match="not found"):
+        ck.get("block.1.mlp.mlp1_weight")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ck.get("block.0.mlp.mlp1_weight")
+
+
+def test_mxfp4_argument_errors():
+    lib = _lib.lib()
+    assert lib.tllm_mxfp4_dequant_bf16(None, None, None, 0, None) == 0
+    assert lib.tllm_mxfp4_dequant_bf16(None, None, None, 5, None) == -1
+    assert lib.tllm_mxfp4_dequant_bf16(None, None, None, -1, None) == -1
+    assert lib.tllm_mxfp4_dequant_bf16(C.c_void_p(8), C.c_void_p(1), C.c_void_p(16), 5, None) != 0   # blocks not 16-byte aligned
+    assert "aligned" in _err()

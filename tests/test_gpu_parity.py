@@ -723,3 +723,81 @@ def test_attention_block_decode_chain(gpu):
         yr = O.out_residual_ref(tr.view(bs, 4096), w_out, b_out, d["x"])
         close(t, tr.float())
         close(y.view(bs, 2880), yr)
+
+
+# ----------------------------------------------------------------------------------- MXFP4 checkpoint expansion
+def _bits_equal_nan_aware(out, ref):
+    out = out.cpu()
+    nan = torch.isnan(ref)
+    assert torch.equal(torch.isnan(out), nan)
+    assert torch.equal(out.view(torch.int16)[~nan], ref.view(torch.int16)[~nan])
+
+
+def test_mxfp4_every_byte_and_scale(gpu):
+    """All 256 byte values under all 256 scale bytes, bit for bit (denormal products at the low scales, inf at the
+    top, 0 * inf = nan at scale 255 as torch.ldexp gives in the reference)."""
+    blocks = torch.arange(256, dtype=torch.uint8).reshape(1, 16, 16).repeat(256, 1, 1)
+    scales = torch.arange(256, dtype=torch.uint8).reshape(256, 1).repeat(1, 16)
+    out = T.mxfp4_dequant(blocks.to(gpu), scales.to(gpu))
+    assert out.shape == (256, 512) and out.dtype == torch.bfloat16
+    _bits_equal_nan_aware(out, O.mxfp4_dequant_ref(blocks, scales))
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (1, 255), (257, 3), (4, 64, 90), (2, 5, 7, 11)])
+def test_mxfp4_shapes(gpu, shape):
+    g = torch.Generator().manual_seed(sum(shape))
+    blocks = torch.randint(0, 256, (*shape, 16), dtype=torch.uint8, generator=g)
+    scales = torch.randint(100, 140, shape, dtype=torch.uint8, generator=g)
+    out = T.mxfp4_dequant(blocks.to(gpu), scales.to(gpu))
+    assert out.shape == (*shape[:-1], shape[-1] * 32)
+    _bits_equal_nan_aware(out, O.mxfp4_dequant_ref(blocks, scales))
+    # expansion into a caller's buffer, and non-contiguous inputs
+    dst = torch.empty(out.numel(), dtype=torch.bfloat16, device=gpu)
+    res = T.mxfp4_dequant(blocks.to(gpu), scales.to(gpu), out=dst)
+    assert res.data_ptr() == dst.data_ptr() and torch.equal(res, out)
+    if len(shape) >= 2:
+        bt = blocks.to(gpu).transpose(0, 1)
+        st = scales.to(gpu).transpose(0, 1)
+        _bits_equal_nan_aware(T.mxfp4_dequant(bt, st), O.mxfp4_dequant_ref(blocks.transpose(0, 1).contiguous(), scales.transpose(0, 1).contiguous()))
+
+
+def test_mxfp4_empty(gpu):
+    out = T.mxfp4_dequant(torch.empty(0, 3, 16, dtype=torch.uint8, device=gpu), torch.empty(0, 3, dtype=torch.uint8, device=gpu))
+    assert out.shape == (0, 96)
+
+
+def test_mxfp4_moe_weight_shape(gpu):
+    """The gpt-oss-20b mlp1 weight, [32 experts, 5760, 2880] stored as [32, 5760, 90, 16] blocks: one expert against
+    the oracle, the whole tensor through exact scaling (scale + 1 doubles every value) and block independence."""
+    g = torch.Generator(device=gpu).manual_seed(11)
+    blocks = torch.randint(0, 256, (32, 5760, 90, 16), dtype=torch.uint8, device=gpu, generator=g)
+    scales = torch.randint(110, 130, (32, 5760, 90), dtype=torch.uint8, device=gpu, generator=g)
+    out = T.mxfp4_dequant(blocks, scales)
+    assert out.shape == (32, 5760, 2880)
+    for e in (0, 31):
+        _bits_equal_nan_aware(out[e], O.mxfp4_dequant_ref(blocks[e].cpu(), scales[e].cpu()))
+    out2 = T.mxfp4_dequant(blocks, scales + 1)
+    assert torch.equal(out2, out * 2)
+    del out2
+    # a reversed copy of the blocks expands to the reversed rows
+    flip = T.mxfp4_dequant(blocks.flip(1), scales.flip(1))
+    assert torch.equal(flip, out.flip(1))
+
+
+def test_checkpoint_mxfp4_on_gpu(gpu, tmp_path):
+    from safetensors.torch import save_file
+
+    g = torch.Generator().manual_seed(21)
+    blocks = torch.randint(0, 256, (4, 96, 6, 16), dtype=torch.uint8, generator=g)
+    scales = torch.randint(115, 128, (4, 96, 6), dtype=torch.uint8, generator=g)
+    bias = torch.randn(4, 96, generator=g).bfloat16()
+    save_file({"block.2.mlp.mlp2_weight.blocks": blocks, "block.2.mlp.mlp2_weight.scales": scales}, str(tmp_path / "a.safetensors"))
+    save_file({"block.2.mlp.mlp2_bias": bias}, str(tmp_path / "b.safetensors"))
+    ck = T.Checkpoint(str(tmp_path), gpu)
+    w = ck.get("block.2.mlp.mlp2_weight")
+    assert w.is_cuda and w.shape == (4, 96, 192)
+    _bits_equal_nan_aware(w, O.mxfp4_dequant_ref(blocks, scales))
+    b = ck.get("block.2.mlp.mlp2_bias")
+    assert b.is_cuda and torch.equal(b.cpu(), bias)
+    dst = torch.empty(4, 96, 192, dtype=torch.bfloat16, device=gpu)
+    assert ck.get("block.2.mlp.mlp2_weight", out=dst) is dst and torch.equal(dst, w)

@@ -305,3 +305,54 @@ def test_attention_decode_ref_pins():
     ke = k[:, :1].expand(-1, n_keys, -1, -1)
     out = O.attention_decode_ref(q, ke, v, torch.full((6,), -1e4), 0.25, None, 39).view(bs, n_kv, groups, hd)
     torch.testing.assert_close(out, v.float().mean(dim=1)[:, :, None, :].expand(-1, -1, groups, -1), rtol=1e-5, atol=1e-6)
+
+
+def _e2m1(nib: int) -> float:
+    """OCP MX e2m1: sign bit 3, two exponent bits (bias 1), one mantissa bit; exponent 0 is subnormal (0 or 0.5)."""
+    s, e, m = nib >> 3, (nib >> 1) & 3, nib & 1
+    mag = 0.5 * m if e == 0 else (1 + 0.5 * m) * 2.0 ** (e - 1)
+    return -mag if s else mag
+
+
+def test_mxfp4_dequant_ref_pins():
+    # the table is the e2m1 format
+    assert [_e2m1(n) for n in range(16)] == list(O.FP4_VALUES)
+    # every (byte, scale) pair with a finite result: element 2k = low nibble, 2k+1 = high nibble, times an exact power of two
+    bytes_ = torch.arange(256, dtype=torch.uint8)
+    blocks = bytes_.reshape(1, 16, 16).repeat(255, 1, 1)               # [scale, G=16, B=16]: all 256 byte values per scale
+    scales = torch.arange(255, dtype=torch.uint8).reshape(255, 1).repeat(1, 16)
+    got = O.mxfp4_dequant_ref(blocks, scales)
+    assert got.shape == (255, 512) and got.dtype == torch.bfloat16
+    want = np.empty((255, 512), dtype=np.float64)
+    for s in range(255):
+        for byte in range(256):
+            want[s, 2 * byte] = _e2m1(byte & 15) * 2.0 ** (s - 127)
+            want[s, 2 * byte + 1] = _e2m1(byte >> 4) * 2.0 ** (s - 127)
+    # finite products are exactly representable in bf16 (one mantissa bit, exponents -128..129); 6 * 2^127 and
+    # 4 * 2^127 overflow fp32 / bf16 to inf
+    bf16_max = float(torch.finfo(torch.bfloat16).max)
+    want_t = torch.from_numpy(want)
+    finite = want_t.abs() <= bf16_max
+    assert torch.equal(got.double()[finite], want_t[finite])
+    assert torch.isinf(got.double()[~finite]).all() and (torch.sign(got.double()[~finite]) == torch.sign(want_t[~finite])).all()
+    assert (~finite).sum() > 0
+    # signed zeros survive
+    assert torch.signbit(O.mxfp4_dequant_ref(torch.full((1, 16), 0x88, dtype=torch.uint8), torch.tensor([127], dtype=torch.uint8))).all()
+    # torch.ldexp on the looked-up bf16 values, the library call the reference makes (weights.py:112), scale 255 included
+    blocks = torch.randint(0, 256, (3, 7, 16), dtype=torch.uint8, generator=torch.Generator().manual_seed(5))
+    scales = torch.randint(0, 256, (3, 7), dtype=torch.uint8, generator=torch.Generator().manual_seed(6))
+    scales[0, 0] = 255
+    scales[0, 1] = 0
+    lut = torch.tensor(O.FP4_VALUES, dtype=torch.bfloat16)
+    # second formulation (weights.py:119-139): stack (lo, hi) on a new last axis and flatten it
+    idx = torch.stack((blocks & 0x0F, blocks >> 4), dim=-1).reshape(3, 7, 32).int()
+    alt = torch.ldexp(lut[idx], (scales.int() - 127).unsqueeze(-1)).reshape(3, 7 * 32)
+    got = O.mxfp4_dequant_ref(blocks, scales)
+    assert got.shape == alt.shape
+    assert torch.equal(got.view(torch.int16)[~torch.isnan(alt)], alt.view(torch.int16)[~torch.isnan(alt)])
+    assert torch.equal(torch.isnan(got), torch.isnan(alt)) and torch.isnan(alt).any()    # 0 * 2^128 = nan in both
+    # nibble order by a planted byte: 0x21 -> (0.5, 1.0)
+    one = torch.zeros(1, 16, dtype=torch.uint8)
+    one[0, 3] = 0x21
+    out = O.mxfp4_dequant_ref(one, torch.tensor([128], dtype=torch.uint8))
+    assert out[6].item() == 1.0 and out[7].item() == 2.0 and out.count_nonzero() == 2

@@ -7,6 +7,7 @@ from .ops import (
     attention_decode,
     embedding_forward,
     linear_qkv_forward,
+    mxfp4_dequant,
     out_residual_decode_forward,
     qkv_decode_forward,
     qkv_rope_cache_decode_forward,
@@ -21,11 +22,12 @@ from .ops import (
     unembedding_decode_fp8_forward,
     unembedding_forward,
 )
+from .weights import Checkpoint
 from .yarn import YarnParams, gpt_oss_yarn
 
 __all__ = [
-    "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
-    "attention_decode", "embedding_forward", "linear_qkv_forward", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
+    "Checkpoint", "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
+    "attention_decode", "embedding_forward", "linear_qkv_forward", "mxfp4_dequant", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
     "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu", "UnEmbedding", "unembedding_decode_forward", "unembedding_decode_argmax_forward",
     "unembedding_decode_fp8_forward", "unembedding_decode_fp8_argmax_forward", "unembedding_forward",
 ]

@@ -526,3 +526,27 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: t
                                           work.data_ptr() if work is not None else None, nbytes, _stream())
     check(rc, "attention_decode")
     return o.view(bs, 1, n_heads * 64)
+
+
+def mxfp4_dequant(blocks: torch.Tensor, scales: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Expand MXFP4 checkpoint data to bf16 (Checkpoint._get_mxfp4_tensor, weights.py:68-117).
+
+    ``blocks`` uint8 ``[..., G, 16]`` holds 32 e2m1 values per 16 bytes, low nibble first; ``scales`` uint8
+    ``[..., G]`` holds the shared power-of-two exponent, biased by 127. Returns ``[..., G * 32]`` bf16; ``out``, if
+    given, must be a contiguous bf16 tensor of that many elements (it is filled in place, so a caller can expand
+    straight into a slice of a preallocated parameter)."""
+    _on_gpu(blocks, scales, out)
+    assert blocks.dtype == torch.uint8 and scales.dtype == torch.uint8, "MXFP4 blocks and scales are uint8"
+    assert blocks.shape[:-1] == scales.shape, f"{blocks.shape=} does not match {scales.shape=}"
+    assert blocks.shape[-1] == 16, "an MXFP4 block is 16 bytes"
+    *prefix, G, B = blocks.shape
+    blocks = blocks.contiguous()
+    scales = scales.contiguous()
+    n_blocks = scales.numel()
+    shape = (*prefix, G * B * 2)
+    if out is None:
+        out = torch.empty(shape, dtype=_BF16, device=blocks.device)
+    else:
+        assert out.dtype == _BF16 and out.is_contiguous() and out.numel() == n_blocks * 32, "out must be contiguous bf16 of 32 values per block"
+    check(lib().tllm_mxfp4_dequant_bf16(blocks.data_ptr(), scales.data_ptr(), out.data_ptr(), n_blocks, _stream()), "mxfp4_dequant")
+    return out.view(shape) if out.shape != torch.Size(shape) else out
