@@ -639,16 +639,16 @@ def test_unembedding_full_vocabulary_and_module(gpu, monkeypatch):
 
 
 # ----------------------------------------------------------------------------------- decode attention
-def _attn_case(gpu, batch_size, num_keys, sliding_window, start_q, start_dtype=torch.int32, seed=0, with_sinks=True, groups=8):
+def _attn_case(gpu, batch_size, num_keys, sliding_window, start_q, start_dtype=torch.int32, seed=0, with_sinks=True, groups=8, kv_heads=8):
     g = torch.Generator().manual_seed(seed)
-    q = torch.randn(batch_size, 1, 8, groups, 64, generator=g).bfloat16()
-    k = torch.randn(batch_size, num_keys, 8, 64, generator=g).bfloat16()
-    v = torch.randn(batch_size, num_keys, 8, 64, generator=g).bfloat16()
-    sinks = torch.randn(8 * groups, generator=g).bfloat16() if with_sinks else None
+    q = torch.randn(batch_size, 1, kv_heads, groups, 64, generator=g).bfloat16()
+    k = torch.randn(batch_size, num_keys, kv_heads, 64, generator=g).bfloat16()
+    v = torch.randn(batch_size, num_keys, kv_heads, 64, generator=g).bfloat16()
+    sinks = torch.randn(kv_heads * groups, generator=g).bfloat16() if with_sinks else None
     o1 = T.attention_decode(q.to(gpu), k.to(gpu), v.to(gpu), sinks.to(gpu) if with_sinks else None, 0.125, sliding_window,
                             torch.tensor([start_q], dtype=start_dtype, device=gpu))
     o2 = O.attention_decode_ref(q, k, v, sinks, 0.125, sliding_window, start_q)
-    assert o1.shape == (batch_size, 1, 8 * groups * 64) and o1.dtype == torch.bfloat16
+    assert o1.shape == (batch_size, 1, kv_heads * groups * 64) and o1.dtype == torch.bfloat16
     # the reference's own bar (attention_tt_decode.py:429, 454) ...
     torch.testing.assert_close(o1.float().cpu(), o2.bfloat16().float(), atol=1e-2, rtol=1e-1)
     # ... and the tolerance of the other bf16 outputs of this library
@@ -690,6 +690,29 @@ def test_attention_decode_edges(gpu):
     close(o1, O.attention_decode_ref(q, kc[:, :300], vc[:, :300], sinks, 0.125, None, 299))
     with pytest.raises(AssertionError):
         T.attention_decode(q.to(gpu).expand(-1, 2, -1, -1, -1), kc.to(gpu), vc.to(gpu), sinks.to(gpu), 0.125, None, torch.tensor([1], device=gpu))
+
+
+@pytest.mark.parametrize("case", [
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8191),                 # 32 splits of 256 keys
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8000, start_dtype=torch.int64),   # ragged last split
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=100),                  # most splits hold no key at all
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=0),                    # one key
+    dict(batch_size=16, num_keys=8192, sliding_window=4096, start_q=7000),                # window under the split planning
+    dict(batch_size=256, num_keys=300, sliding_window=None, start_q=299),                 # one split: written straight to the output
+    dict(batch_size=256, num_keys=300, sliding_window=None, start_q=280, with_sinks=False),
+    dict(batch_size=32, num_keys=2048, sliding_window=None, start_q=2047, kv_heads=4, groups=2),   # four wavefronts, two heads each
+    dict(batch_size=64, num_keys=1024, sliding_window=None, start_q=1000, kv_heads=2, groups=16),  # widest group
+], ids=lambda c: "-".join(f"{k[0]}{v}" for k, v in c.items() if not isinstance(v, torch.dtype)))
+def test_attention_decode_row_workgroups(gpu, case):
+    """Large batch x context: the workgroup shape with one wavefront per KV head (chosen inside the library from
+    batch, heads and context; these cases all fall on it)."""
+    from tritonllm_amd._lib import lib
+    c = dict(case)
+    kvh = c.get("kv_heads", 8)
+    splits = lib().tllm_attention_decode_splits(c["batch_size"], kvh, c["num_keys"], c["sliding_window"] or 0)
+    ctx = min(c["sliding_window"] or c["num_keys"], c["num_keys"])
+    assert c["batch_size"] * splits >= 224 and ctx >= 256 * splits, "case no longer selects the row-shaped workgroups"
+    _attn_case(gpu, seed=11 + c["start_q"], **c)
 
 
 def test_attention_block_decode_chain(gpu):

@@ -6,8 +6,15 @@
 //   out[h]   = sum_n exp(s[h, n] - m) v[n] / (sum_n exp(s[h, n] - m) + exp(sink[h] - m)),   m = max(sink[h], max_n s[h, n])
 //
 // The reference runs one program per query head, so the G heads of a group each read the same K and V; here a
-// workgroup takes a (batch row, KV head, context split) and serves all G heads from one pass over K and V:
-//   * four wavefronts take 32-key blocks of the split in turn, each with its own running (max, sum, accumulator);
+// wavefront serves all G heads of a KV head from one pass over K and V, in one of two workgroup shapes:
+//   * ROWS (large batch x context): a workgroup takes a (batch row, context split) and has one wavefront per KV head,
+//     each walking the split's 32-key blocks in order. Together the wavefronts read whole cache rows (all KV heads
+//     of a token are adjacent in memory), so the workgroup streams one contiguous range of K and one of V; with
+//     nontemporal loads that pattern measures 6.8 TB/s on its own, where one-KV-head-per-workgroup streams stop at
+//     5.2 TB/s (128-byte pieces at a 1 KB stride, the sibling heads arriving from other workgroups at other times);
+//   * HEAD (few batch rows): a workgroup takes a (batch row, KV head, context split); four wavefronts take the
+//     split's blocks in turn, each with its own running (max, sum, accumulator), and meet once at the end through
+//     LDS. This shape yields n_kv_heads times more workgroups, which is what fills the machine at batch 1;
 //   * S^T = K . Q^T on v_mfma_f32_16x16x32_bf16 with the keys on M: K rows are K-contiguous in memory, so a lane
 //     loads its 16 bytes of a key row straight into operand layout; Q sits in registers as the B operand;
 //   * the accumulator layout of S^T (lane = head, registers = keys) IS the A-operand layout of P for O = P . V when
@@ -15,8 +22,8 @@
 //     rows are d-contiguous, goes through a wavefront-private LDS tile and is gathered in that same key order;
 //   * the per-head rescale factor exp(m_old - m_new) lives in the S^T layout and is fetched into the O layout
 //     (registers = heads) by ds_bpermute;
-//   * wavefronts meet once at the end through LDS; with more than one context split the workgroups leave
-//     (max, sum, accumulator) in a workspace and a second small kernel folds them and the sink.
+//   * with more than one context split the workgroups leave (max, sum, accumulator) in a workspace and a second
+//     small kernel folds them and the sink.
 // start_q is read from device memory (int32 or int64), so a captured graph follows the growing context.
 #include "common.h"
 
@@ -39,7 +46,8 @@ struct AttnArgs {
 };
 
 namespace {
-constexpr int AW = 4;                 // wavefronts per workgroup
+constexpr int AW = 4;                 // wavefronts per workgroup, HEAD shape
+constexpr int RW = 8;                 // most wavefronts (= KV heads) per workgroup, ROWS shape
 constexpr int VROW = 128 + 16;        // V tile row in LDS: 64 bf16 + padding, bytes
 constexpr int VTILE = 32 * VROW;
 constexpr float kNegBig = -1.0e30f;
@@ -50,14 +58,16 @@ __device__ __forceinline__ int attn_start_q(const AttnArgs& a) {
   return a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
 }
 
-__global__ __launch_bounds__(AW * 64) void attn_decode_kernel(AttnArgs a) {
-  __shared__ __align__(16) unsigned char vt[AW * VTILE];
-  __shared__ float s_m[AW][16], s_l[AW][16];
-  __shared__ float s_acc[AW][16][64 + 1];
+template <bool ROWS>
+__global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(AttnArgs a) {
+  __shared__ __align__(16) unsigned char vt[(ROWS ? RW : AW) * VTILE];
+  __shared__ float s_m[ROWS ? 1 : AW][16], s_l[ROWS ? 1 : AW][16];
+  __shared__ float s_acc[ROWS ? 1 : AW][ROWS ? 1 : 16][64 + 1];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, g = lane >> 4;
-  const int kvh = blockIdx.x / a.splits, split = blockIdx.x - kvh * a.splits;
+  const int kvh = ROWS ? wave : blockIdx.x / a.splits;
+  const int split = ROWS ? blockIdx.x : blockIdx.x - kvh * a.splits;
   const int64_t b = blockIdx.y;
   const int G = a.group;
   const int n_q_heads = a.n_kv_heads * G;
@@ -94,6 +104,11 @@ __global__ __launch_bounds__(AW * 64) void attn_decode_kernel(AttnArgs a) {
   // Rows past the end of the split are clamped to its last key (finite values; their probabilities are zeroed).
   // Addressing is a block base (uniform) plus a 32-bit lane offset: row * token stride + a lane constant.
   const unsigned ts_b = static_cast<unsigned>(a.kv_ts) * 2u;   // token stride, bytes (a 32-key block spans < 4 GB)
+  // The ROWS stream is read once and is far larger than the caches: nontemporal. The HEAD shape serves short
+  // contexts, where the cache lines of a token are shared with sibling workgroups and may still be cache-resident.
+  auto ld = [](const unsigned char* p) {
+    return ROWS ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p)) : *reinterpret_cast<const bf16x8*>(p);
+  };
   bf16x8 ka[2][2], vr[4];
   auto load_block = [&](int k0) {
     const int last = s_hi - k0 - 1;                            // last valid row of the block (>= 31 except in the final one)
@@ -103,19 +118,21 @@ __global__ __launch_bounds__(AW * 64) void attn_decode_kernel(AttnArgs a) {
     for (int kb = 0; kb < 2; ++kb) {
       const int r = 16 * kb + r16;
       const unsigned off = static_cast<unsigned>(r < last ? r : last) * ts_b + 16u * g;
-      ka[kb][0] = *reinterpret_cast<const bf16x8*>(kb0 + off);
-      ka[kb][1] = *reinterpret_cast<const bf16x8*>(kb0 + off + 64);
+      ka[kb][0] = ld(kb0 + off);
+      ka[kb][1] = ld(kb0 + off + 64);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = i * 64 + lane;
       const int r = c >> 3;
-      vr[i] = *reinterpret_cast<const bf16x8*>(vb0 + static_cast<unsigned>(r < last ? r : last) * ts_b + 16u * (c & 7));
+      vr[i] = ld(vb0 + static_cast<unsigned>(r < last ? r : last) * ts_b + 16u * (c & 7));
     }
   };
 
-  if (nblk > 0 && wave < nblk) load_block(s_lo + 32 * wave);
-  for (int blk = wave; blk < nblk; blk += AW) {
+  constexpr int STEP = ROWS ? 1 : AW;                          // ROWS: every wavefront walks all blocks (of its own KV head)
+  const int first = ROWS ? 0 : wave;
+  if (first < nblk) load_block(s_lo + 32 * first);
+  for (int blk = first; blk < nblk; blk += STEP) {
     const int k0 = s_lo + 32 * blk;
     // ---- S^T for the block's two 16-key halves
     f32x4_t st[2];
@@ -132,7 +149,7 @@ __global__ __launch_bounds__(AW * 64) void attn_decode_kernel(AttnArgs a) {
     }
     // The next block's loads go out before this one's arithmetic. Unconditional (a load under a branch makes the
     // compiler wait for it where the paths join): the last round simply requests its own block again.
-    load_block(s_lo + 32 * (blk + AW < nblk ? blk + AW : blk));
+    load_block(s_lo + 32 * (blk + STEP < nblk ? blk + STEP : blk));
 
     // ---- online softmax for head r16: this lane holds keys k0 + 16 kb + 4 g + i
     float sc[8];
@@ -193,7 +210,37 @@ __global__ __launch_bounds__(AW * 64) void attn_decode_kernel(AttnArgs a) {
     __builtin_amdgcn_wave_barrier();
   }
 
-  // ---- the four wavefronts meet: (max, sum) per head, accumulator per (head, d)
+  if constexpr (ROWS) {
+    // ---- each wavefront owns its heads outright: O sits in lane (d = 16 nb + r16), registers = heads 4 g + i; the
+    // (max, sum) of head h sit in the lanes with r16 == h
+    float* p = a.part + ((static_cast<int64_t>(split) * gridDim.y + b) * n_q_heads + static_cast<int64_t>(kvh) * G) * PART;
+    if (a.splits > 1 && g == 0 && r16 < G) {
+      p[r16 * PART + 64] = m_run;
+      p[r16 * PART + 65] = l_run;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int hh = 4 * g + i;
+      const float m_h = __shfl(m_run, hh, 64), l_h = __shfl(l_run, hh, 64);
+      if (hh >= G) continue;
+      if (a.splits > 1) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) p[hh * PART + 16 * nb + r16] = acc[nb][i];
+      } else {
+        const int head = kvh * G + hh;
+        const float sink = a.sinks ? static_cast<float>(a.sinks[head]) : 0.f;
+        const float m_f = fmaxf(m_h, sink);
+        const float f = __expf(m_h - m_f);
+        const float z = l_h * f + __expf(sink - m_f);
+        bf16* orow = a.out + b * a.out_rs + static_cast<int64_t>(head) * 64;
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) orow[16 * nb + r16] = static_cast<bf16>(acc[nb][i] * f / z);
+      }
+    }
+    return;
+  }
+
+  // ---- HEAD: the four wavefronts meet: (max, sum) per head, accumulator per (head, d)
   if (g == 0) {
     s_m[wave][r16] = m_run;
     s_l[wave][r16] = l_run;
@@ -280,21 +327,38 @@ __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(AttnArgs a, int 
 
 using namespace tllm;
 
-// Context splits, from measurements at B = 1 and 8, contexts 1K - 32K: first enough workgroups to give every CU one
-// (with one batch row and eight KV heads that alone asks for 32 splits), beyond that about 1024 keys per workgroup
-// (eight 32-key blocks per wavefront: fewer and the per-workgroup start-up dominates, more and too few wavefronts
-// are resident to cover the load latency); never less than 128 keys per split. A sliding window bounds the context.
-extern "C" int tllm_attention_decode_splits(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
+// Workgroup shape and context splits, from measurements at B = 1 .. 32, contexts 1K - 128K.
+// ROWS (a workgroup per (batch row, split), one wavefront per KV head) streams faster but yields n_kv_heads times
+// fewer workgroups, each wavefront walking its blocks one after the other: it is taken when batch x splits still
+// gives every CU a workgroup with at least 256 keys per split (B = 8: 106 -> 87 us at 32K context, but 17 -> 21 us
+// at 4K, where the splits would be 128 keys; B = 32 at 4K: 56 -> 48 us; B = 2 at 32K: 33 -> 42 us). Splits: first enough
+// workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) / 2048 (HEAD) keys per workgroup, never less than
+// 128 keys per split.
+// A sliding window bounds the context.
+struct AttnPlan { bool rows; int splits; };
+
+static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
   const int64_t ctx = (window > 0 && window < n_kv_ctx) ? window : n_kv_ctx;
-  const int64_t units = batch * n_kv_heads > 0 ? batch * n_kv_heads : 1;
-  const int64_t fill = (256 + units - 1) / units;
-  const int64_t by_work = (ctx + 1023) / 1024;
-  int64_t s = fill > by_work ? fill : by_work;
   const int64_t cap = (ctx + 127) / 128;
-  if (s > cap) s = cap;
-  if (s < 1) s = 1;
-  if (s > 64) s = 64;
-  return (int)s;
+  auto splits_for = [&](int64_t units, int64_t keys_per_wg) {
+    const int64_t by_work = (ctx + keys_per_wg - 1) / keys_per_wg;
+    units = units > 0 ? units : 1;
+    const int64_t fill = (256 + units - 1) / units;
+    int64_t s = fill > by_work ? fill : by_work;
+    if (s > cap) s = cap;
+    if (s < 1) s = 1;
+    if (s > 64) s = 64;
+    return static_cast<int>(s);
+  };
+  if (n_kv_heads >= 2 && n_kv_heads <= RW) {
+    const int s = splits_for(batch, 1024);
+    if (batch * s >= 224 && ctx >= 256 * static_cast<int64_t>(s)) return {true, s};
+  }
+  return {false, splits_for(batch * n_kv_heads, 2048)};
+}
+
+extern "C" int tllm_attention_decode_splits(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
+  return attn_plan(batch, n_kv_heads, n_kv_ctx, window).splits;
 }
 
 extern "C" int64_t tllm_attention_decode_workspace_bytes(int64_t batch, int n_q_heads, int n_kv_heads, int64_t n_kv_ctx, int window) {
@@ -334,14 +398,18 @@ extern "C" int tllm_attention_decode_bf16(const void* q, const void* k, const vo
   a.group = group;
   a.window = window;
   a.sm_scale = sm_scale;
-  a.splits = tllm_attention_decode_splits(batch, n_kv_heads, n_kv_ctx, window);
+  const AttnPlan plan = attn_plan(batch, n_kv_heads, n_kv_ctx, window);
+  a.splits = plan.splits;
   const int64_t need = tllm_attention_decode_workspace_bytes(batch, n_kv_heads * group, n_kv_heads, n_kv_ctx, window);
   TLLM_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 4 == 0), TLLM_E_ARG,
                "attention_decode: workspace of %lld bytes needed (tllm_attention_decode_workspace_bytes), got %lld", (long long)need,
                (long long)workspace_bytes);
   a.part = static_cast<float*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)(n_kv_heads * a.splits), (unsigned)batch), dim3(AW * 64), 0, st, a);
+  if (plan.rows)
+    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3((unsigned)a.splits, (unsigned)batch), dim3(n_kv_heads * 64), 0, st, a);
+  else
+    hipLaunchKernelGGL(attn_decode_kernel<false>, dim3((unsigned)(n_kv_heads * a.splits), (unsigned)batch), dim3(AW * 64), 0, st, a);
   int rc = check_launch("attention_decode");
   if (rc != TLLM_OK || a.splits == 1) return rc;
   hipLaunchKernelGGL(attn_decode_reduce_kernel, dim3((unsigned)(n_kv_heads * group), (unsigned)batch), dim3(64), 0, st, a, (int)batch);
