@@ -4,33 +4,35 @@
 //
 // Tiling for 256 CUs: a workgroup computes a 128-token x 320-column tile (five whole heads),
 // so T = 2048 is exactly 16 x 16 = 256 tiles -- one per CU, no tail wave -- and T = 8192 is
-// exactly four per CU. Four wavefronts form a 2 x 2 grid; each owns 64 x 160 of the tile as
-// 2 x 5 v_mfma_f32_32x32x16_bf16 blocks (160 fp32 accumulators per lane) and reads 7 operand
-// fragments from LDS per 10 MFMAs. K is walked in slices of 64 (one 128-byte line per row) through
+// exactly four per CU. Eight wavefronts form a 4 x 2 grid (two per SIMD); each owns 32 x 160 of the tile as
+// 1 x 5 v_mfma_f32_32x32x16_bf16 blocks (80 fp32 accumulators per lane) and reads 6 operand
+// fragments from LDS per 5 MFMAs. K is walked in slices of 64 (one 128-byte line per row) through
 // two LDS stages filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers,
 // no ds_write). Such a load puts the 64 lanes' 16-byte chunks at consecutive LDS addresses, so rows
 // cannot be padded; instead the chunk order inside each row is XOR-swizzled with the row index --
 // applied by choosing which *global* chunk a lane fetches -- and the fragment reads undo it, which
 // keeps the 128-bit fragment reads of 16 consecutive rows conflict-free.
-// With one tile per CU (one wavefront per SIMD) nothing but the kernel's own schedule overlaps anything:
+// With one tile per CU nothing but the kernel's own schedule overlaps anything:
 //   * the one barrier per slice sits before the slice's last k16 step; the stage just finished is handed to
-//     the slice after next, whose loads go out one per MFMA behind that step and the next (never fourteen
-//     in a row: a CU's load queue is bounded and a wavefront that overflows it stalls, MFMAs included);
+//     the slice after next, whose loads go out one per MFMA behind that step and the next (never all in a row:
+//     a CU's load queue is bounded and a wavefront that overflows it stalls, MFMAs included);
 //   * the fragment reads of the next k16 step are pinned between the MFMAs of the current one
-//     (sched_group_barrier): hoisted to the top of the iteration, as the compiler does by itself, the four
-//     wavefronts read their 112 KB per slice in one burst with no MFMA running;
+//     (sched_group_barrier): hoisted to the top of the iteration, as the compiler does by itself, the
+//     wavefronts read a slice's fragments in one burst with no MFMA running;
 //   * an L2 miss still costs more than a slice of MFMAs and LDS has no room for a third stage, so
 //     three slices ahead every workgroup touches (one dword per line) its share of the lines its
-//     XCD's tiles are going to need, which pulls them into that XCD's L2 in time;
-//   * measured with cycle stamps per k16 step (one build with the stamps compiled in), per slice of 64:
-//     the two steps that only multiply take ~375 cycles each (320 of MFMAs); the two that also carry load
-//     instructions take 590 and 715 -- every load instruction holds the wavefront 35-50 cycles, because the
-//     CU's one address unit serves the four wavefronts' 1 KB loads at ~16 cycles apiece and they all come at
-//     once; waits for the look-ahead loads and at the barrier add ~180. 2240 cycles for 1280 of MFMAs, at a
-//     shader clock of 1.83-1.92 GHz under this load (the published peak assumes 2.4 GHz).
-//     LDS is not the limit (a microbenchmark reads > 400 B/clk/CU with 128-bit reads). Tried and measured, no
-//     better: four extra wavefronts that only load (the multipliers then wait at the barrier for data that is
-//     requested in one burst, 71-75 us), and the same with K slices of 32 in a four-stage ring (77 us).
+//     XCD's tiles are going to need, which pulls them into that XCD's L2 in time (86 % L2 hits counted).
+// Where the time goes at T = 2048 (66 us; builds with parts of the loop compiled out): the MFMAs, barriers,
+// prologue and epilogue alone take 43 us (30 us of MFMAs at the 1.9 GHz this load clocks at), adding the
+// fragment reads 55 us, the global->LDS loads alone (no MFMA, no fragment read) 56 us, everything 66 us. The
+// loads are the wall: with two stages the loads of slice i+2 cannot start before slice i has been read by
+// everyone and must have landed before slice i+1 has been, so every slice pays its 56 KB through the CU's
+// 64 B/clk address unit (~900 cycles) plus an L2 round trip inside one slice's 1280 cycles of MFMAs, and a third
+// stage of this tile does not fit (3 x 56 KB > 160 KB). Measured without gain: the 2 x 2 grid of 64 x 160
+// wavefronts this kernel started with (70 us: one wavefront per SIMD, nothing to cover a stalled load issue),
+// pairs of 64 x 160 wavefronts taking alternate k16 steps (fewer fragment reads, 68 us), four extra wavefronts that
+// only load (71-75 us), K slices of 32 in a four-stage ring (77 us), other spreads of the loads over the steps and
+// other prefetch distances (+-1 us).
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
@@ -70,8 +72,7 @@ constexpr int SMEM = NS * STAGE + CS_BYTES;
 static_assert(BM * OROW * 2 <= NS * STAGE, "the epilogue's output image reuses the stage ring");
 static_assert(SMEM <= 160 * 1024, "LDS per workgroup");
 constexpr int BLOCKS = STAGE / 1024;      // 1 KiB blocks per stage
-constexpr int LPW = BLOCKS / 4;           // load instructions per wavefront per stage
-static_assert(KS % 2 == 0 && BLOCKS % 4 == 0 && CHUNKS == 8 && NS == 2, "the schedule and the swizzle below are written for BK = 64, two stages");
+static_assert(KS % 2 == 0 && BLOCKS % 8 == 0 && CHUNKS == 8 && NS == 2, "the schedule and the swizzle below are written for BK = 64, two stages");
 }  // namespace
 
 // Chunk swizzle of LDS row r: the 16-byte chunk c of the row is stored at chunk position c ^ swz(r).
@@ -92,7 +93,19 @@ __device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
   }
 }
 
-__global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
+// WROWS wavefront rows x 2 wavefront columns: 4 x 2 (two wavefronts per SIMD, 32 x 160 each) is what is launched;
+// 2 x 2 (one per SIMD, 64 x 160 each) compiles from the same source.
+template <int WROWS>
+__global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
+  constexpr int NW = WROWS * 2;             // wavefronts
+  constexpr int NT = NW * 64;               // threads
+  constexpr int MB = BM / (32 * WROWS);     // 32-token blocks per wavefront
+  constexpr int LPW = BLOCKS / NW;          // load instructions per wavefront per stage
+  constexpr int NMF = MB * 5;               // MFMAs per k16 step
+  constexpr int NRD = MB + 5;               // fragment reads per k16 step
+  constexpr int NL_LAST = LPW < NMF ? LPW : NMF;   // loads handed out behind a slice's last step ...
+  constexpr int NL_FIRST = LPW - NL_LAST;          // ... and behind the next slice's first step
+  static_assert(NL_FIRST <= NMF, "a slice's loads fit behind two k16 steps");
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -156,7 +169,8 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   // 72 lanes of one load. Nothing waits for these loads; they only pull the lines into the XCD's L2.
   // Every wavefront issues exactly one such load per slice (18 working lanes each; idle lanes and
   // unswizzled launches re-touch a line that is needed anyway), so the wait counts below are constants.
-  const int tch = lane < 18 ? wave * 18 + lane : 72;
+  constexpr int TPW = 72 / NW;                        // touch lanes per wavefront
+  const int tch = lane < TPW ? wave * TPW + lane : 72;
   const unsigned char* touch_ptr = reinterpret_cast<const unsigned char*>(src[0]);
   if (share_q >= 0 && tch < 72) {
     if (tch < 32) {
@@ -188,27 +202,27 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
                                        (__attribute__((address_space(3))) void*)(dst + blk_off[j]), 16, 0, 0);
   };
 
-  f32x16 acc[2][5];
+  f32x16 acc[MB][5];
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb)
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int nb = 0; nb < 5; ++nb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
 
   // fragment addressing: byte offset of (row, chunk c) inside a stage is row*LROW + ((c ^ swz(row)) << 4)
-  const int fa_row = 64 * wm + l32, fb_row = BM + 160 * wn + l32;
-  int fa_off[KS][2], fb_off[KS][5];                     // [k16 step within the slice][block]
+  const int fa_row = 32 * MB * wm + l32, fb_row = BM + 160 * wn + l32;
+  int fa_off[KS][MB], fb_off[KS][5];                     // [k16 step within the slice][block]
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) fa_off[kk][mb] = (fa_row + 32 * mb) * LROW + (((2 * kk + lh) ^ swz(fa_row + 32 * mb)) << 4);
+    for (int mb = 0; mb < MB; ++mb) fa_off[kk][mb] = (fa_row + 32 * mb) * LROW + (((2 * kk + lh) ^ swz(fa_row + 32 * mb)) << 4);
 #pragma unroll
     for (int nb = 0; nb < 5; ++nb) fb_off[kk][nb] = (fb_row + 32 * nb) * LROW + (((2 * kk + lh) ^ swz(fb_row + 32 * nb)) << 4);
   }
-  auto load_frags = [&](const unsigned char* st, int kk, bf16x8 (&fa)[2], bf16x8 (&fb)[5]) {
+  auto load_frags = [&](const unsigned char* st, int kk, bf16x8 (&fa)[MB], bf16x8 (&fb)[5]) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(st + fa_off[kk][mb]);
+    for (int mb = 0; mb < MB; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(st + fa_off[kk][mb]);
 #pragma unroll
     for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(st + fb_off[kk][nb]);
   };
@@ -227,17 +241,25 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   //   * a CU takes only so many loads into its queue and a wavefront that issues one more stalls, MFMAs
   //     included (there is one wavefront per SIMD), until the queue has drained that far; fourteen loads in a
   //     row do exactly that. Handed out one per MFMA (32 cycles) they never find the queue full.
-  bf16x8 fa[2][2], fb[2][5];
+  bf16x8 fa[2][MB], fb[2][5];
+  auto read_frag = [&](int cur, const unsigned char* nst, int nkk, int i) {   // fragment i of the next step: activations first
+    if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nst + fa_off[nkk][i < MB ? i : 0]);
+    else fb[cur ^ 1][i - MB] = *reinterpret_cast<const bf16x8*>(nst + fb_off[nkk][i - MB]);
+  };
   auto step = [&](int cur, const unsigned char* nst, int nkk, int lit, int j0, int n) {
 #pragma unroll
-    for (int m = 0; m < 10; ++m) {
+    for (int m = 0; m < NMF; ++m) {
       const int mb = m / 5, nb = m % 5;
       acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][nb], fa[cur][mb], acc[mb][nb], 0, 0, 0);   // weights on M, tokens on N
-      if (m < 2) fa[cur ^ 1][m] = *reinterpret_cast<const bf16x8*>(nst + fa_off[nkk][m]);
-      else if (m < 7) fb[cur ^ 1][m - 2] = *reinterpret_cast<const bf16x8*>(nst + fb_off[nkk][m - 2]);
+      // NRD reads over NMF MFMAs: one each (7 over 10), or two behind the first when there are more reads than MFMAs (6 over 5)
+      constexpr int EXTRA = NRD > NMF ? NRD - NMF : 0;
+      const int r0 = m == 0 ? 0 : m + EXTRA, nr = m == 0 ? 1 + EXTRA : (m + EXTRA < NRD ? 1 : 0);
+#pragma unroll
+      for (int i = 0; i < nr; ++i) read_frag(cur, nst, nkk, r0 + i);
       if (m < n) issue_load(lit, j0 + m);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // one MFMA
-      if (m < 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // one LDS read
+      if (nr == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // its LDS reads
+      if (nr == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       if (m < n) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // one VMEM read
     }
   };
@@ -251,18 +273,19 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
   float2* cs_tab = reinterpret_cast<float2*>(smem + NS * STAGE);
   if (a.has_rope) {
     const int f = tid & 31;
-    int64_t pos[BM / 8];
+    constexpr int RPP = NT / 32;                       // rows per pass
+    int64_t pos[BM / RPP];
 #pragma unroll
-    for (int j = 0; j < BM / 8; ++j) {
-      int64_t grow = row0 + (tid >> 5) + 8 * j;
+    for (int j = 0; j < BM / RPP; ++j) {
+      int64_t grow = row0 + (tid >> 5) + RPP * j;
       if (grow >= a.rows) grow = a.rows - 1;
       pos[j] = rope_position_raw(ra, grow);
     }
 #pragma unroll
-    for (int j = 0; j < BM / 8; ++j) {
+    for (int j = 0; j < BM / RPP; ++j) {
       float c, sn;
       rope_cos_sin(ra, fr, rope_wrap(pos[j], ra.max_ctx), f, &c, &sn);
-      cs_tab[((tid >> 5) + 8 * j) * CSROW + f] = make_float2(c, sn);
+      cs_tab[((tid >> 5) + RPP * j) * CSROW + f] = make_float2(c, sn);
     }
   }
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPW) : "memory");
@@ -283,7 +306,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
     for (int kk = 0; kk < KS; ++kk) {
       if (kk + 1 < KS) {
         if (kk == 0 && it > 0) {
-          step(kk & 1, st, kk + 1, it + NS - 1, 10, LPW - 10);
+          step(kk & 1, st, kk + 1, it + NS - 1, NL_LAST, NL_FIRST);
           issue_touch(it + kTouchDist);             // youngest in the queue: the wait below leaves it outstanding
         } else {
           step(kk & 1, st, kk + 1, 0, 0, 0);
@@ -293,7 +316,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
         // share has, and everyone has issued its last reads of slice it. Spelled out, because __syncthreads()
         // carries a fence that drains every load in flight, the look-ahead ones included.
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * (LPW + kTouch) + kTouch) : "memory");
-        step(kk & 1, nx, 0, it + NS, 0, 10);
+        step(kk & 1, nx, 0, it + NS, 0, NL_LAST);
       }
     }
   }
@@ -336,8 +359,8 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
         }
       }
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        const int r = 64 * wm + 32 * mb + l32;
+      for (int mb = 0; mb < MB; ++mb) {
+        const int r = 32 * MB * wm + 32 * mb + l32;
         float cs[8] = {1.f, 0.f, 1.f, 0.f, 1.f, 0.f, 1.f, 0.f};
         if (rotate) {
           const f32x4 c01 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0);
@@ -376,7 +399,7 @@ __global__ __launch_bounds__(256) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra
                       (reinterpret_cast<uintptr_t>(a.v) % 16 == 0) && a.q_rs % 8 == 0 && a.k_rs % 8 == 0 && a.v_rs % 8 == 0 &&
                       a.kv_slot_stride % 8 == 0;
 #pragma unroll 4
-  for (int ch = tid; ch < BM * (BN / 8); ch += 256) {
+  for (int ch = tid; ch < BM * (BN / 8); ch += NT) {
     const int r = ch / (BN / 8), cc = ch - r * (BN / 8);
     const int hl = cc >> 3, d8 = (cc & 7) * 8;
     const int head = head0 + hl;
@@ -429,9 +452,10 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
     launch_qkv_generic(a, ra, fr, st);
     return check_launch("qkv_rope_prefill(generic)");
   }
+  constexpr int WROWS = 4;
   static bool attr_set = false;   // raising the dynamic-LDS limit is idempotent; a benign race at worst repeats it
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel<WROWS>), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_prefill: cannot raise LDS limit: %s", hipGetErrorString(e));
     attr_set = true;
   }
@@ -441,6 +465,6 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   const int64_t tiles = tiles_m * tiles_n;
   TLLM_REQUIRE(tiles < (1ll << 31), TLLM_E_SHAPE, "qkv_rope_prefill: too many tiles");
   const int swizzle = (tiles_m % 8 == 0 && tiles_n % 4 == 0) ? 1 : 0;
-  hipLaunchKernelGGL(qkv_prefill_kernel, dim3((unsigned)tiles), dim3(256), SMEM, st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
+  hipLaunchKernelGGL(qkv_prefill_kernel<WROWS>, dim3((unsigned)tiles), dim3(WROWS * 128), SMEM, st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
   return check_launch("qkv_rope_prefill");
 }
