@@ -31,8 +31,9 @@
 // stage of this tile does not fit (3 x 56 KB > 160 KB). Measured without gain: the 2 x 2 grid of 64 x 160
 // wavefronts this kernel started with (70 us: one wavefront per SIMD, nothing to cover a stalled load issue),
 // pairs of 64 x 160 wavefronts taking alternate k16 steps (fewer fragment reads, 68 us), four extra wavefronts that
-// only load (71-75 us), K slices of 32 in a four-stage ring (77 us), other spreads of the loads over the steps and
-// other prefetch distances (+-1 us).
+// only load (71-75 us), K slices of 32 in a four-stage ring (77 us), a four-deep feed with two more slices in flight
+// into registers and written to LDS by ds_write (70.6 us -- so the two-stage window above is not the whole story),
+// other spreads of the loads over the steps and other prefetch distances (+-1 us).
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
