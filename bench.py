@@ -2,7 +2,7 @@
 """Benchmark of the gpt-oss layer-kernel path on one MI355X.
 
 A *step* is one pass of the hot path over one decode batch of B = 8 tokens at gpt-oss-20b
-shapes (BASELINE.json configs[1]): token-embedding gather [8] -> RMSNorm [8, 2880] ->
+shapes (the batch-8 decode configuration): token-embedding gather [8] -> RMSNorm [8, 2880] ->
 QKV + bias + YaRN rotary (2880 -> 5120, weight streaming) -> clamped SwiGLU [32, 5760].
 Every step uses the next of 24 distinct layer weight sets (708 MB of QKV weights), so the
 weights come from HBM, not from the 256 MB Infinity Cache. The K timed steps are captured
@@ -83,6 +83,15 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
                                           norm_scale=scales[i % N_LAYERS] if fused else None,
                                           weight_scale=wq[i % N_LAYERS][1] if w8 else None)
         flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of[("norm_qkv" if fused else "qkv") + ("_w8" if w8 else "")](n)
+    elif kind == "embed_norm_qkv_rope_decode":
+        idp = torch.randint(0, VOCAB_BENCH, (n,), generator=g, dtype=torch.int32).to(dev)
+        pp = torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
+        xo = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev)
+        qo = (torch.empty(n, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev),
+              torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev))
+        fn = lambda i: T.embed_qkv_rope_forward(idp, table, scales[i % N_LAYERS], 1e-5, weights[i % N_LAYERS], biases[i % N_LAYERS],
+                                                NQ, NKV, HD, yarn=yarn, positions=pp, out=qo, x_out=xo)
+        nbytes = bytes_of["norm_qkv"](n) + n * HIDDEN * 2
     elif kind in ("out_residual_decode", "out_residual_decode_w8"):
         w8 = kind.endswith("_w8")
         ow = [torch.empty(HIDDEN, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
@@ -164,6 +173,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--fuse-gather", action="store_true",
+                    help="the step's embedding gather rides in the QKV kernel too (2 launches per step instead of 3)")
     ap.add_argument("--unfused", action="store_true",
                     help="run RMSNorm as its own launch in front of the QKV kernel (default: normalised inside the QKV decode kernel)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -214,6 +225,11 @@ def main() -> int:
 
     def step(i: int) -> None:
         l = i % N_LAYERS
+        if args.fuse_gather:
+            T.embed_qkv_rope_forward(ids, table, scales[l], 1e-5, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=positions,
+                                     out=(q, k, v), x_out=h)
+            T.swiglu(swiglu_x, out=s_out)
+            return
         T.embedding_forward(ids, table, out=h)
         if args.unfused:
             T.rmsnorm_forward(x, scales[l], 1e-5, out=t)
@@ -326,6 +342,13 @@ def main() -> int:
                                                                            yarn=yarn, positions=pr, mode="decode", out=qo,
                                                                            norm_scale=scales[i % N_LAYERS]),
                          bytes_of["norm_qkv"](r), n=240)
+        # the first layer of a token step: the gather rides in the same launch (embedding_B8 + norm_qkv_rope_decode_B8 in one)
+        qo = (torch.empty(B, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev),
+              torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev))
+        bench_kernel("embed_norm_qkv_rope_decode_B8",
+                     lambda i, qo=qo: T.embed_qkv_rope_forward(ids, table, scales[i % N_LAYERS], 1e-5, weights[i % N_LAYERS], biases[i % N_LAYERS],
+                                                               NQ, NKV, HD, yarn=yarn, positions=positions, out=qo, x_out=h),
+                     bytes_of["norm_qkv"](B) + bytes_of["embedding"](B), n=240)
         # the same stream with the weight quantised to fp8 e4m3 + per-row scales (the reference's ATTN_FP8 option)
         wq = [T.quantize_fp8_rows(w) for w in weights]
         for r in (1, 8, 32):
@@ -514,7 +537,8 @@ def main() -> int:
         "config": {"workload": "configs[1]: B=8 decode step = embedding gather[8] + RMSNorm[8,2880] + QKV+bias+YaRN-RoPE(2880->5120) + "
                                "clamped SwiGLU[32,5760]; 24 rotating weight sets; HIP-graph replay of all steps",
                    "batch": B, "layers_rotated": N_LAYERS,
-                   "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel"},
+                   "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel",
+                   "gather": "inside the QKV decode kernel (x = table rows)" if args.fuse_gather else "own launch (x ~ N(0,1) as the configuration states)"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "attention_blocks24": attn_stack,
         "wall_s_timed_region": round(wall, 4),
     }

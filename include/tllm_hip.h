@@ -154,6 +154,20 @@ int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int sc
                                    int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
                                    const TllmRope* rope, void* stream);
 
+/* The first layer of a decode step in one launch: token-embedding gather (torch.nn.Embedding, model.py:906-908, 920)
+ * feeding the first block's RMSNorm + QKV + bias + rotary (model.py:476, 489-503). x_out[r, :] = table[ids[r], :]
+ * (bit-exact, [rows, hidden] dense: the residual stream the following layers read), and q / k / v as
+ * tllm_norm_qkv_rope_decode_bf16 computes them from x_out. ids: int32 or int64 [rows]; an id outside [0, vocab)
+ * reads row 0 or vocab - 1 and sets *oob_flag (may be NULL) -- unlike tllm_embedding_bf16, which writes zeros for it.
+ * w_scale: NULL for a bf16 W, else W holds fp8 bytes as in tllm_qkv_rope_decode_w8_bf16. norm_scale must not be
+ * NULL; hidden 2880, head_dim 64, rows <= 16 (larger batches: gather, then the QKV entry point). */
+int tllm_embed_norm_qkv_rope_decode_bf16(const void* ids, int ids_is_i64, const void* table, int64_t vocab, void* x_out,
+                                         int32_t* oob_flag, const void* norm_scale, int scale_is_bf16, float eps,
+                                         const void* W, const float* w_scale, const void* b, void* q, void* k, void* v,
+                                         int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
+                                         int64_t kv_slot_stride, int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads,
+                                         int head_dim, const TllmRope* rope, void* stream);
+
 /* The decode projection with an fp8 weight: W8 is [n_heads*64, hidden] OCP e4m3 bytes, w_scale one fp32
  * per output row, W[n][k] = fp8(W8[n][k]) * w_scale[n] (the reference's per-row quantisation,
  * triton_kernels.py:261-268; its use in the fused decode kernel, :927-940 and :963-965, argument

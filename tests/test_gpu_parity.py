@@ -251,6 +251,67 @@ def test_norm_qkv_fused_decode_parity(gpu, yarn, rows, scale_dtype):
     close(v, v2.float().cpu())
 
 
+@pytest.mark.parametrize("rows", [1, 5, 8, 9, 16, 20])
+@pytest.mark.parametrize("scale_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("id_dtype", [torch.int32, torch.int64])
+def test_embed_norm_qkv_one_launch(gpu, yarn, rows, scale_dtype, id_dtype):
+    """The first layer of a decode step in one launch: gathered rows bit-exact, q / k / v identical to what the
+    separate gather + fused norm/QKV kernel gives (same arithmetic on the same rows) and within tolerance of the oracle.
+    20 rows exercises the composed path behind the same call."""
+    d = O.make_inputs(rows, seed=500 + rows, norm_scale_dtype=scale_dtype)
+    g = torch.Generator().manual_seed(rows)
+    vocab = 1000
+    table = (torch.randn(vocab, 2880, generator=g) * (2.0 ** (torch.arange(vocab) % 7 - 3))[:, None]).bfloat16()
+    ids = torch.randint(0, vocab, (rows,), generator=g, dtype=id_dtype)
+    ids[0] = vocab - 1
+    if rows > 1:
+        ids[-1] = 0
+    flag = torch.zeros(1, dtype=torch.int32, device=gpu)
+    x, q, k, v = T.embed_qkv_rope_forward(ids.to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, d["w"].to(gpu), d["b"].to(gpu),
+                                          64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), oob_flag=flag)
+    x_ref = O.embedding_ref(table, ids)
+    assert torch.equal(x.cpu(), x_ref)
+    assert flag.item() == 0
+    q, k, v = q.clone(), k.clone(), v.clone()
+    t_ref = O.rmsnorm_ref(x_ref, d["norm_scale"].float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"])
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    q2, k2, v2 = T.qkv_rope_forward(x_ref.to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu),
+                                    mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
+
+
+def test_embed_norm_qkv_fp8_weight_and_bad_ids(gpu, yarn):
+    d = O.make_inputs(8, seed=77)
+    g = torch.Generator().manual_seed(3)
+    table = torch.randn(64, 2880, generator=g).bfloat16()
+    ids = torch.randint(0, 64, (8,), generator=g, dtype=torch.int64)
+    w8, ws = T.quantize_fp8_rows(d["w"].to(gpu))
+    x, q, k, v = T.embed_qkv_rope_forward(ids.to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, w8, d["b"].to(gpu), 64, 8, 64,
+                                          yarn=yarn, positions=d["positions"].to(gpu), weight_scale=ws)
+    assert torch.equal(x.cpu(), table[ids])
+    q, k, v = q.clone(), k.clone(), v.clone()
+    q2, k2, v2 = T.qkv_rope_forward(x, w8, d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), mode="decode",
+                                    norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5, weight_scale=ws)
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
+    # ids outside the table: clamped to the nearest row, flag raised, no fault
+    bad = ids.clone()
+    bad[2], bad[5] = -7, 64
+    flag = torch.zeros(1, dtype=torch.int32, device=gpu)
+    x, q, k, v = T.embed_qkv_rope_forward(bad.to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64,
+                                          yarn=yarn, positions=d["positions"].to(gpu), oob_flag=flag)
+    assert flag.item() == 1
+    want = table[bad.clamp(0, 63)]
+    assert torch.equal(x.cpu(), want)
+    # pooled outputs and a caller-provided x_out
+    xo = torch.empty(8, 2880, dtype=torch.bfloat16, device=gpu)
+    x, *_ = T.embed_qkv_rope_forward(ids.to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64,
+                                     yarn=yarn, positions=d["positions"].to(gpu), x_out=xo)
+    assert x.data_ptr() == xo.data_ptr() and torch.equal(xo.cpu(), table[ids])
+
+
 @pytest.mark.parametrize("rows", [17, 32, 50])
 def test_norm_qkv_fused_entry_point_beyond_16_rows(gpu, yarn, rows, monkeypatch):
     """The host picks two launches beyond 16 rows (faster there); the C entry point itself must still be right."""

@@ -47,6 +47,7 @@ SIGNATURES = {
     "tllm_qkv_rope_decode_bf16": (_i32, _QKV_SIG),
     "tllm_qkv_rope_prefill_bf16": (_i32, _QKV_SIG),
     "tllm_norm_qkv_rope_decode_bf16": (_i32, [_vp, _vp, _i32, _f32] + _QKV_SIG[1:]),
+    "tllm_embed_norm_qkv_rope_decode_bf16": (_i32, [_vp, _i32, _vp, _i64, _vp, _vp, _vp, _i32, _f32, _vp, _vp] + _QKV_SIG[2:]),
     "tllm_out_residual_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "tllm_unembedding_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "tllm_unembedding_argmax_workspace_bytes": (_i64, [_i64]),

@@ -22,6 +22,14 @@ struct QkvArgs {
   const void* norm_scale;     // fused RMSNorm prologue (decode fast path only): scale [hidden], fp32 or bf16
   float norm_eps;
   const float* w_scale;        // fp8 weight (decode fast path only): one fp32 scale per output row
+  // fused token-embedding gather (decode fast path with the fused norm only): x[r] = emb_table[emb_ids[r]], also
+  // written to emb_out (the residual stream the following layers read)
+  const void* emb_ids;         // int32 or int64 [rows]
+  int emb_ids_i64;
+  const bf16* emb_table;       // [emb_vocab, hidden]
+  int64_t emb_vocab;
+  bf16* emb_out;               // [rows, hidden] dense
+  int32_t* emb_oob;            // may be null
 };
 
 // KV-cache slot the new token goes to (0 when the outputs are plain tensors). A global load: call it early.

@@ -55,6 +55,12 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
   a->norm_scale = nullptr;
   a->norm_eps = 0.f;
   a->w_scale = nullptr;
+  a->emb_ids = nullptr;
+  a->emb_ids_i64 = 0;
+  a->emb_table = nullptr;
+  a->emb_vocab = 0;
+  a->emb_out = nullptr;
+  a->emb_oob = nullptr;
   return TLLM_OK;
 }
 
@@ -209,8 +215,13 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 // (triton_kernels.py:261-268, 927-940, 963-965). Half the bytes to stream; the values are widened to bf16 (exact)
 // on their way into the LDS patch, so the MFMAs and the fp32 accumulation are those of the bf16 kernel, and the
 // row scale multiplies the finished sum.
-template <int XR, int CH, int NORM, bool W8>
+// EMB: the activation rows are gathered from an embedding table by token id (the first layer of a decode step:
+// model.py:906-920 feeds the gather straight into the first block's norm + QKV); the workgroup with blockIdx.x == 0
+// also writes the gathered rows out, as the residual stream. An id outside the table reads row 0 or vocab - 1 and
+// raises the flag.
+template <int XR, int CH, int NORM, bool W8, bool EMB = false>
 __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
+  static_assert(!EMB || NORM != 0, "the fused gather exists with the fused norm only");
   constexpr int NW = 15, SPW = 6, NCH = SPW / CH, PAIRS = 10;
   constexpr int KV = 360;                 // 16-byte vectors per activation row (hidden 2880)
   constexpr int KVW = W8 ? 180 : 360;     // ... per weight row
@@ -274,6 +285,27 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   bf16x8 sc16 = {};
   if constexpr (NORM == 1) sc32 = reinterpret_cast<const f32x4*>(a.norm_scale)[wave * (SPW * 8) + (lane < SPW * 8 ? lane : SPW * 8 - 1)];
   if constexpr (NORM == 2) sc16 = reinterpret_cast<const bf16x8*>(a.norm_scale)[wave * (SPW * 4) + (lane < SPW * 4 ? lane : SPW * 4 - 1)];
+  // EMB: where each of this lane's activation rows starts in the table (one id per load slot, fetched first)
+  const bf16x8* xsrc[XL];
+  if constexpr (EMB) {
+    int64_t id[XL];
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      int e = i * 64 + lane;
+      e = e < XR * CPR ? e : XR * CPR - 1;
+      int r = e / CPR;
+      r = r < nvalid ? r : nvalid - 1;
+      id[i] = a.emb_ids_i64 ? reinterpret_cast<const int64_t*>(a.emb_ids)[row0 + r]
+                            : static_cast<int64_t>(reinterpret_cast<const int*>(a.emb_ids)[row0 + r]);
+    }
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const bool ok = id[i] >= 0 && id[i] < a.emb_vocab;
+      if (!ok && a.emb_oob) *a.emb_oob = 1;
+      const int64_t idc = id[i] < 0 ? 0 : (id[i] < a.emb_vocab ? id[i] : a.emb_vocab - 1);
+      xsrc[i] = reinterpret_cast<const bf16x8*>(a.emb_table) + idc * KV + wave * (SPW * 4);
+    }
+  }
   auto load_x = [&]() {
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
@@ -284,7 +316,8 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
         int r = e / CPR;
         const int kc = e - r * CPR;
         r = r < nvalid ? r : nvalid - 1;
-        xr[j * XL + i] = xg[r * KV + j * CPR + kc];
+        if constexpr (EMB) xr[j * XL + i] = xsrc[i][j * CPR + kc];
+        else xr[j * XL + i] = xg[r * KV + j * CPR + kc];
       }
     }
   };
@@ -365,6 +398,17 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
         ssq = fmaf(f, f, ssq);
       }
       if (e < XR * CPR) tmp[(c / XL) * (XR * CPR) + e] = ssq;
+    }
+    if constexpr (EMB) {
+      if (blockIdx.x == 0) {                  // one workgroup per row chunk leaves the gathered rows behind
+        bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + row0 * KV + wave * (SPW * 4);
+#pragma unroll
+        for (int c = 0; c < NCH * XL; ++c) {
+          const int e = (c % XL) * 64 + lane;
+          const int r = e / CPR, kc = e - r * CPR;
+          if (e < XR * CPR && r < nvalid) xo[r * KV + (c / XL) * CPR + kc] = xr[c];
+        }
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -526,6 +570,22 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 
 using namespace tllm;
 
+static void launch_cu_embed(int xr, int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+#define TLLM_CUE(XR, NORM)                                                                                          \
+  do {                                                                                                              \
+    if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, 3, NORM, true, true>), grid, dim3(960), 0, st, a, ra, fr);  \
+    else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, 3, NORM, false, true>), grid, dim3(960), 0, st, a, ra, fr);    \
+  } while (0)
+  if (xr == 8) {
+    if (norm == 1) TLLM_CUE(8, 1);
+    else TLLM_CUE(8, 2);
+  } else {
+    if (norm == 1) TLLM_CUE(16, 1);
+    else TLLM_CUE(16, 2);
+  }
+#undef TLLM_CUE
+}
+
 static void launch_cu(int xr, int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
 #define TLLM_CU1(XR, CH, NORM)                                                                                  \
   do {                                                                                                          \
@@ -552,21 +612,45 @@ static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, 
   const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
   const int64_t chunks = (rows + xr - 1) / xr;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
-  launch_cu(xr, norm, w8, dim3((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks), st, a, ra, fr);
+  const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
+  if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
+  else launch_cu(xr, norm, w8, grid, st, a, ra, fr);
   return check_launch(what);
 }
 
-// Common body of the two entry points that exist for the gpt-oss shape only (fused norm and/or fp8 weight).
+struct EmbedSrc {
+  const void* ids;
+  int ids_i64;
+  const void* table;
+  int64_t vocab;
+  int32_t* oob_flag;
+};
+
+// Common body of the entry points that exist for the gpt-oss shape only (fused gather, fused norm and/or fp8 weight).
 static int decode_2880_entry(const char* what, const void* x, const void* norm_scale, int scale_is_bf16, float eps, const void* W,
                              const float* w_scale, bool w8, const void* b, void* q, void* k, void* v, int64_t q_row_stride,
                              int64_t k_row_stride, int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows, int64_t hidden,
-                             int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope, void* stream) {
+                             int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope, void* stream,
+                             const EmbedSrc* emb = nullptr) {
   QkvArgs a;
   RopeArgs ra;
   YarnFreqs fr;
   int rc = qkv_validate(what, x, W, q, k, v, q_row_stride, k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads,
                         n_kv_heads, head_dim, rope, &a, &ra, &fr);
   if (rc != TLLM_OK) return rc;
+  if (emb) {
+    TLLM_REQUIRE(emb->ids && emb->table && emb->vocab > 0, TLLM_E_ARG, "%s: ids, table must not be NULL and vocab positive", what);
+    TLLM_REQUIRE(norm_scale != nullptr, TLLM_E_ARG, "%s: the fused gather needs the fused norm (norm_scale is NULL)", what);
+    TLLM_REQUIRE(rows <= 16, TLLM_E_SHAPE, "%s: at most 16 rows (got %lld): gather, then call the QKV entry point", what, (long long)rows);
+    TLLM_REQUIRE(aligned16(emb->table) && reinterpret_cast<uintptr_t>(emb->ids) % (emb->ids_i64 ? 8 : 4) == 0, TLLM_E_ALIGN,
+                 "%s: table must be 16-byte aligned and ids aligned to their size", what);
+    a.emb_ids = emb->ids;
+    a.emb_ids_i64 = emb->ids_i64;
+    a.emb_table = static_cast<const bf16*>(emb->table);
+    a.emb_vocab = emb->vocab;
+    a.emb_out = const_cast<bf16*>(a.x);
+    a.emb_oob = emb->oob_flag;
+  }
   TLLM_REQUIRE(hidden == 2880 && head_dim == 64, TLLM_E_SHAPE,
                "%s: this kernel exists for hidden 2880 / head_dim 64 only (got %lld / %d)", what, (long long)hidden, head_dim);
   TLLM_REQUIRE(aligned16(x) && aligned16(W) && aligned16(norm_scale), TLLM_E_ALIGN, "%s: x, W and norm_scale must be 16-byte aligned", what);
@@ -591,6 +675,18 @@ extern "C" int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_sc
   }
   return decode_2880_entry("norm_qkv_rope_decode", x, norm_scale, scale_is_bf16, eps, W, nullptr, false, b, q, k, v, q_row_stride,
                            k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads, n_kv_heads, head_dim, rope, stream);
+}
+
+extern "C" int tllm_embed_norm_qkv_rope_decode_bf16(const void* ids, int ids_is_i64, const void* table, int64_t vocab, void* x_out,
+                                                    int32_t* oob_flag, const void* norm_scale, int scale_is_bf16, float eps, const void* W,
+                                                    const float* w_scale, const void* b, void* q, void* k, void* v, int64_t q_row_stride,
+                                                    int64_t k_row_stride, int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows,
+                                                    int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope,
+                                                    void* stream) {
+  const EmbedSrc emb{ids, ids_is_i64, table, vocab, oob_flag};
+  return decode_2880_entry("embed_norm_qkv_rope_decode", x_out, norm_scale, scale_is_bf16, eps, W, w_scale, w_scale != nullptr, b, q, k, v,
+                           q_row_stride, k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads, n_kv_heads, head_dim, rope,
+                           stream, &emb);
 }
 
 extern "C" int tllm_qkv_rope_decode_w8_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps, const void* W8,

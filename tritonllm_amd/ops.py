@@ -304,6 +304,72 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     return q, k, v
 
 
+EMBED_FUSED_MAX_ROWS = 16
+
+
+def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: torch.Tensor, norm_eps: float, weight: torch.Tensor,
+                           bias: torch.Tensor | None, num_q_heads: int, num_kv_heads: int, head_dim: int, *,
+                           yarn: YarnParams | None = None, cos: torch.Tensor | None = None, sin: torch.Tensor | None = None,
+                           positions: torch.Tensor | None = None, offset: torch.Tensor | None = None,
+                           tokens_per_batch: int | None = None, max_context_length: int = 131072, rotate: bool = True,
+                           out: tuple | None = None, x_out: torch.Tensor | None = None, weight_scale: torch.Tensor | None = None,
+                           oob_flag: torch.Tensor | None = None):
+    """The first layer of a decode step: ``x = table[ids]`` (torch.nn.Embedding, model.py:906-908, 920), then the first
+    block's ``RMSNorm(x)`` + QKV + bias + rotary (model.py:476, 489-503). Returns ``(x, q, k, v)`` with ``x [rows, hidden]``
+    the gathered rows (bit-exact; the residual stream), q / k / v as ``qkv_rope_forward(x, ..., norm_scale=...)`` gives them.
+
+    Up to 16 ids at the gpt-oss shape this is ONE launch (the gather rides in the QKV kernel's activation loads);
+    otherwise it is the gather followed by ``qkv_rope_forward``. In the single launch an id outside the table reads
+    row 0 / vocab - 1 instead of producing a zero row; ``oob_flag`` is set either way."""
+    _on_gpu(ids, table, norm_scale, weight, bias, positions, offset, cos, sin, weight_scale, x_out, oob_flag)
+    assert ids.ndim == 1 and ids.dtype in (torch.int32, torch.int64)
+    assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
+    rows, (vocab, hidden) = ids.shape[0], table.shape
+    fused = 0 < rows <= EMBED_FUSED_MAX_ROWS and hidden == 2880 and head_dim == 64
+    if x_out is None:
+        x_out = torch.empty(rows, hidden, dtype=_BF16, device=table.device)
+    assert x_out.shape == (rows, hidden) and x_out.dtype == _BF16 and x_out.is_contiguous()
+    if not fused:
+        embedding_forward(ids, table, out=x_out, oob_flag=oob_flag)
+        q, k, v = qkv_rope_forward(x_out, weight, bias, num_q_heads, num_kv_heads, head_dim, yarn=yarn, cos=cos, sin=sin,
+                                   positions=positions, offset=offset, tokens_per_batch=tokens_per_batch,
+                                   max_context_length=max_context_length, rotate=rotate, out=out, norm_scale=norm_scale,
+                                   norm_eps=norm_eps, weight_scale=weight_scale)
+        return x_out, q, k, v
+    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
+    total_out, hidden_w = weight.shape
+    assert hidden == hidden_w and total_out == (num_q_heads + 2 * num_kv_heads) * head_dim
+    assert bias is None or bias.shape == (total_out,)
+    assert norm_scale.dtype in (torch.float32, _BF16) and norm_scale.shape == (hidden,)
+    if oob_flag is not None:
+        assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
+    ids = ids if ids.is_contiguous() else ids.contiguous()
+    norm_scale = norm_scale if norm_scale.is_contiguous() else norm_scale.contiguous()
+    _, weight, bias = _prep_linear(x_out, weight, bias)
+    w_scale = None if weight_scale is None else _prep_weight_scale(weight, weight_scale)
+    q_dim, kv_dim = num_q_heads * head_dim, num_kv_heads * head_dim
+    if out is None:
+        q = scratch_pool.get((rows, q_dim), _BF16, table.device)
+        kv = scratch_pool.get((2, rows, kv_dim), _BF16, table.device)
+        k, v = kv[0], kv[1]
+    else:
+        q, k, v = out
+        assert q.shape == (rows, q_dim) and k.shape == (rows, kv_dim) and v.shape == (rows, kv_dim)
+        assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1
+    keep: list = []
+    desc = None
+    if rotate:
+        desc = _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch if tokens_per_batch else rows, max_context_length, keep)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    rc = lib().tllm_embed_norm_qkv_rope_decode_bf16(
+        ids.data_ptr(), int(ids.dtype == torch.int64), table.data_ptr(), vocab, x_out.data_ptr(), ptr(oob_flag), norm_scale.data_ptr(),
+        int(norm_scale.dtype == _BF16), float(norm_eps), weight.data_ptr(), ptr(w_scale), ptr(bias), q.data_ptr(), k.data_ptr(),
+        v.data_ptr(), q.stride(0), k.stride(0), v.stride(0), 0, rows, hidden, num_q_heads, num_kv_heads, head_dim,
+        C.byref(desc) if desc is not None else None, _stream())
+    check(rc, "embed_norm_qkv_rope_decode")
+    return x_out, q, k, v
+
+
 def _split_head_dim(q_dim: int, kv_dim: int) -> int:
     """A head size that tiles both q_dim and kv_dim (no rotation: any even tiling will do)."""
     if q_dim % 64 == 0 and kv_dim % 64 == 0:
