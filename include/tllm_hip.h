@@ -232,6 +232,9 @@ int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_sc
  * scratch (4-byte aligned) that needs for the same arguments -- 0 for short contexts; the reference allocates its
  * acc/m/l partials per call (:343-345). head_dim must be 64, group <= 16. */
 int tllm_attention_decode_splits(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window);
+/* Diagnostic: KV heads served by one workgroup for these arguments (8 or 4: one wavefront per head, contiguous
+ * cache rows; 0: one KV head per workgroup). No counterpart in the reference. */
+int tllm_attention_decode_heads_per_workgroup(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window);
 int64_t tllm_attention_decode_workspace_bytes(int64_t batch, int n_q_heads, int n_kv_heads, int64_t n_kv_ctx, int window);
 int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, const void* sinks, void* out,
                                int64_t q_row_stride, int64_t out_row_stride, int64_t kv_batch_stride,

@@ -156,3 +156,22 @@ def test_mxfp4_argument_errors():
     assert lib.tllm_mxfp4_dequant_bf16(None, None, None, -1, None) == -1
     assert lib.tllm_mxfp4_dequant_bf16(C.c_void_p(8), C.c_void_p(1), C.c_void_p(16), 5, None) != 0   # blocks not 16-byte aligned
     assert "aligned" in _err()
+
+
+def test_attention_decode_shape_planning():
+    """The host-side choice of workgroup shape and splits (no launch): small batches keep one KV head per workgroup."""
+    hpw = _lib.lib().tllm_attention_decode_heads_per_workgroup
+    splits = _lib.lib().tllm_attention_decode_splits
+    assert [hpw(b, 8, 4096, 0) for b in (1, 4, 8)] == [0, 0, 0]
+    assert hpw(16, 8, 4096, 0) == 4 and splits(16, 8, 4096, 0) == 8
+    assert hpw(32, 8, 4096, 0) == 4 and splits(32, 8, 4096, 0) == 4
+    assert hpw(8, 8, 32768, 0) == 8 and splits(8, 8, 32768, 0) == 32
+    assert hpw(4, 8, 32768, 0) == 4 and splits(4, 8, 32768, 0) == 32
+    assert hpw(2, 8, 32768, 0) == 4 and splits(2, 8, 32768, 0) == 64
+    assert hpw(2, 8, 16384, 0) == 0
+    assert hpw(1, 8, 131072, 0) == 0
+    assert hpw(64, 8, 131072, 128) == 0 and splits(64, 8, 131072, 128) == 1      # a sliding window bounds the context
+    for b in (1, 3, 8, 100):
+        for ctx in (1, 127, 128, 129, 5000, 131072):
+            s = splits(b, 8, ctx, 0)
+            assert 1 <= s <= 64 and (s == 1 or ctx >= 128 * (s - 1))

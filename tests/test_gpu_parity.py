@@ -754,25 +754,24 @@ def test_attention_decode_edges(gpu):
 
 
 @pytest.mark.parametrize("case", [
-    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8191),                 # 32 splits of 256 keys
-    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8000, start_dtype=torch.int64),   # ragged last split
-    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=100),                  # most splits hold no key at all
-    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=0),                    # one key
-    dict(batch_size=16, num_keys=8192, sliding_window=4096, start_q=7000),                # window under the split planning
-    dict(batch_size=256, num_keys=300, sliding_window=None, start_q=299),                 # one split: written straight to the output
-    dict(batch_size=256, num_keys=300, sliding_window=None, start_q=280, with_sinks=False),
-    dict(batch_size=32, num_keys=2048, sliding_window=None, start_q=2047, kv_heads=4, groups=2),   # four wavefronts, two heads each
-    dict(batch_size=64, num_keys=1024, sliding_window=None, start_q=1000, kv_heads=2, groups=16),  # widest group
+    dict(batch_size=8, num_keys=32768, sliding_window=None, start_q=32767, hpw=8),        # 32 splits of 1024 keys, eight heads per workgroup
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8191, hpw=4),          # four heads per workgroup, 16 splits
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8000, start_dtype=torch.int64, hpw=4),   # ragged last split
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=100, hpw=4),           # most splits hold no key at all
+    dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=0, hpw=4),             # one key
+    dict(batch_size=16, num_keys=8192, sliding_window=4096, start_q=7000, hpw=4),         # window under the split planning
+    dict(batch_size=256, num_keys=600, sliding_window=None, start_q=599, hpw=8),          # one split: written straight to the output
+    dict(batch_size=256, num_keys=600, sliding_window=None, start_q=580, with_sinks=False, hpw=8),
+    dict(batch_size=64, num_keys=2048, sliding_window=None, start_q=2047, kv_heads=4, groups=2, hpw=4),    # a model with four KV heads
+    dict(batch_size=32, num_keys=4096, sliding_window=None, start_q=4000, kv_heads=16, groups=4, hpw=8),   # sixteen KV heads: two groups of eight
 ], ids=lambda c: "-".join(f"{k[0]}{v}" for k, v in c.items() if not isinstance(v, torch.dtype)))
 def test_attention_decode_row_workgroups(gpu, case):
-    """Large batch x context: the workgroup shape with one wavefront per KV head (chosen inside the library from
-    batch, heads and context; these cases all fall on it)."""
+    """Large batch x context: the workgroup shape with one wavefront per KV head over groups of eight or four heads
+    (chosen inside the library from batch, heads and context; each case states the grouping it expects)."""
     from tritonllm_amd._lib import lib
     c = dict(case)
-    kvh = c.get("kv_heads", 8)
-    splits = lib().tllm_attention_decode_splits(c["batch_size"], kvh, c["num_keys"], c["sliding_window"] or 0)
-    ctx = min(c["sliding_window"] or c["num_keys"], c["num_keys"])
-    assert c["batch_size"] * splits >= 224 and ctx >= 256 * splits, "case no longer selects the row-shaped workgroups"
+    hpw = c.pop("hpw")
+    assert lib().tllm_attention_decode_heads_per_workgroup(c["batch_size"], c.get("kv_heads", 8), c["num_keys"], c["sliding_window"] or 0) == hpw
     _attn_case(gpu, seed=11 + c["start_q"], **c)
 
 

@@ -53,6 +53,7 @@ SIGNATURES = {
     "tllm_unembedding_argmax_workspace_bytes": (_i64, [_i64]),
     "tllm_unembedding_argmax_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "tllm_attention_decode_splits": (_i32, [_i64, _i32, _i64, _i32]),
+    "tllm_attention_decode_heads_per_workgroup": (_i32, [_i64, _i32, _i64, _i32]),
     "tllm_attention_decode_workspace_bytes": (_i64, [_i64, _i32, _i32, _i64, _i32]),
     "tllm_attention_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _vp,
                                           _i32, _vp, _i64, _vp]),

@@ -7,11 +7,12 @@
 //
 // The reference runs one program per query head, so the G heads of a group each read the same K and V; here a
 // wavefront serves all G heads of a KV head from one pass over K and V, in one of two workgroup shapes:
-//   * ROWS (large batch x context): a workgroup takes a (batch row, context split) and has one wavefront per KV head,
-//     each walking the split's 32-key blocks in order. Together the wavefronts read whole cache rows (all KV heads
-//     of a token are adjacent in memory), so the workgroup streams one contiguous range of K and one of V; with
-//     nontemporal loads that pattern measures 6.8 TB/s on its own, where one-KV-head-per-workgroup streams stop at
-//     5.2 TB/s (128-byte pieces at a 1 KB stride, the sibling heads arriving from other workgroups at other times);
+//   * ROWS (large batch x context): a workgroup takes a (batch row, context split, group of eight or four adjacent
+//     KV heads) and has one wavefront per KV head, each walking the split's 32-key blocks in order. Together the
+//     wavefronts read whole (or half) cache rows -- all KV heads of a token are adjacent in memory -- so the workgroup
+//     streams long contiguous runs of K and of V; with nontemporal loads the whole-row pattern measures 6.8 TB/s on
+//     its own, where one-KV-head-per-workgroup streams stop at 5.2 TB/s (128-byte pieces at a 1 KB stride, the
+//     sibling heads arriving from other workgroups at other times);
 //   * HEAD (few batch rows): a workgroup takes a (batch row, KV head, context split); four wavefronts take the
 //     split's blocks in turn, each with its own running (max, sum, accumulator), and meet once at the end through
 //     LDS. This shape yields n_kv_heads times more workgroups, which is what fills the machine at batch 1;
@@ -66,8 +67,10 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, g = lane >> 4;
-  const int kvh = ROWS ? wave : blockIdx.x / a.splits;
-  const int split = ROWS ? blockIdx.x : blockIdx.x - kvh * a.splits;
+  // ROWS: blockIdx.x = head group * splits + split, the group's KV heads on the workgroup's wavefronts
+  const int grp = blockIdx.x / a.splits;
+  const int kvh = ROWS ? grp * static_cast<int>(blockDim.x >> 6) + wave : grp;
+  const int split = blockIdx.x - grp * a.splits;
   const int64_t b = blockIdx.y;
   const int G = a.group;
   const int n_q_heads = a.n_kv_heads * G;
@@ -328,14 +331,15 @@ __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(AttnArgs a, int 
 using namespace tllm;
 
 // Workgroup shape and context splits, from measurements at B = 1 .. 32, contexts 1K - 128K.
-// ROWS (a workgroup per (batch row, split), one wavefront per KV head) streams faster but yields n_kv_heads times
-// fewer workgroups, each wavefront walking its blocks one after the other: it is taken when batch x splits still
-// gives every CU a workgroup with at least 256 keys per split (B = 8: 106 -> 87 us at 32K context, but 17 -> 21 us
-// at 4K, where the splits would be 128 keys; B = 32 at 4K: 56 -> 48 us; B = 2 at 32K: 33 -> 42 us). Splits: first enough
-// workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) / 2048 (HEAD) keys per workgroup, never less than
-// 128 keys per split.
+// ROWS (a workgroup per (batch row, split, group of 8 or 4 KV heads), one wavefront per KV head) streams faster but
+// yields fewer workgroups, each wavefront walking its blocks one after the other: it is taken when it still gives
+// every CU a workgroup with at least 512 keys per split, in the head grouping that makes the splits longest
+// (us, HEAD -> ROWS: B = 8 at 32K 106 -> 86, at 8K 33 -> 27, at 4K 17 -> 17-21 (HEAD kept); B = 32 at 4K 56 -> 47;
+// B = 16 at 4K 32 -> 27; B = 4 at 32K 61 -> 47, at 16K 34 -> 28; B = 2 at 32K 34 -> 30, at 16K 18 -> 20 (HEAD kept);
+// B = 1: HEAD throughout). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
+// 2048 (HEAD) keys per workgroup, never less than 128 keys per split.
 // A sliding window bounds the context.
-struct AttnPlan { bool rows; int splits; };
+struct AttnPlan { int heads_per_wg; int splits; };   // heads_per_wg 0: the HEAD shape
 
 static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
   const int64_t ctx = (window > 0 && window < n_kv_ctx) ? window : n_kv_ctx;
@@ -350,11 +354,25 @@ static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int w
     if (s > 64) s = 64;
     return static_cast<int>(s);
   };
-  if (n_kv_heads >= 2 && n_kv_heads <= RW) {
-    const int s = splits_for(batch, 1024);
-    if (batch * s >= 224 && ctx >= 256 * static_cast<int64_t>(s)) return {true, s};
+  // eight or four KV heads per workgroup: whichever fills the machine with the longest splits (ties: the wider one)
+  AttnPlan best{0, 0};
+  int64_t best_keys = 0;
+  for (int hpw = RW; hpw >= 4; hpw >>= 1) {
+    if (n_kv_heads % hpw != 0) continue;
+    const int64_t units = batch * (n_kv_heads / hpw);
+    const int s = splits_for(units, 1024);
+    const int64_t keys = ctx / s;
+    if (units * s >= 224 && keys >= 512 && keys > best_keys) {
+      best = {hpw, s};
+      best_keys = keys;
+    }
   }
-  return {false, splits_for(batch * n_kv_heads, 2048)};
+  if (best.heads_per_wg) return best;
+  return {0, splits_for(batch * n_kv_heads, 2048)};
+}
+
+extern "C" int tllm_attention_decode_heads_per_workgroup(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
+  return attn_plan(batch, n_kv_heads, n_kv_ctx, window).heads_per_wg;
 }
 
 extern "C" int tllm_attention_decode_splits(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
@@ -406,8 +424,9 @@ extern "C" int tllm_attention_decode_bf16(const void* q, const void* k, const vo
                (long long)workspace_bytes);
   a.part = static_cast<float*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (plan.rows)
-    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3((unsigned)a.splits, (unsigned)batch), dim3(n_kv_heads * 64), 0, st, a);
+  if (plan.heads_per_wg)
+    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3((unsigned)(n_kv_heads / plan.heads_per_wg * a.splits), (unsigned)batch),
+                       dim3(plan.heads_per_wg * 64), 0, st, a);
   else
     hipLaunchKernelGGL(attn_decode_kernel<false>, dim3((unsigned)(n_kv_heads * a.splits), (unsigned)batch), dim3(AW * 64), 0, st, a);
   int rc = check_launch("attention_decode");
