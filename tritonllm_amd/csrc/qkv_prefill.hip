@@ -72,7 +72,8 @@ constexpr int OROW = BN + 4;       // epilogue staging row, elements (648 B: an 
 constexpr int CSROW = 34;                  // float2 per row of the cos/sin table: 32 frequencies + padding, so that
                                            // lanes reading the same frequency of 32 different rows spread over the banks
 constexpr int CS_BYTES = BM * CSROW * 8;   // cos/sin of (tile row, frequency) as float2
-constexpr int SMEM = NS * STAGE + CS_BYTES;
+constexpr int BIAS_BYTES = BN * 4;         // the tile's bias as fp32, head-local column order
+constexpr int SMEM = NS * STAGE + CS_BYTES + BIAS_BYTES;
 static_assert(BM * OROW * 2 <= NS * STAGE, "the epilogue's output image reuses the stage ring");
 static_assert(SMEM <= 160 * 1024, "LDS per workgroup");
 constexpr int BLOCKS = STAGE / 1024;      // 1 KiB blocks per stage
@@ -275,6 +276,14 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // LDS region while the first slices are in flight (the positions are global loads: all 16 are issued
   // before any is used).
   float2* cs_tab = reinterpret_cast<float2*>(smem + NS * STAGE);
+  // the tile's 320 bias values, widened once (fetched per group inside the epilogue they were twenty dependent
+  // global loads per lane, each waited for)
+  float* bias_s = reinterpret_cast<float*>(smem + NS * STAGE + CS_BYTES);
+  if (tid < BN) {
+    int h = head0 + (tid >> 6);
+    if (h >= total_heads) h = total_heads - 1;
+    bias_s[tid] = a.bias ? static_cast<float>(a.bias[h * 64 + (tid & 63)]) : 0.f;
+  }
   if (a.has_rope) {
     const int f = tid & 31;
     constexpr int RPP = NT / 32;                       // rows per pass
@@ -352,43 +361,38 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       if (g >= ngrp) continue;
       // first of the four consecutive low dims of this group, and where its partner lives
       const int d0 = hp < 2 ? (8 * g + 4 * lh) : (16 * wn + 8 * g + 4 * lh);
-      float b_lo[4] = {0.f, 0.f, 0.f, 0.f}, b_hi[4] = {0.f, 0.f, 0.f, 0.f};
-      if (a.bias) {
-        const bf16x4 bl = *reinterpret_cast<const bf16x4*>(a.bias + head * 64 + d0);
-        const bf16x4 bh = *reinterpret_cast<const bf16x4*>(a.bias + head * 64 + 32 + d0);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          b_lo[j] = static_cast<float>(bl[j]);
-          b_hi[j] = static_cast<float>(bh[j]);
-        }
-      }
+      const f32x4 b_lo = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + d0);
+      const f32x4 b_hi = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + 32 + d0);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int r = 32 * MB * wm + 32 * mb + l32;
-        float cs[8] = {1.f, 0.f, 1.f, 0.f, 1.f, 0.f, 1.f, 0.f};
-        if (rotate) {
-          const f32x4 c01 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0);
-          const f32x4 c23 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0 + 2);
+        float lo[4], hi[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            cs[j] = c01[j];
-            cs[4 + j] = c23[j];
+        for (int j = 0; j < 4; ++j) {
+          if (hp < 2) {
+            lo[j] = acc[mb][2 * hp][4 * g + j] + b_lo[j];
+            hi[j] = acc[mb][2 * hp + 1][4 * g + j] + b_hi[j];
+          } else {
+            lo[j] = acc[mb][4][4 * g + j] + b_lo[j];
+            hi[j] = acc[mb][4][8 + 4 * g + j] + b_hi[j];
           }
         }
         bf16x4 olo, ohi;
+        if (rotate) {                                      // uniform per wavefront and head
+          const f32x4 c01 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0);       // (cos, sin) of dims d0, d0 + 1
+          const f32x4 c23 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0 + 2);   // ... d0 + 2, d0 + 3
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float lo, hi;
-          if (hp < 2) {
-            lo = acc[mb][2 * hp][4 * g + j] + b_lo[j];
-            hi = acc[mb][2 * hp + 1][4 * g + j] + b_hi[j];
-          } else {
-            lo = acc[mb][4][4 * g + j] + b_lo[j];
-            hi = acc[mb][4][8 + 4 * g + j] + b_hi[j];
+          for (int j = 0; j < 4; ++j) {
+            const float c = j < 2 ? c01[2 * j] : c23[2 * j - 4], sn = j < 2 ? c01[2 * j + 1] : c23[2 * j - 3];
+            olo[j] = static_cast<bf16>(lo[j] * c - hi[j] * sn);
+            ohi[j] = static_cast<bf16>(hi[j] * c + lo[j] * sn);
           }
-          const float c = cs[2 * j], sn = cs[2 * j + 1];
-          olo[j] = static_cast<bf16>(rotate ? lo * c - hi * sn : lo);
-          ohi[j] = static_cast<bf16>(rotate ? hi * c + lo * sn : hi);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            olo[j] = static_cast<bf16>(lo[j]);
+            ohi[j] = static_cast<bf16>(hi[j]);
+          }
         }
         *reinterpret_cast<bf16x4*>(img + r * OROW + hl * 64 + d0) = olo;
         *reinterpret_cast<bf16x4*>(img + r * OROW + hl * 64 + 32 + d0) = ohi;
