@@ -418,6 +418,14 @@ def test_qkv_rope_prefill_long_context(gpu, yarn):
     _check_qkv(gpu, yarn, 8192, "prefill", seed=4, prefill_positions=True)
 
 
+@pytest.mark.parametrize("rows", [2049, 2304, 3841, 4000, 4096, 5000])
+def test_qkv_rope_prefill_256_token_tiles(gpu, yarn, rows):
+    """Row counts that would need a second round of 128-token tiles run on 256-token tiles instead (two-pass epilogue,
+    table built after the K loop; 8192 rows in the long-context test too): ragged last tiles, the XCD-swizzled and the
+    plain tile order, arbitrary positions. 5000 rows fall back on 128-token tiles in three rounds."""
+    _check_qkv(gpu, yarn, rows, "prefill", seed=rows, prefill_positions=rows % 2 == 0, max_pos=131072)
+
+
 def test_qkv_decode_and_prefill_agree(gpu, yarn):
     d = O.make_inputs(40, seed=21)
     args = (d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64)

@@ -18,10 +18,9 @@
 //     a CU's load queue is bounded and a wavefront that overflows it stalls, MFMAs included);
 //   * the fragment reads of the next k16 step are pinned between the MFMAs of the current one
 //     (sched_group_barrier): hoisted to the top of the iteration, as the compiler does by itself, the
-//     wavefronts read a slice's fragments in one burst with no MFMA running;
-//   * an L2 miss still costs more than a slice of MFMAs and LDS has no room for a third stage, so
-//     three slices ahead every workgroup touches (one dword per line) its share of the lines its
-//     XCD's tiles are going to need, which pulls them into that XCD's L2 in time (86 % L2 hits counted).
+//     wavefronts read a slice's fragments in one burst with no MFMA running.
+// (An L2 warm-up -- every workgroup touching, three slices ahead, its share of the lines its XCD's tiles would need --
+// paid with one wavefront per SIMD; with two it measures as noise or a small loss and is gone.)
 // Where the time goes at T = 2048 (66 us; builds with parts of the loop compiled out): the MFMAs, barriers,
 // prologue and epilogue alone take 43 us (30 us of MFMAs at the 1.9 GHz this load clocks at), adding the
 // fragment reads 55 us, the global->LDS loads alone (no MFMA, no fragment read) 56 us, everything 66 us. The
@@ -37,6 +36,10 @@
 // The feed itself: 256 tiles x 2.58 MB = 660 MB through the L2s in those 44 us (~15 TB/s, 7.1 M requests of 128 B);
 // doubling the requests (every wavefront touching its own lines ahead of time) cost 13 %, so only fewer bytes per
 // flop -- a larger tile, which T = 2048 on 256 CUs does not allow -- would lift the wall.
+// From T = 4096 up there are enough tokens for 256 x 320 tiles (BM = 256: eight wavefronts of 64 x 160, 36 % fewer
+// bytes per flop through the L2s): 238 -> 213 us at T = 8192 (1131 TFLOP/s). Its 160 accumulators leave room for
+// single-buffered weight fragments only, the cos/sin table is built after the K loop inside the idle stage ring
+// (no LDS for it next to 2 x 72 KB of stages) and the epilogue runs in two passes of 128 rows.
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
@@ -56,28 +59,31 @@
 namespace tllm {
 
 namespace {
-constexpr int BM = 128;            // tokens per tile
 constexpr int HPT = 5;             // heads per tile
 constexpr int BN = HPT * 64;       // 320 columns per tile
 constexpr int BK = 64;             // K slice: one 128-byte line per row
 constexpr int NS = 2;              // LDS stages
-constexpr int kTouchDist = 3;      // slices of lead of the L2 warm-up
 constexpr int KS = BK / 16;        // k16 MFMA steps per slice
 constexpr int CHUNKS = BK / 8;     // 16-byte chunks per LDS row
 constexpr int LROW = BK * 2;       // LDS row, bytes (unpadded: rows are swizzled instead)
 constexpr int RPB = 1024 / LROW;   // rows per 1 KiB block (one load instruction)
-constexpr int A_BYTES = BM * LROW;
-constexpr int STAGE = (BM + BN) * LROW;
+constexpr int stage_bytes(int bm) { return (bm + BN) * LROW; }   // one LDS stage of a bm-token tile
 constexpr int OROW = BN + 4;       // epilogue staging row, elements (648 B: an odd number of 8-byte units)
 constexpr int CSROW = 34;                  // float2 per row of the cos/sin table: 32 frequencies + padding, so that
                                            // lanes reading the same frequency of 32 different rows spread over the banks
-constexpr int CS_BYTES = BM * CSROW * 8;   // cos/sin of (tile row, frequency) as float2
+constexpr int EROWS = 128;                 // rows the epilogue finishes per pass (one pass for a 128-token tile, two for 256)
+constexpr int CS_BYTES = EROWS * CSROW * 8;   // cos/sin of (row, frequency) as float2
+constexpr int IMG_BYTES = (EROWS * OROW * 2 + 1023) / 1024 * 1024;   // bf16 image of a pass's rows
 constexpr int BIAS_BYTES = BN * 4;         // the tile's bias as fp32, head-local column order
-constexpr int SMEM = NS * STAGE + CS_BYTES + BIAS_BYTES;
-static_assert(BM * OROW * 2 <= NS * STAGE, "the epilogue's output image reuses the stage ring");
-static_assert(SMEM <= 160 * 1024, "LDS per workgroup");
-constexpr int BLOCKS = STAGE / 1024;      // 1 KiB blocks per stage
-static_assert(KS % 2 == 0 && BLOCKS % 8 == 0 && CHUNKS == 8 && NS == 2, "the schedule and the swizzle below are written for BK = 64, two stages");
+// A 128-token tile keeps the cos/sin table in its own region next to the two stages; a 256-token tile has no room for
+// that (2 x 72 KB of stages), keeps only the rows' positions and builds the table inside the idle stage ring, per pass.
+constexpr int prefill_smem(int bm) {
+  return bm == 128 ? NS * stage_bytes(128) + CS_BYTES + BIAS_BYTES : NS * stage_bytes(bm) + BIAS_BYTES + bm * 8;
+}
+static_assert(IMG_BYTES <= NS * stage_bytes(128) && IMG_BYTES + CS_BYTES <= NS * stage_bytes(256), "the epilogue reuses the stage ring");
+static_assert(prefill_smem(128) <= 160 * 1024 && prefill_smem(256) <= 160 * 1024, "LDS per workgroup");
+static_assert(KS % 2 == 0 && stage_bytes(128) % 8192 == 0 && stage_bytes(256) % 8192 == 0 && CHUNKS == 8 && NS == 2,
+              "the schedule and the swizzle below are written for BK = 64, two stages");
 }  // namespace
 
 // Chunk swizzle of LDS row r: the 16-byte chunk c of the row is stored at chunk position c ^ swz(r).
@@ -100,8 +106,12 @@ __device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
 
 // WROWS wavefront rows x 2 wavefront columns: 4 x 2 (two wavefronts per SIMD, 32 x 160 each) is what is launched;
 // 2 x 2 (one per SIMD, 64 x 160 each) compiles from the same source.
-template <int WROWS>
+// BM: tokens per tile. 128 makes T = 2048 one tile per CU; 256 (from T = 4096 up) reads each weight slice for twice
+// the tokens: 36 % fewer bytes per flop through the L2s, which is what bounds the 128-token tile.
+template <int BM, int WROWS>
 __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
+  constexpr int STAGE = stage_bytes(BM);
+  constexpr int BLOCKS = STAGE / 1024;      // 1 KiB blocks per stage
   constexpr int NW = WROWS * 2;             // wavefronts
   constexpr int NT = NW * 64;               // threads
   constexpr int MB = BM / (32 * WROWS);     // 32-token blocks per wavefront
@@ -112,13 +122,14 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   constexpr int NL_FIRST = LPW - NL_LAST;          // ... and behind the next slice's first step
   static_assert(NL_FIRST <= NMF, "a slice's loads fit behind two k16 steps");
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar: which operand a load belongs to is then a scalar choice
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
   // ---- tile assignment: XCD-aware. Consecutive block ids go to different XCDs (8 of them, each
   // with its own L2), so give every XCD a compact 8 x 4 super-block of tiles to maximise L2 reuse.
-  int tile_m, tile_n, share_q = -1, share_p = -1;     // position inside the XCD's super-block (-1: unknown)
+  int tile_m, tile_n;
   {
     const int b = blockIdx.x;
     if (swizzle) {
@@ -128,8 +139,6 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       const int sbm = tiles_m >> 3;
       tile_m = (sb % sbm) * 8 + (in & 7);
       tile_n = (sb / sbm) * 4 + (in >> 3);
-      share_q = in >> 3;
-      share_p = in & 7;
     } else {
       tile_m = b % tiles_m;
       tile_n = b / tiles_m;
@@ -147,63 +156,41 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // each starts its round of blocks at a different one so that at any moment they pull on different
   // rows (different L2 channels) instead of queueing on the same line.
   const int rot = (blockIdx.x >> 3) % LPW;
-  const bf16x8* src[LPW];
+  // A load's source is a scalar base (the tile's first activation row, or the weight) plus a 32-bit byte offset per
+  // lane: half the registers of a pointer per load, and the loads can use the scalar-base addressing form.
+  const unsigned char* const x_base = reinterpret_cast<const unsigned char*>(a.x) + row0 * a.hidden * 2;
+  const unsigned char* const w_base = reinterpret_cast<const unsigned char*>(a.W);
+  unsigned soff[LPW];
   int blk_off[LPW];                                          // LDS byte offset of load j's block inside the wavefront's share
+  bool src_is_x[LPW];                                        // scalar: a 1 KiB block lies entirely in one operand
 #pragma unroll
   for (int j = 0; j < LPW; ++j) {
     const int bj = (j + rot) % LPW;
     blk_off[j] = bj * 1024;
-    const int r = (wave * LPW + bj) * RPB + lane / CHUNKS;  // LDS row: 0..127 activations, 128..447 weights
+    const int r = (wave * LPW + bj) * RPB + lane / CHUNKS;  // LDS row: 0..BM-1 activations, then 320 weight rows
     const int c = (lane % CHUNKS) ^ swz(r);
-    if (r < BM) {
-      int64_t gr = row0 + r;
-      if (gr >= a.rows) gr = a.rows - 1;                // clamp: valid memory, result rows are never stored
-      src[j] = reinterpret_cast<const bf16x8*>(a.x) + gr * kvec + c;
+    src_is_x[j] = (wave * LPW + bj) * RPB < BM;
+    if (src_is_x[j]) {
+      int64_t lr = r;
+      if (row0 + lr >= a.rows) lr = a.rows - 1 - row0;      // clamp: valid memory, result rows are never stored
+      soff[j] = static_cast<unsigned>((lr * kvec + c) * 16);
     } else {
       int hl, dim;
       w_tile_row(r - BM, &hl, &dim);
       int h = head0 + hl;
       if (h >= total_heads) h = total_heads - 1;        // clamp for a ragged last tile
-      src[j] = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(h) * 64 + dim) * kvec + c;
+      soff[j] = static_cast<unsigned>(((static_cast<int64_t>(h) * 64 + dim) * kvec + c) * 16);
     }
   }
-  // L2 warm-up. With one tile per CU an L2 miss stalls the whole pipeline for longer than a slice of MFMAs
-  // lasts, and LDS has room for only two stages of BK = 64. So three slices ahead each workgroup touches
-  // (one dword per 128-byte line) its share of the lines its XCD's 32 tiles will need: a quarter of its
-  // activation rows (four tiles share them) and an eighth of its weight rows (eight tiles share them) --
-  // 72 lanes of one load. Nothing waits for these loads; they only pull the lines into the XCD's L2.
-  // Every wavefront issues exactly one such load per slice (18 working lanes each; idle lanes and
-  // unswizzled launches re-touch a line that is needed anyway), so the wait counts below are constants.
-  constexpr int TPW = 72 / NW;                        // touch lanes per wavefront
-  const int tch = lane < TPW ? wave * TPW + lane : 72;
-  const unsigned char* touch_ptr = reinterpret_cast<const unsigned char*>(src[0]);
-  if (share_q >= 0 && tch < 72) {
-    if (tch < 32) {
-      int64_t gr = row0 + 32 * share_q + tch;
-      if (gr >= a.rows) gr = a.rows - 1;
-      touch_ptr = reinterpret_cast<const unsigned char*>(a.x) + gr * a.hidden * 2;
-    } else {
-      int hl, dim;
-      w_tile_row(40 * share_p + (tch - 32), &hl, &dim);
-      int h = head0 + hl;
-      if (h >= total_heads) h = total_heads - 1;
-      touch_ptr = reinterpret_cast<const unsigned char*>(a.W) + (static_cast<int64_t>(h) * 64 + dim) * a.hidden * 2;
-    }
-  }
-  // The destination register must stay reserved for as long as a touch may be in flight (the data lands
-  // whenever it lands): it is threaded through every asm as read-write and consumed after the final drain.
-  unsigned touch_sink = 0;
-  auto issue_touch = [&](int it) {
-    const int itc = it < n_iter ? it : n_iter - 1;
-    asm volatile("global_load_dword %0, %1, off" : "+v"(touch_sink) : "v"(touch_ptr + itc * (BK * 2)) : "memory");
+  auto src_ptr = [&](int j, int itc) -> const unsigned char* {
+    return (src_is_x[j] ? x_base : w_base) + static_cast<int64_t>(itc) * (BK * 2) + soff[j];
   };
-  constexpr int kTouch = 1;                              // touch loads per wavefront per slice
   auto issue_loads = [&](int it) {                      // slice `it` -> stage it % NS; past the end: re-read the last slice (never consumed)
     unsigned char* dst = smem + (it % NS) * STAGE + wave * (LPW * 1024);
     const int itc = it < n_iter ? it : n_iter - 1;
 #pragma unroll
     for (int j = 0; j < LPW; ++j)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + itc * CHUNKS),
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src_ptr(j, itc),
                                        (__attribute__((address_space(3))) void*)(dst + blk_off[j]), 16, 0, 0);
   };
 
@@ -217,24 +204,24 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
 
   // fragment addressing: byte offset of (row, chunk c) inside a stage is row*LROW + ((c ^ swz(row)) << 4)
   const int fa_row = 32 * MB * wm + l32, fb_row = BM + 160 * wn + l32;
-  int fa_off[KS][MB], fb_off[KS][5];                     // [k16 step within the slice][block]
+  // The k16 step kk wants chunks 2 kk + lh of the row; with the row's swizzle that is position (2 kk + lh) ^ swz(row),
+  // and because a row starts on a 128-byte boundary the step enters as an XOR of bits 5-6 of the byte offset: one
+  // register per 32-row block instead of one per block and step.
+  int fa_o[MB], fb_o[5];
 #pragma unroll
-  for (int kk = 0; kk < KS; ++kk) {
+  for (int mb = 0; mb < MB; ++mb) fa_o[mb] = (fa_row + 32 * mb) * LROW + ((lh ^ swz(fa_row + 32 * mb)) << 4);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) fa_off[kk][mb] = (fa_row + 32 * mb) * LROW + (((2 * kk + lh) ^ swz(fa_row + 32 * mb)) << 4);
-#pragma unroll
-    for (int nb = 0; nb < 5; ++nb) fb_off[kk][nb] = (fb_row + 32 * nb) * LROW + (((2 * kk + lh) ^ swz(fb_row + 32 * nb)) << 4);
-  }
+  for (int nb = 0; nb < 5; ++nb) fb_o[nb] = (fb_row + 32 * nb) * LROW + ((lh ^ swz(fb_row + 32 * nb)) << 4);
   auto load_frags = [&](const unsigned char* st, int kk, bf16x8 (&fa)[MB], bf16x8 (&fb)[5]) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(st + fa_off[kk][mb]);
+    for (int mb = 0; mb < MB; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(st + (fa_o[mb] ^ (kk << 5)));
 #pragma unroll
-    for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(st + fb_off[kk][nb]);
+    for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(st + (fb_o[nb] ^ (kk << 5)));
   };
   auto issue_load = [&](int it, int j) {                // one load instruction of slice `it`
     unsigned char* dst = smem + (it % NS) * STAGE + wave * (LPW * 1024);
     const int itc = it < n_iter ? it : n_iter - 1;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + itc * CHUNKS),
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src_ptr(j, itc),
                                      (__attribute__((address_space(3))) void*)(dst + blk_off[j]), 16, 0, 0);
   };
   // One k16 step: ten MFMAs on the fragments in buffer `cur`. Behind MFMA m goes the LDS read of fragment m of
@@ -248,10 +235,31 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   //     row do exactly that. Handed out one per MFMA (32 cycles) they never find the queue full.
   bf16x8 fa[2][MB], fb[2][5];
   auto read_frag = [&](int cur, const unsigned char* nst, int nkk, int i) {   // fragment i of the next step: activations first
-    if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nst + fa_off[nkk][i < MB ? i : 0]);
-    else fb[cur ^ 1][i - MB] = *reinterpret_cast<const bf16x8*>(nst + fb_off[nkk][i - MB]);
+    if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nst + (fa_o[i < MB ? i : 0] ^ (nkk << 5)));
+    else fb[cur ^ 1][i - MB] = *reinterpret_cast<const bf16x8*>(nst + (fb_o[i - MB] ^ (nkk << 5)));
   };
   auto step = [&](int cur, const unsigned char* nst, int nkk, int lit, int j0, int n) {
+    if constexpr (MB == 2) {
+      // 64 x 160 per wavefront: the two MFMAs that share a weight fragment are issued back to back and the fragment is
+      // reloaded for the next step right behind them (weight fragments single-buffered: 20 registers instead of 40, which
+      // is what keeps this variant's 160 accumulators + fragments inside 256 registers); the activation fragments of the
+      // next step go into their second buffer behind the first two pairs.
+#pragma unroll
+      for (int nb = 0; nb < 5; ++nb) {
+        acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][nb], fa[cur][0], acc[0][nb], 0, 0, 0);
+        acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][nb], fa[cur][1], acc[1][nb], 0, 0, 0);
+        fb[0][nb] = *reinterpret_cast<const bf16x8*>(nst + (fb_o[nb] ^ (nkk << 5)));
+        if (nb < 2) fa[cur ^ 1][nb] = *reinterpret_cast<const bf16x8*>(nst + (fa_o[nb] ^ (nkk << 5)));
+        if (2 * nb < n) issue_load(lit, j0 + 2 * nb);
+        if (2 * nb + 1 < n) issue_load(lit, j0 + 2 * nb + 1);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        if (nb < 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (2 * nb + 1 < n) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        else if (2 * nb < n) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int m = 0; m < NMF; ++m) {
       const int mb = m / 5, nb = m % 5;
@@ -272,33 +280,49 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // prologue: slices 0..NS-2 in flight, slice 0 landed
 #pragma unroll
   for (int i = 0; i < NS - 1; ++i) issue_loads(i);
-  // cos/sin of (tile row, frequency) for the epilogue, computed from the YaRN parameters into its own
-  // LDS region while the first slices are in flight (the positions are global loads: all 16 are issued
-  // before any is used).
-  float2* cs_tab = reinterpret_cast<float2*>(smem + NS * STAGE);
+  // cos/sin of (row, frequency) for the epilogue, computed from the YaRN parameters. A 128-token tile builds the table
+  // here, into its own LDS region, while the first slices are in flight (the positions are global loads: all of
+  // them are issued before any is used). A 256-token tile only parks the rows' positions in LDS now and builds the
+  // table after the K loop, inside the idle stage ring, 128 rows at a time.
+  constexpr bool CS_EARLY = BM == EROWS;
+  constexpr int CS_OFF = CS_EARLY ? NS * STAGE : IMG_BYTES;
+  constexpr int BIAS_OFF = CS_EARLY ? NS * STAGE + CS_BYTES : NS * STAGE;
+  float2* cs_tab = reinterpret_cast<float2*>(smem + CS_OFF);
   // the tile's 320 bias values, widened once (fetched per group inside the epilogue they were twenty dependent
   // global loads per lane, each waited for)
-  float* bias_s = reinterpret_cast<float*>(smem + NS * STAGE + CS_BYTES);
+  float* bias_s = reinterpret_cast<float*>(smem + BIAS_OFF);
+  int64_t* pos_s = reinterpret_cast<int64_t*>(smem + BIAS_OFF + BIAS_BYTES);   // 256-token tile only
   if (tid < BN) {
     int h = head0 + (tid >> 6);
     if (h >= total_heads) h = total_heads - 1;
     bias_s[tid] = a.bias ? static_cast<float>(a.bias[h * 64 + (tid & 63)]) : 0.f;
   }
-  if (a.has_rope) {
+  constexpr int RPP = NT / 32;                         // table rows per round of the whole workgroup
+  auto fill_cs_rows = [&](auto&& pos_of) {             // the table of EROWS rows; pos_of(row) -> raw position
     const int f = tid & 31;
-    constexpr int RPP = NT / 32;                       // rows per pass
-    int64_t pos[BM / RPP];
+    int64_t pos[EROWS / RPP];
 #pragma unroll
-    for (int j = 0; j < BM / RPP; ++j) {
-      int64_t grow = row0 + (tid >> 5) + RPP * j;
-      if (grow >= a.rows) grow = a.rows - 1;
-      pos[j] = rope_position_raw(ra, grow);
-    }
+    for (int j = 0; j < EROWS / RPP; ++j) pos[j] = pos_of((tid >> 5) + RPP * j);
 #pragma unroll
-    for (int j = 0; j < BM / RPP; ++j) {
+    for (int j = 0; j < EROWS / RPP; ++j) {
       float c, sn;
       rope_cos_sin(ra, fr, rope_wrap(pos[j], ra.max_ctx), f, &c, &sn);
       cs_tab[((tid >> 5) + RPP * j) * CSROW + f] = make_float2(c, sn);
+    }
+  };
+  if (a.has_rope) {
+    if constexpr (CS_EARLY) {
+      fill_cs_rows([&](int r) {
+        int64_t grow = row0 + r;
+        if (grow >= a.rows) grow = a.rows - 1;
+        return rope_position_raw(ra, grow);
+      });
+    } else {
+      for (int r = tid; r < BM; r += NT) {
+        int64_t grow = row0 + r;
+        if (grow >= a.rows) grow = a.rows - 1;
+        pos_s[r] = rope_position_raw(ra, grow);
+      }
     }
   }
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPW) : "memory");
@@ -311,7 +335,6 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // this last step (ten of them) and of the next slice's first step (the other four) -- a whole slice of
   // MFMAs before they are needed.
   issue_loads(NS - 1);
-  issue_touch(kTouchDist);
   for (int it = 0; it < n_iter; ++it) {
     const unsigned char* st = smem + (it % NS) * STAGE;
     const unsigned char* nx = smem + ((it + 1) % NS) * STAGE;
@@ -320,22 +343,20 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       if (kk + 1 < KS) {
         if (kk == 0 && it > 0) {
           step(kk & 1, st, kk + 1, it + NS - 1, NL_LAST, NL_FIRST);
-          issue_touch(it + kTouchDist);             // youngest in the queue: the wait below leaves it outstanding
         } else {
           step(kk & 1, st, kk + 1, 0, 0, 0);
         }
       } else {
-        // Slice it+1 has landed (this wavefront's share; the touch stays in flight), then the barrier: everyone's
+        // Slice it+1 has landed (this wavefront's share), then the barrier: everyone's
         // share has, and everyone has issued its last reads of slice it. Spelled out, because __syncthreads()
         // carries a fence that drains every load in flight, the look-ahead ones included.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * (LPW + kTouch) + kTouch) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * LPW) : "memory");
         step(kk & 1, nx, 0, it + NS, 0, NL_LAST);
       }
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch_sink)::"memory");   // drain the look-ahead loads before LDS is reused
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // drain the look-ahead loads before LDS is reused
   __syncthreads();
-  if (touch_sink == 0x7fc12345u && tid == 1023) a.q[0] = static_cast<bf16>(0.f);   // keeps the sink register alive; never true
 
   // ---- epilogue -------------------------------------------------------------------------------
   // The stage ring is idle now and becomes a bf16 image of the output tile (rows padded to 656 B so the
@@ -343,14 +364,28 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // rotation with the cos/sin table, one RNE) into the image; then the tile leaves as coalesced
   // 128-bit stores, eight columns of one head per lane.
   bf16* img = reinterpret_cast<bf16*>(smem);
+  const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(a.q) % 16 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(a.v) % 16 == 0) && a.q_rs % 8 == 0 && a.k_rs % 8 == 0 && a.v_rs % 8 == 0 &&
+                      a.kv_slot_stride % 8 == 0;
 
   // Accumulator layout (weights on the MFMA's M side): the lane owns token l32 of each 32-token block and,
   // in each 32-column block, columns 8*(v>>2) + 4*lh + (v&3) -- runs of four consecutive columns, so
   // bias, cos/sin and the image stores all move in 4-element vectors. A whole head is two blocks (low
   // dims, their partners: same register index); the mixed block holds the wavefront's 16 low dims of
   // the middle head in rows 0-15 and their partners in rows 16-31 (register v and v + 8).
+  // A pass finishes EROWS rows: the wavefronts that hold them write the image, then everyone copies it out.
+#pragma unroll
+  for (int pass = 0; pass < BM / EROWS; ++pass) {
+  if constexpr (!CS_EARLY) {
+    if (pass > 0) __syncthreads();                        // the previous pass's image and table have been read
+    if (a.has_rope) fill_cs_rows([&](int r) { return pos_s[EROWS * pass + r]; });
+    __syncthreads();
+  }
+  const bool my_pass = (32 * MB * wm) / EROWS == pass;     // uniform per wavefront
 #pragma unroll
   for (int hp = 0; hp < 3; ++hp) {
+    if (!my_pass) break;
     const int hl = (hp < 2) ? (3 * wn + hp) : 2;
     int head = head0 + hl;
     if (head >= total_heads) head = total_heads - 1;        // ragged last tile: computed, never copied out
@@ -365,7 +400,7 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       const f32x4 b_hi = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + 32 + d0);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const int r = 32 * MB * wm + 32 * mb + l32;
+        const int r = 32 * MB * wm + 32 * mb + l32 - EROWS * pass;   // row inside the pass
         float lo[4], hi[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -402,16 +437,12 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   __syncthreads();
 
   // copy-out: chunk = 8 consecutive dims of one head of one row
-  const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(a.q) % 16 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 16 == 0) &&
-                      (reinterpret_cast<uintptr_t>(a.v) % 16 == 0) && a.q_rs % 8 == 0 && a.k_rs % 8 == 0 && a.v_rs % 8 == 0 &&
-                      a.kv_slot_stride % 8 == 0;
 #pragma unroll 4
-  for (int ch = tid; ch < BM * (BN / 8); ch += NT) {
+  for (int ch = tid; ch < EROWS * (BN / 8); ch += NT) {
     const int r = ch / (BN / 8), cc = ch - r * (BN / 8);
     const int hl = cc >> 3, d8 = (cc & 7) * 8;
     const int head = head0 + hl;
-    const int64_t grow = row0 + r;
+    const int64_t grow = row0 + EROWS * pass + r;
     if (head >= total_heads || grow >= a.rows) continue;
     bf16* dst;
     if (head < a.n_q_heads)
@@ -436,6 +467,7 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       for (int e = 0; e < 8; ++e) dst[e] = val[e];
     }
   }
+  }   // pass
 }
 
 }  // namespace tllm
@@ -455,7 +487,9 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   a.bias = (const bf16*)b;
   if (rows == 0) return TLLM_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool fast = head_dim == 64 && hidden % BK == 0 && aligned16(x) && aligned16(W);
+  // the kernel addresses a tile's rows and the weight with 32-bit byte offsets
+  const bool fast = head_dim == 64 && hidden % BK == 0 && aligned16(x) && aligned16(W) &&
+                    static_cast<int64_t>(n_q_heads + 2 * n_kv_heads) * 64 * hidden * 2 < (1ll << 32) && 256 * hidden * 2 < (1ll << 32);
   if (!fast) {
     launch_qkv_generic(a, ra, fr, st);
     return check_launch("qkv_rope_prefill(generic)");
@@ -463,16 +497,31 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   constexpr int WROWS = 4;
   static bool attr_set = false;   // raising the dynamic-LDS limit is idempotent; a benign race at worst repeats it
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel<WROWS>), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel<128, WROWS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, prefill_smem(128));
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel<256, WROWS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              prefill_smem(256));
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_prefill: cannot raise LDS limit: %s", hipGetErrorString(e));
     attr_set = true;
   }
   const int heads = n_q_heads + 2 * n_kv_heads;
+  // Tile height by a two-number cost model: a round of 128-token tiles over the 256 CUs takes ~65 us, a round of
+  // 256-token tiles ~109 us (3 : 5); whichever needs less in total. T = 2048 is one round of 128s; anything that would
+  // need a second round of 128s is one round of 256s instead, T = 8192 two rounds of 256s instead of four of 128s.
+  const int64_t tn = (heads + HPT - 1) / HPT;
+  const int64_t rounds128 = (((rows + 127) / 128) * tn + 255) / 256, rounds256 = (((rows + 255) / 256) * tn + 255) / 256;
+  const int BM = rounds256 * 5 < rounds128 * 3 ? 256 : 128;
   const int64_t tiles_m = (rows + BM - 1) / BM;
   const int tiles_n = (heads + HPT - 1) / HPT;
   const int64_t tiles = tiles_m * tiles_n;
   TLLM_REQUIRE(tiles < (1ll << 31), TLLM_E_SHAPE, "qkv_rope_prefill: too many tiles");
   const int swizzle = (tiles_m % 8 == 0 && tiles_n % 4 == 0) ? 1 : 0;
-  hipLaunchKernelGGL(qkv_prefill_kernel<WROWS>, dim3((unsigned)tiles), dim3(WROWS * 128), SMEM, st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
+  if (BM == 256)
+    hipLaunchKernelGGL((qkv_prefill_kernel<256, WROWS>), dim3((unsigned)tiles), dim3(WROWS * 128), prefill_smem(256), st, a, ra, fr,
+                       (int)tiles_m, tiles_n, swizzle);
+  else
+    hipLaunchKernelGGL((qkv_prefill_kernel<128, WROWS>), dim3((unsigned)tiles), dim3(WROWS * 128), prefill_smem(128), st, a, ra, fr,
+                       (int)tiles_m, tiles_n, swizzle);
   return check_launch("qkv_rope_prefill");
 }
