@@ -182,17 +182,6 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       soff[j] = static_cast<unsigned>(((static_cast<int64_t>(h) * 64 + dim) * kvec + c) * 16);
     }
   }
-  auto src_ptr = [&](int j, int itc) -> const unsigned char* {
-    return (src_is_x[j] ? x_base : w_base) + static_cast<int64_t>(itc) * (BK * 2) + soff[j];
-  };
-  auto issue_loads = [&](int it) {                      // slice `it` -> stage it % NS; past the end: re-read the last slice (never consumed)
-    unsigned char* dst = smem + (it % NS) * STAGE + wave * (LPW * 1024);
-    const int itc = it < n_iter ? it : n_iter - 1;
-#pragma unroll
-    for (int j = 0; j < LPW; ++j)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src_ptr(j, itc),
-                                       (__attribute__((address_space(3))) void*)(dst + blk_off[j]), 16, 0, 0);
-  };
 
   f32x16 acc[MB][5];
 #pragma unroll
@@ -221,8 +210,16 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   auto issue_load = [&](int it, int j) {                // one load instruction of slice `it`
     unsigned char* dst = smem + (it % NS) * STAGE + wave * (LPW * 1024);
     const int itc = it < n_iter ? it : n_iter - 1;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src_ptr(j, itc),
-                                     (__attribute__((address_space(3))) void*)(dst + blk_off[j]), 16, 0, 0);
+    // Spelled out rather than through __builtin_amdgcn_global_load_lds: this is the scalar-base form (64-bit base in
+    // SGPRs, 32-bit lane offset, LDS block address in M0), where the builtin builds a 64-bit address per lane; 14 / 13
+    // fewer registers in the two tile heights and 2-3 % faster. The lanes' 16 bytes land at M0 + 16 * lane.
+    const unsigned lds_off = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst + blk_off[j]));
+    const unsigned char* sb = (src_is_x[j] ? x_base : w_base) + static_cast<int64_t>(itc) * (BK * 2);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
+  };
+  auto issue_loads = [&](int it) {                      // all of slice `it` -> stage it % NS
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) issue_load(it, j);
   };
   // One k16 step: ten MFMAs on the fragments in buffer `cur`. Behind MFMA m goes the LDS read of fragment m of
   // the next step (seven of them, into buffer cur ^ 1) and, for m < n, one global->LDS load instruction
