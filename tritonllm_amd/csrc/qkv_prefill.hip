@@ -3,8 +3,8 @@
 //   D[T, 5120] = X[T, 2880] . W[5120, 2880]^T      (both operands K-contiguous)
 //
 // Tiling for 256 CUs: a workgroup computes a 128-token x 320-column tile (five whole heads),
-// so T = 2048 is exactly 16 x 16 = 256 tiles -- one per CU, no tail wave -- and T = 8192 is
-// exactly four per CU. Eight wavefronts form a 4 x 2 grid (two per SIMD); each owns 32 x 160 of the tile as
+// so T = 2048 is exactly 16 x 16 = 256 tiles -- one per CU, no tail wave (longer inputs take 256-token tiles, see
+// the end of this comment). Eight wavefronts form a 4 x 2 grid (two per SIMD); each owns 32 x 160 of the tile as
 // 1 x 5 v_mfma_f32_32x32x16_bf16 blocks (80 fp32 accumulators per lane) and reads 6 operand
 // fragments from LDS per 5 MFMAs. K is walked in slices of 64 (one 128-byte line per row) through
 // two LDS stages filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers,
@@ -221,15 +221,15 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
 #pragma unroll
     for (int j = 0; j < LPW; ++j) issue_load(it, j);
   };
-  // One k16 step: ten MFMAs on the fragments in buffer `cur`. Behind MFMA m goes the LDS read of fragment m of
-  // the next step (seven of them, into buffer cur ^ 1) and, for m < n, one global->LDS load instruction
-  // (j0 + m) of slice `lit`. The interleaving is pinned with sched_group_barrier, for two reasons:
-  //   * left alone, the compiler hoists all 28 fragment reads of a slice to the top of the iteration; the four
-  //     wavefronts then read 112 KB from LDS in one burst (~900 cycles with no MFMA running) and do their 40
-  //     MFMAs afterwards -- the two costs add up instead of overlapping;
+  // One k16 step: NMF MFMAs on the fragments in buffer `cur`. Behind the MFMAs go the LDS reads of the next step's
+  // fragments (into buffer cur ^ 1) and, for m < n, one global->LDS load instruction (j0 + m) of slice `lit`.
+  // The interleaving is pinned with sched_group_barrier, for two reasons:
+  //   * left alone, the compiler hoists all fragment reads of a slice to the top of the iteration; the wavefronts
+  //     then read them from LDS in one burst with no MFMA running and do their MFMAs afterwards -- the two costs
+  //     add up instead of overlapping;
   //   * a CU takes only so many loads into its queue and a wavefront that issues one more stalls, MFMAs
-  //     included (there is one wavefront per SIMD), until the queue has drained that far; fourteen loads in a
-  //     row do exactly that. Handed out one per MFMA (32 cycles) they never find the queue full.
+  //     included, until the queue has drained that far; a slice's loads in a row do exactly that. Handed out one
+  //     per MFMA (32 cycles) they never find the queue full.
   bf16x8 fa[2][MB], fb[2][5];
   auto read_frag = [&](int cur, const unsigned char* nst, int nkk, int i) {   // fragment i of the next step: activations first
     if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nst + (fa_o[i < MB ? i : 0] ^ (nkk << 5)));
@@ -329,8 +329,8 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // Steady state: slices it+1 .. it+NS-1 are in flight or landed while slice it is multiplied. The one
   // barrier per slice sits before the slice's last k16 step; from there on the stage of slice `it` is free
   // (all reads of it have been issued) and is handed to slice it+NS, whose loads go out behind the MFMAs of
-  // this last step (ten of them) and of the next slice's first step (the other four) -- a whole slice of
-  // MFMAs before they are needed.
+  // this last step and, what does not fit there, of the next slice's first step -- a whole slice of MFMAs
+  // before they are needed.
   issue_loads(NS - 1);
   for (int it = 0; it < n_iter; ++it) {
     const unsigned char* st = smem + (it % NS) * STAGE;
