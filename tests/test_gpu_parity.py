@@ -783,6 +783,22 @@ def test_attention_decode_row_workgroups(gpu, case):
     _attn_case(gpu, seed=11 + c["start_q"], **c)
 
 
+@pytest.mark.parametrize("batch_size,num_keys", [(2, 600), (8, 8192)])
+def test_attention_decode_strided_cache_views(gpu, batch_size, num_keys):
+    """K / V handed over as views of a larger allocation: more tokens and more heads per token than are used, so both
+    the batch stride and the token stride differ from the dense ones (small case: one KV head per workgroup; large
+    case: the row-shaped workgroups, whose wavefronts then read 8 of every 10 heads' worth of each cache row)."""
+    g = torch.Generator().manual_seed(batch_size + num_keys)
+    q = torch.randn(batch_size, 1, 8, 8, 64, generator=g).bfloat16()
+    kc = torch.randn(batch_size, num_keys + 100, 10, 64, generator=g).bfloat16()
+    vc = torch.randn(batch_size, num_keys + 100, 10, 64, generator=g).bfloat16()
+    sinks = torch.randn(64, generator=g).bfloat16()
+    kg, vg = kc.to(gpu)[:, :num_keys, 1:9], vc.to(gpu)[:, :num_keys, 1:9]
+    assert kg.stride(1) == 640 and not kg.is_contiguous()
+    o1 = T.attention_decode(q.to(gpu), kg, vg, sinks.to(gpu), 0.125, None, torch.tensor([num_keys - 1], device=gpu))
+    close(o1, O.attention_decode_ref(q, kc[:, :num_keys, 1:9], vc[:, :num_keys, 1:9], sinks, 0.125, None, num_keys - 1))
+
+
 def test_attention_block_decode_chain(gpu):
     """The whole attention block of a decode step as model.py:471-573 strings it together -- RMSNorm, QKV + bias + RoPE
     with the new k/v written into the cache at `offset`, attention over the cache with sinks (full and windowed),
