@@ -122,9 +122,10 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         ak = [torch.empty(n, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
         av = [torch.empty(n, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
         asink = torch.empty(NQ, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
-        astart = torch.tensor([ctx - 1], dtype=torch.int64, device=dev)
+        astart = torch.tensor([int(os.environ.get("TLLM_BENCH_START_Q", ctx - 1))], dtype=torch.int64, device=dev)
         win = 128 if mode == "win" else None
-        fn = lambda i: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart)
+        hint = int(os.environ["TLLM_BENCH_KV_HINT"]) if "TLLM_BENCH_KV_HINT" in os.environ else None
+        fn = lambda i: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart, kv_len_hint=hint)
         keys = min(ctx, 128) if win else ctx
         nbytes = n * NKV * keys * HD * 2 * 2 + n * NQ * HD * 2 * 2
     elif kind == "rmsnorm":

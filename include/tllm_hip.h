@@ -230,7 +230,13 @@ int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_sc
  * start_q: DEVICE scalar, int32 or int64 (start_q_is_i64), read by the kernel; window 0 = none.
  * Long contexts are split over workgroups: tllm_attention_decode_workspace_bytes(...) says how much device
  * scratch (4-byte aligned) that needs for the same arguments -- 0 for short contexts; the reference allocates its
- * acc/m/l partials per call (:343-345). head_dim must be 64, group <= 16. */
+ * acc/m/l partials per call (:343-345). head_dim must be 64, group <= 16.
+ * The launch (workgroup shape, number of splits) is planned on the host from n_kv_ctx, the size of the cache, like the
+ * reference's SPLIT_K (:311-315); the kernels then use only as many of the planned splits as the context they read
+ * from start_q needs. kv_len_hint (0: none) lets a caller that knows roughly how many keys are visible -- a decode
+ * loop knows its position on the host -- have the launch planned for that instead of for the whole cache: results do
+ * not depend on it, a hint that is too small only costs speed. Pass min(hint, n_kv_ctx) as n_kv_ctx to the three
+ * planning helpers below when a hint is used. */
 int tllm_attention_decode_splits(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window);
 /* Diagnostic: KV heads served by one workgroup for these arguments (8 or 4: one wavefront per head, contiguous
  * cache rows; 0: one KV head per workgroup). No counterpart in the reference. */
@@ -240,7 +246,7 @@ int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, cons
                                int64_t q_row_stride, int64_t out_row_stride, int64_t kv_batch_stride,
                                int64_t kv_token_stride, int64_t batch, int64_t n_kv_ctx, int n_kv_heads, int group,
                                int head_dim, float sm_scale, int window, const void* start_q, int start_q_is_i64,
-                               void* workspace, int64_t workspace_bytes, void* stream);
+                               int64_t kv_len_hint, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* MXFP4 -> bf16 expansion of checkpoint tensors (Checkpoint._get_mxfp4_tensor, weights.py:68-117): blocks
  * [n_blocks][16] bytes, 32 e2m1 values per block with the low nibble first (table weights.py:11-14); scales [n_blocks]

@@ -799,6 +799,28 @@ def test_attention_decode_strided_cache_views(gpu, batch_size, num_keys):
     close(o1, O.attention_decode_ref(q, kc[:, :num_keys, 1:9], vc[:, :num_keys, 1:9], sinks, 0.125, None, num_keys - 1))
 
 
+@pytest.mark.parametrize("batch_size,cache,start_q", [(8, 32768, 4095), (8, 32768, 1000), (8, 32768, 31), (1, 32768, 4095),
+                                                      (2, 16384, 8000), (16, 8192, 2500)])
+@pytest.mark.parametrize("hint", [None, "exact", "small", "large"])
+def test_attention_decode_short_context_in_a_large_cache(gpu, batch_size, cache, start_q, hint):
+    """K / V are the whole preallocated cache and the context is a fraction of it: the launch is planned for the cache
+    (or for the hint), the kernels use the splits the context needs. The result does not depend on the hint, whether
+    it is right, far too small or too large."""
+    g = torch.Generator().manual_seed(batch_size + start_q)
+    q = torch.randn(batch_size, 1, 8, 8, 64, generator=g).bfloat16()
+    k = torch.randn(batch_size, start_q + 1, 8, 64, generator=g).bfloat16()
+    v = torch.randn(batch_size, start_q + 1, 8, 64, generator=g).bfloat16()
+    sinks = torch.randn(64, generator=g).bfloat16()
+    kc = torch.full((batch_size, cache, 8, 64), float("nan"), dtype=torch.bfloat16, device=gpu)   # unused slots must never be read into a result
+    vc = torch.full((batch_size, cache, 8, 64), float("nan"), dtype=torch.bfloat16, device=gpu)
+    kc[:, :start_q + 1] = k.to(gpu)
+    vc[:, :start_q + 1] = v.to(gpu)
+    h = {None: None, "exact": start_q + 1, "small": 100, "large": 10 * cache}[hint]
+    o1 = T.attention_decode(q.to(gpu), kc, vc, sinks.to(gpu), 0.125, None, torch.tensor([start_q], dtype=torch.int64, device=gpu),
+                            kv_len_hint=h)
+    close(o1, O.attention_decode_ref(q, k, v, sinks, 0.125, None, start_q))
+
+
 def test_attention_block_decode_chain(gpu):
     """The whole attention block of a decode step as model.py:471-573 strings it together -- RMSNorm, QKV + bias + RoPE
     with the new k/v written into the cache at `offset`, attention over the cache with sinks (full and windowed),

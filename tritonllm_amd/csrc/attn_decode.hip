@@ -42,9 +42,27 @@ struct AttnArgs {
   const void* start_q;    // device scalar
   int start_is_i64;
   int64_t q_rs, out_rs, kv_bs, kv_ts;
-  int n_kv_ctx, n_kv_heads, group, window, splits;
+  int n_kv_ctx, n_kv_heads, group, window;
+  int splits;             // planned on the host (grid size, workspace stride); the kernels use no more than the context needs
+  int fill, keys_shift;   // the planning inputs that do not depend on the context: splits that fill the CUs, log2 of the target keys per workgroup
   float sm_scale;
 };
+
+// Context splits for `units` independent (batch row, head group) streams over `ctx` visible keys: first enough
+// workgroups to fill the 256 CUs, beyond that about keys_per_wg keys each, never less than 128 keys per split, at most
+// 64. The host plans the launch with it from the size of the cache (or the caller's hint of the current length); the
+// kernels evaluate it again with the length they read from start_q and leave the splits beyond that idle, so a cache
+// allocated for 131072 tokens costs a context of 4096 no more splits than it needs.
+__host__ __device__ inline int attn_fill(int64_t units) { return static_cast<int>((256 + (units > 0 ? units : 1) - 1) / (units > 0 ? units : 1)); }
+
+__host__ __device__ inline int attn_splits_for(int fill, int ctx, int keys_shift) {   // a few 32-bit shifts and compares: the kernels run this
+  const int cap = ((ctx - 1) >> 7) + 1;                        // ctx >= 1
+  const int by_work = ((ctx - 1) >> keys_shift) + 1;
+  int s = fill > by_work ? fill : by_work;
+  s = s < cap ? s : cap;
+  s = s > 1 ? s : 1;
+  return s < 64 ? s : 64;
+}
 
 namespace {
 constexpr int AW = 4;                 // wavefronts per workgroup, HEAD shape
@@ -59,6 +77,19 @@ __device__ __forceinline__ int attn_start_q(const AttnArgs& a) {
   return a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
 }
 
+// Visible keys lo .. hi-1 and the number of splits that take part (<= the planned a.splits).
+__device__ __forceinline__ int attn_live_splits(const AttnArgs& a, int* lo_out, int* hi_out) {
+  const int start_q = attn_start_q(a);
+  int hi = start_q + 1 < a.n_kv_ctx ? start_q + 1 : a.n_kv_ctx;
+  hi = hi > 0 ? hi : 0;
+  int lo = a.window > 0 ? (start_q - a.window + 1 > 0 ? start_q - a.window + 1 : 0) : 0;
+  lo = lo < hi ? lo : hi;
+  *lo_out = lo;
+  *hi_out = hi;
+  const int s = attn_splits_for(a.fill, hi - lo > 0 ? hi - lo : 1, a.keys_shift);
+  return s < a.splits ? s : a.splits;
+}
+
 template <bool ROWS>
 __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(AttnArgs a) {
   __shared__ __align__(16) unsigned char vt[(ROWS ? RW : AW) * VTILE];
@@ -67,22 +98,36 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, g = lane >> 4;
-  // ROWS: blockIdx.x = head group * splits + split, the group's KV heads on the workgroup's wavefronts
-  const int grp = blockIdx.x / a.splits;
-  const int kvh = ROWS ? grp * static_cast<int>(blockDim.x >> 6) + wave : grp;
-  const int split = blockIdx.x - grp * a.splits;
-  const int64_t b = blockIdx.y;
   const int G = a.group;
   const int n_q_heads = a.n_kv_heads * G;
 
-  // ---- key range of this split
-  const int start_q = attn_start_q(a);
-  int hi = start_q + 1 < a.n_kv_ctx ? start_q + 1 : a.n_kv_ctx;
-  hi = hi > 0 ? hi : 0;
-  int lo = a.window > 0 ? (start_q - a.window + 1 > 0 ? start_q - a.window + 1 : 0) : 0;
-  lo = lo < hi ? lo : hi;
+  // ---- key range of this split; the splits the context does not need leave at once (the whole workgroup)
+  // The grid is (head groups x planned splits, batch rows), x fastest. When the context needs fewer splits than were
+  // planned, the workgroups are renumbered so that the live ones are the first live x groups x batch in launch order
+  // -- they then spread over the CUs exactly as a launch planned for this context would, and the rest exit at once
+  // (left where they were launched, live and idle workgroups pile up unevenly: 140 against 89 us at B = 8 with
+  // 32768 of a 131072-token cache in use).
+  int lo, hi;
+  const int live = attn_live_splits(a, &lo, &hi);
+  int grp, split;
+  int64_t b;
+  if (live == a.splits) {
+    grp = blockIdx.x / a.splits;
+    split = blockIdx.x - grp * a.splits;
+    b = blockIdx.y;
+  } else {
+    const unsigned ngrp = gridDim.x / a.splits;
+    const unsigned idx = blockIdx.y * gridDim.x + blockIdx.x, per_row = live * ngrp;
+    if (idx >= per_row * gridDim.y) return;
+    const unsigned bb = idx / per_row, r = idx - bb * per_row;
+    b = bb;
+    grp = r / live;
+    split = r - grp * live;
+  }
+  // ROWS: the group's KV heads sit on the workgroup's wavefronts
+  const int kvh = ROWS ? grp * static_cast<int>(blockDim.x >> 6) + wave : grp;
   const int len = hi - lo;
-  int chunk = (len + a.splits - 1) / a.splits;
+  int chunk = (len + live - 1) / live;
   chunk = (chunk + 31) & ~31;                                 // whole 32-key blocks per split
   const int s_lo = lo + split * chunk < hi ? lo + split * chunk : hi;
   const int s_hi = s_lo + chunk < hi ? s_lo + chunk : hi;
@@ -297,26 +342,34 @@ __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(AttnArgs a, int 
   const int n_q_heads = a.n_kv_heads * a.group;
   const int64_t split_stride = static_cast<int64_t>(batch) * n_q_heads * PART;
   const float* p0 = a.part + (b * n_q_heads + head) * PART;
-  const bool has = lane < a.splits;
-  const float m_s = has ? p0[lane * split_stride + 64] : kNegBig;
-  const float l_s = has ? p0[lane * split_stride + 65] : 0.f;
+  // (max, sum) of every planned split and the accumulators of the first eight are requested before start_q is known
+  // (one memory round trip for up to eight splits, not three); the records of splits that did not take part are
+  // whatever the workspace held and are masked out once the number of live splits is known.
+  const float m_raw = lane < a.splits ? p0[lane * split_stride + 64] : kNegBig;
+  const float l_raw = lane < a.splits ? p0[lane * split_stride + 65] : 0.f;
+  float v[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) v[u] = p0[(u < a.splits ? u : a.splits - 1) * split_stride + lane];
+  int lo, hi;
+  const int live = attn_live_splits(a, &lo, &hi);            // the splits that wrote a record
+  const bool has = lane < live;
+  const float m_s = has ? m_raw : kNegBig;
+  const float l_s = has ? l_raw : 0.f;
   float m_all = m_s;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, o, 64));
   const float f_s = __expf(m_s - m_all);                     // 0 for the lanes without a split
   const float l_all = wave_sum(l_s * f_s);
   float o = 0.f;
-  for (int s0 = 0; s0 < a.splits; s0 += 8) {
-    float v[8];
+  for (int s0 = 0; s0 < live; s0 += 8) {
+    if (s0 > 0) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int s = s0 + u < a.splits ? s0 + u : a.splits - 1;
-      v[u] = p0[s * split_stride + lane];
+      for (int u = 0; u < 8; ++u) v[u] = p0[(s0 + u < live ? s0 + u : live - 1) * split_stride + lane];
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const float f = __shfl(f_s, s0 + u < a.splits ? s0 + u : 0, 64);
-      o += (s0 + u < a.splits) ? v[u] * f : 0.f;
+      const float f = __shfl(f_s, s0 + u < live ? s0 + u : 0, 64);
+      o += (s0 + u < live) ? v[u] * f : 0.f;
     }
   }
   const float sink = a.sinks ? static_cast<float>(a.sinks[head]) : 0.f;
@@ -339,36 +392,25 @@ using namespace tllm;
 // B = 1: HEAD throughout). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
 // 2048 (HEAD) keys per workgroup, never less than 128 keys per split.
 // A sliding window bounds the context.
-struct AttnPlan { int heads_per_wg; int splits; };   // heads_per_wg 0: the HEAD shape
+struct AttnPlan { int heads_per_wg; int splits; int fill; int keys_shift; };   // heads_per_wg 0: the HEAD shape
 
 static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
   const int64_t ctx = (window > 0 && window < n_kv_ctx) ? window : n_kv_ctx;
-  const int64_t cap = (ctx + 127) / 128;
-  auto splits_for = [&](int64_t units, int64_t keys_per_wg) {
-    const int64_t by_work = (ctx + keys_per_wg - 1) / keys_per_wg;
-    units = units > 0 ? units : 1;
-    const int64_t fill = (256 + units - 1) / units;
-    int64_t s = fill > by_work ? fill : by_work;
-    if (s > cap) s = cap;
-    if (s < 1) s = 1;
-    if (s > 64) s = 64;
-    return static_cast<int>(s);
-  };
   // eight or four KV heads per workgroup: whichever fills the machine with the longest splits (ties: the wider one)
-  AttnPlan best{0, 0};
+  AttnPlan best{0, 0, 0, 0};
   int64_t best_keys = 0;
   for (int hpw = RW; hpw >= 4; hpw >>= 1) {
     if (n_kv_heads % hpw != 0) continue;
     const int64_t units = batch * (n_kv_heads / hpw);
-    const int s = splits_for(units, 1024);
+    const int s = attn_splits_for(attn_fill(units), static_cast<int>(ctx), 10);
     const int64_t keys = ctx / s;
     if (units * s >= 224 && keys >= 512 && keys > best_keys) {
-      best = {hpw, s};
+      best = {hpw, s, attn_fill(units), 10};
       best_keys = keys;
     }
   }
   if (best.heads_per_wg) return best;
-  return {0, splits_for(batch * n_kv_heads, 2048)};
+  return {0, attn_splits_for(attn_fill(batch * n_kv_heads), static_cast<int>(ctx), 11), attn_fill(batch * n_kv_heads), 11};
 }
 
 extern "C" int tllm_attention_decode_heads_per_workgroup(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
@@ -387,7 +429,8 @@ extern "C" int64_t tllm_attention_decode_workspace_bytes(int64_t batch, int n_q_
 extern "C" int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, const void* sinks, void* out, int64_t q_row_stride,
                                           int64_t out_row_stride, int64_t kv_batch_stride, int64_t kv_token_stride, int64_t batch,
                                           int64_t n_kv_ctx, int n_kv_heads, int group, int head_dim, float sm_scale, int window,
-                                          const void* start_q, int start_q_is_i64, void* workspace, int64_t workspace_bytes, void* stream) {
+                                          const void* start_q, int start_q_is_i64, int64_t kv_len_hint, void* workspace,
+                                          int64_t workspace_bytes, void* stream) {
   TLLM_REQUIRE(batch >= 0 && n_kv_ctx >= 1 && n_kv_ctx < (1ll << 31) && n_kv_heads >= 1, TLLM_E_SHAPE,
                "attention_decode: batch %lld, n_kv_ctx %lld, n_kv_heads %d", (long long)batch, (long long)n_kv_ctx, n_kv_heads);
   TLLM_REQUIRE(head_dim == 64, TLLM_E_SHAPE, "attention_decode: head_dim %d (only 64 is built)", head_dim);
@@ -416,9 +459,13 @@ extern "C" int tllm_attention_decode_bf16(const void* q, const void* k, const vo
   a.group = group;
   a.window = window;
   a.sm_scale = sm_scale;
-  const AttnPlan plan = attn_plan(batch, n_kv_heads, n_kv_ctx, window);
+  TLLM_REQUIRE(kv_len_hint >= 0, TLLM_E_ARG, "attention_decode: kv_len_hint %lld", (long long)kv_len_hint);
+  const int64_t plan_ctx = (kv_len_hint > 0 && kv_len_hint < n_kv_ctx) ? kv_len_hint : n_kv_ctx;
+  const AttnPlan plan = attn_plan(batch, n_kv_heads, plan_ctx, window);
   a.splits = plan.splits;
-  const int64_t need = tllm_attention_decode_workspace_bytes(batch, n_kv_heads * group, n_kv_heads, n_kv_ctx, window);
+  a.fill = plan.fill;
+  a.keys_shift = plan.keys_shift;
+  const int64_t need = tllm_attention_decode_workspace_bytes(batch, n_kv_heads * group, n_kv_heads, plan_ctx, window);
   TLLM_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 4 == 0), TLLM_E_ARG,
                "attention_decode: workspace of %lld bytes needed (tllm_attention_decode_workspace_bytes), got %lld", (long long)need,
                (long long)workspace_bytes);

@@ -550,11 +550,16 @@ def unembedding_decode_fp8_argmax_forward(hidden, weight_fp8, weight_scale):
 
 # --------------------------------------------------------------------------------------- decode attention
 def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Tensor | None, sm_scale: float,
-                     bandwidth: int | None, start_q: torch.Tensor) -> torch.Tensor:
+                     bandwidth: int | None, start_q: torch.Tensor, kv_len_hint: int | None = None) -> torch.Tensor:
     """One new token per batch row against the KV cache, with sinks and an optional sliding window
     (attention_tt_decode.py:290-408): ``q [bs, 1, n_kv_heads, repeat_kv, 64]``, ``k, v [bs, n_kv_ctx, n_kv_heads, 64]``,
     ``sinks [n_kv_heads * repeat_kv]`` bf16, ``start_q`` a device tensor of one int32/int64 element (read on the
-    device), ``bandwidth`` the sliding window (``None`` / 0: none). Returns ``[bs, 1, n_heads * 64]`` (pooled)."""
+    device), ``bandwidth`` the sliding window (``None`` / 0: none). Returns ``[bs, 1, n_heads * 64]`` (pooled).
+
+    ``k`` / ``v`` are usually the whole preallocated cache; the launch is planned from its size and the kernels then use
+    only the splits the context at ``start_q`` needs. ``kv_len_hint`` (an extension; the host's idea of how many keys
+    are visible, e.g. the decode loop's position + 1) plans the launch for that length instead, which is faster when
+    the context is far shorter than the cache; the result never depends on it."""
     _on_gpu(q, k, v, sinks, start_q)
     assert len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64)
     bs, n_ctx, n_kv_heads, repeat_kv, head_dim_q = q.shape
@@ -584,12 +589,14 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: t
         sinks = sinks if sinks.is_contiguous() else sinks.contiguous()
     window = int(bandwidth) if bandwidth else 0
     o = scratch_pool.get((bs, n_heads * 64), q.dtype, q.device)
-    nbytes = lib().tllm_attention_decode_workspace_bytes(bs, n_heads, n_kv_heads, n_kv_ctx, window)
+    hint = 0 if kv_len_hint is None else max(int(kv_len_hint), 1)
+    plan_ctx = min(hint, n_kv_ctx) if hint else n_kv_ctx
+    nbytes = lib().tllm_attention_decode_workspace_bytes(bs, n_heads, n_kv_heads, plan_ctx, window)
     work = scratch_pool.get((max(nbytes // 4, 1),), torch.float32, q.device) if nbytes else None
     rc = lib().tllm_attention_decode_bf16(q2.data_ptr(), k.data_ptr(), v.data_ptr(), sinks.data_ptr() if sinks is not None else None,
                                           o.data_ptr(), q2.stride(0), o.stride(0), k.stride(0), k.stride(1), bs, n_kv_ctx, n_kv_heads,
                                           repeat_kv, 64, float(sm_scale), window, start_q.data_ptr(), int(start_q.dtype == torch.int64),
-                                          work.data_ptr() if work is not None else None, nbytes, _stream())
+                                          hint, work.data_ptr() if work is not None else None, nbytes, _stream())
     check(rc, "attention_decode")
     return o.view(bs, 1, n_heads * 64)
 
