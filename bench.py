@@ -396,6 +396,17 @@ def main() -> int:
             bench_kernel(f"attention_decode_{'win' if win else 'ctx'}{ctx}_B{r}",
                          lambda i, aq=aq, ak=ak, av=av, asink=asink, astart=astart, win=win: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart),
                          r * NKV * keys * HD * 2 * 2 + r * NQ * HD * 2 * 2, n=96)
+            if ctx == 32768:
+                # the model's usual case: the cache is allocated for many more tokens than are in use (4096 of 32768 here)
+                astart4k = torch.tensor([4095], dtype=torch.int64, device=dev)
+                nb4k = r * NKV * 4096 * HD * 2 * 2 + r * NQ * HD * 2 * 2
+                bench_kernel(f"attention_decode_4096of{ctx}_B{r}",
+                             lambda i, aq=aq, ak=ak, av=av, asink=asink: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, None, astart4k),
+                             nb4k, n=96)
+                bench_kernel(f"attention_decode_4096of{ctx}_hint_B{r}",
+                             lambda i, aq=aq, ak=ak, av=av, asink=asink: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, None, astart4k,
+                                                                                            kv_len_hint=4096),
+                             nb4k, n=96)
             del ak, av
         # unembedding over the full vocabulary (the embedding table doubles as the [201088, 2880] weight: 1.16 GB per launch)
         for r in (1, 8):
