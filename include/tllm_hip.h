@@ -248,6 +248,20 @@ int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, cons
                                int head_dim, float sm_scale, int window, const void* start_q, int start_q_is_i64,
                                int64_t kv_len_hint, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Prefill attention with sinks and an optional sliding window: n_q query positions per batch row against the keys
+ * written so far. Replaces attention (attention_tt.py:166-236, kernel :17-164; definition attention_ref.py:4-42).
+ * q [batch, n_q, n_kv_heads * group, 64] with batch / token strides in elements (heads adjacent: the layout the QKV
+ * projection writes), k / v [batch, n_kv_ctx, n_kv_heads, 64] with batch / token strides (a view of the KV cache
+ * will do), sinks [n_kv_heads * group] bf16 or NULL (logit 0, :103-106), out [batch, n_q, n_kv_heads * group * 64].
+ * Query i sits at position start_q + i (start_q: one int32 / int64 element in device memory, read on the device) and
+ * sees keys n <= position, n < n_kv_ctx and, when window > 0, n > position - window. Unlike the reference, no
+ * transposed or padded copies of q, k, v are made. head_dim must be 64, sm_scale positive. */
+int tllm_attention_prefill_bf16(const void* q, const void* k, const void* v, const void* sinks, void* out,
+                                int64_t q_batch_stride, int64_t q_token_stride, int64_t out_batch_stride,
+                                int64_t out_token_stride, int64_t kv_batch_stride, int64_t kv_token_stride,
+                                int64_t batch, int64_t n_q, int64_t n_kv_ctx, int n_kv_heads, int group, int head_dim,
+                                float sm_scale, int window, const void* start_q, int start_q_is_i64, void* stream);
+
 /* MXFP4 -> bf16 expansion of checkpoint tensors (Checkpoint._get_mxfp4_tensor, weights.py:68-117): blocks
  * [n_blocks][16] bytes, 32 e2m1 values per block with the low nibble first (table weights.py:11-14); scales [n_blocks]
  * e8m0 bytes (bias 127); out [n_blocks][32] bf16 = FP4[nibble] * 2^(scale - 127), formed in fp32 and rounded once, as

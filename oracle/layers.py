@@ -33,6 +33,8 @@ force and special cases -- in ``tests/test_oracle_pins.py``:
                                       interleaved == chunked under permutation
     attention_decode_ref              float64 brute force per head, causal / window key ranges, sink limits
                                       (-> -inf: plain softmax; -> +inf: zero output), equal keys => mean of values
+    attention_ref                     every query row equals attention_decode_ref at position start_q + i; float64 brute
+                                      force with a window and a key count below the last position; no visible key => 0
     out_residual_ref                  linear_ref + an fp32 add; float64 brute force
     quantize_fp8_rows_ref /           all 256 e4m3 codes against the OCP bit formula, row maxima map to
     dequant_fp8_ref                   +-448, round-trip error within half a step of the format
@@ -177,6 +179,33 @@ def attention_decode_ref(query: torch.Tensor, key: torch.Tensor, value: torch.Te
     z = w.sum(dim=-1, keepdim=True) + torch.exp(sink - top)
     out = torch.einsum("bhmk,bkhd->bhmd", w / z, value.to(torch.float32))
     return out.reshape(bs, 1, n_kv * groups * hd)
+
+
+def attention_ref(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, sinks: torch.Tensor | None, sm_scale: float = 0.125,
+                  sliding_window: int | None = None, start_q: int = 0) -> torch.Tensor:
+    """attention_ref.py:4-42 for any number of query positions (the prefill case), fp32, returned as fp32
+    ``[bs, n_queries, heads*hd]``.
+
+    query ``[bs, n_queries, kv_heads, groups, hd]``, key/value ``[bs, n_keys, kv_heads, hd]``, sinks ``[kv_heads*groups]``
+    (``None``: logit 0, attention_tt.py:103-106). Query ``i`` sits at position ``start_q + i`` (:20); keys after that
+    position are masked (:21-22), keys older than ``position - sliding_window + 1`` too (:24-26); the sink joins the
+    softmax denominator but contributes no value (:31-36). A query that sees no key yields zeros."""
+    bs, nq, n_kv, groups, hd = query.shape
+    n_keys = key.shape[1]
+    sink = torch.zeros(n_kv * groups) if sinks is None else sinks.to(torch.float32)
+    sink = sink.view(1, n_kv, groups, 1, 1)
+    pos_k = torch.arange(n_keys)
+    pos_q = torch.arange(nq) + int(start_q)
+    masked = pos_k[None, :] > pos_q[:, None]
+    if sliding_window:
+        masked = masked | (pos_k[None, :] < pos_q[:, None] - sliding_window + 1)
+    logits = torch.einsum("bqhmd,bkhd->bhmqk", query.to(torch.float32), key.to(torch.float32)) * sm_scale
+    logits = logits.masked_fill(masked[None, None, None, :, :], float("-inf"))
+    top = torch.maximum(sink, logits.max(dim=-1, keepdim=True).values)
+    w = torch.exp(logits - top)
+    z = w.sum(dim=-1, keepdim=True) + torch.exp(sink - top)
+    out = torch.einsum("bhmqk,bkhd->bqhmd", w / z, value.to(torch.float32))
+    return out.reshape(bs, nq, n_kv * groups * hd)
 
 
 def quantize_fp8_rows_ref(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

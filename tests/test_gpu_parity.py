@@ -821,6 +821,91 @@ def test_attention_decode_short_context_in_a_large_cache(gpu, batch_size, cache,
     close(o1, O.attention_decode_ref(q, k, v, sinks, 0.125, None, start_q))
 
 
+def _attn_prefill_case(gpu, batch_size, num_queries, num_keys, sliding_window, start_q, start_dtype=torch.int32, seed=0, with_sinks=True,
+                       groups=8, kv_heads=8):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(batch_size, num_queries, kv_heads, groups, 64, generator=g).bfloat16()
+    k = torch.randn(batch_size, num_keys, kv_heads, 64, generator=g).bfloat16()
+    v = torch.randn(batch_size, num_keys, kv_heads, 64, generator=g).bfloat16()
+    sinks = torch.randn(kv_heads * groups, generator=g).bfloat16() if with_sinks else None
+    o1 = T.attention(q.to(gpu), k.to(gpu), v.to(gpu), sinks.to(gpu) if with_sinks else None, 0.125, sliding_window,
+                     torch.tensor([start_q], dtype=start_dtype, device=gpu))
+    o2 = O.attention_ref(q, k, v, sinks, 0.125, sliding_window, start_q)
+    assert o1.shape == (batch_size, num_queries, kv_heads * groups * 64) and o1.dtype == torch.bfloat16
+    # the reference's own bar (attention_tt.py:268) and the tolerance of the other bf16 outputs of this library
+    torch.testing.assert_close(o1.float().cpu(), o2.bfloat16().float(), atol=1e-2, rtol=1e-1)
+    close(o1, o2)
+
+
+@pytest.mark.parametrize("batch_size", [1, 2])
+@pytest.mark.parametrize("num_queries", [1, 16])
+@pytest.mark.parametrize("num_keys", [128, 32])
+@pytest.mark.parametrize("sliding_window", [None, 128])
+@pytest.mark.parametrize("start_q", [0, 5])
+def test_attention_prefill_eq(gpu, batch_size, num_queries, num_keys, sliding_window, start_q):
+    """The reference's test_eq (attention_tt.py:245-268), same parameter grid."""
+    _attn_prefill_case(gpu, batch_size, num_queries, num_keys, sliding_window, start_q, seed=start_q + num_keys + num_queries)
+
+
+@pytest.mark.parametrize("case", [
+    dict(batch_size=1, num_queries=300, num_keys=300, sliding_window=None, start_q=0),            # ragged last tile and block
+    dict(batch_size=2, num_queries=257, num_keys=257, sliding_window=128, start_q=0),             # the model's sliding layers
+    dict(batch_size=1, num_queries=1024, num_keys=1024, sliding_window=128, start_q=0),
+    dict(batch_size=1, num_queries=200, num_keys=1000, sliding_window=None, start_q=800, start_dtype=torch.int64),   # a later chunk of a long prompt
+    dict(batch_size=1, num_queries=200, num_keys=1000, sliding_window=100, start_q=800),
+    dict(batch_size=2, num_queries=130, num_keys=400, sliding_window=None, start_q=100),          # keys beyond the last query are never visible
+    dict(batch_size=1, num_queries=100, num_keys=60, sliding_window=None, start_q=0),             # fewer keys than positions
+    dict(batch_size=1, num_queries=100, num_keys=60, sliding_window=16, start_q=30),              # the last queries see no key at all: zeros
+    dict(batch_size=2, num_queries=150, num_keys=150, sliding_window=None, start_q=0, with_sinks=False),
+    dict(batch_size=2, num_queries=150, num_keys=150, sliding_window=64, start_q=0, groups=3),    # odd group: one head per wavefront
+    dict(batch_size=1, num_queries=150, num_keys=150, sliding_window=None, start_q=0, groups=1, kv_heads=4),
+    dict(batch_size=3, num_queries=129, num_keys=140, sliding_window=None, start_q=11, groups=4, kv_heads=2),
+], ids=lambda c: "-".join(f"{k[0]}{v}" for k, v in c.items() if not isinstance(v, torch.dtype)))
+def test_attention_prefill_shapes(gpu, case):
+    _attn_prefill_case(gpu, seed=3 + case["num_queries"] + case["start_q"], **case)
+
+
+def test_attention_prefill_views_of_the_qkv_buffer_and_the_cache(gpu):
+    """q as a slice of the fused projection output, k / v as slices of a larger cache whose other slots hold NaN: the
+    kernel reads them in place (batch and token strides) and never touches a key no query can see."""
+    g = torch.Generator().manual_seed(21)
+    bs, n_tok, start = 2, 200, 40
+    qkv = torch.randn(bs, n_tok, 5120, generator=g).bfloat16()
+    kc = torch.full((bs, 512, 10, 64), float("nan")).bfloat16()
+    vc = torch.full((bs, 512, 10, 64), float("nan")).bfloat16()
+    kc[:, : start + n_tok, 1:9] = torch.randn(bs, start + n_tok, 8, 64, generator=g).bfloat16()
+    vc[:, : start + n_tok, 1:9] = torch.randn(bs, start + n_tok, 8, 64, generator=g).bfloat16()
+    sinks = torch.randn(64, generator=g).bfloat16()
+    q = qkv[:, :, :4096].view(bs, n_tok, 8, 8, 64)
+    qg = qkv.to(gpu)[:, :, :4096].view(bs, n_tok, 8, 8, 64)
+    assert not qg.is_contiguous()
+    kg, vg = kc.to(gpu)[:, :, 1:9], vc.to(gpu)[:, :, 1:9]
+    for window in (None, 128):
+        o1 = T.attention(qg, kg, vg, sinks.to(gpu), 0.125, window, torch.tensor([start], device=gpu))
+        o2 = O.attention_ref(q, kc[:, : start + n_tok, 1:9], vc[:, : start + n_tok, 1:9], sinks, 0.125, window, start)
+        close(o1, o2)
+
+
+def test_attention_prefill_full_prompt(gpu):
+    """The benchmark shape: one prompt of 2048 tokens, 64 query heads over 8 KV heads, both kinds of layer."""
+    _attn_prefill_case(gpu, 1, 2048, 2048, None, 0, seed=31)
+    _attn_prefill_case(gpu, 1, 2048, 2048, 128, 0, seed=32)
+
+
+def test_attention_prefill_argument_errors(gpu):
+    q = torch.zeros(1, 16, 8, 8, 64, dtype=torch.bfloat16, device=gpu)
+    k = torch.zeros(1, 16, 8, 64, dtype=torch.bfloat16, device=gpu)
+    s = torch.zeros(64, dtype=torch.bfloat16, device=gpu)
+    st = torch.tensor([0], device=gpu)
+    with pytest.raises(AssertionError):
+        T.attention(q, k, k[:, :8], s, 0.125, None, st)                       # k and v disagree
+    with pytest.raises(AssertionError):
+        T.attention(q, k, k, s[:32], 0.125, None, st)                         # one sink per query head
+    with pytest.raises((AssertionError, RuntimeError)):
+        T.attention(q, k, k, s, -0.125, None, st)                             # the kernel folds the scale into exp2: positive only
+    assert T.attention(q[:, :0], k, k, s, 0.125, None, st).shape == (1, 0, 4096)
+
+
 def test_attention_block_decode_chain(gpu):
     """The whole attention block of a decode step as model.py:471-573 strings it together -- RMSNorm, QKV + bias + RoPE
     with the new k/v written into the cache at `offset`, attention over the cache with sinks (full and windowed),

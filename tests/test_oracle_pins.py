@@ -307,6 +307,41 @@ def test_attention_decode_ref_pins():
     torch.testing.assert_close(out, v.float().mean(dim=1)[:, :, None, :].expand(-1, -1, groups, -1), rtol=1e-5, atol=1e-6)
 
 
+def test_attention_ref_pins():
+    g = torch.Generator().manual_seed(12)
+    bs, n_keys, n_kv, groups, hd, nq = 2, 24, 2, 3, 16, 9
+    q = torch.randn(bs, nq, n_kv, groups, hd, generator=g).bfloat16()
+    k = torch.randn(bs, n_keys, n_kv, hd, generator=g).bfloat16()
+    v = torch.randn(bs, n_keys, n_kv, hd, generator=g).bfloat16()
+    sinks = torch.randn(n_kv * groups, generator=g).bfloat16()
+    # row i of the many-query form is the one-query form at position start + i (which is pinned by brute force above)
+    for window, start in ((None, 0), (None, 15), (5, 0), (5, 11), (100, 3)):
+        got = O.attention_ref(q, k, v, sinks, 0.25, window, start)
+        for i in range(nq):
+            one = O.attention_decode_ref(q[:, i : i + 1], k, v, sinks, 0.25, window, start + i)
+            torch.testing.assert_close(got[:, i : i + 1], one, rtol=1e-5, atol=1e-6)
+    # float64 brute force where the last positions lie beyond the keys (start + i >= n_keys) and a window cuts the front
+    window, start = 6, 18
+    got = O.attention_ref(q, k, v, sinks, 0.25, window, start).view(bs, nq, n_kv, groups, hd)
+    for b in range(bs):
+        for i in range(nq):
+            p = start + i
+            vis = [n for n in range(n_keys) if n <= p and n >= p - window + 1]
+            for h in range(n_kv):
+                for m in range(groups):
+                    sk = float(sinks[h * groups + m])
+                    sc = [0.25 * sum(float(q[b, i, h, m, d]) * float(k[b, n, h, d]) for d in range(hd)) for n in vis]
+                    top = max(sc + [sk])
+                    wts = [math.exp(x - top) for x in sc]
+                    z = sum(wts) + math.exp(sk - top)
+                    want = [sum(w * float(v[b, n, h, d]) for w, n in zip(wts, vis)) / z for d in range(hd)]
+                    torch.testing.assert_close(got[b, i, h, m].double(), torch.tensor(want, dtype=torch.float64), rtol=1e-4, atol=1e-5)
+    # positions past the keys by more than the window see nothing: zeros (only the sink is left)
+    assert O.attention_ref(q, k, v, sinks, 0.25, 4, 40).abs().max() == 0
+    # no sinks = logit 0
+    torch.testing.assert_close(O.attention_ref(q, k, v, None, 0.25, None, 2), O.attention_ref(q, k, v, torch.zeros(6), 0.25, None, 2))
+
+
 def _e2m1(nib: int) -> float:
     """OCP MX e2m1: sign bit 3, two exponent bits (bias 1), one mantissa bit; exponent 0 is subnormal (0 or 0.5)."""
     s, e, m = nib >> 3, (nib >> 1) & 3, nib & 1

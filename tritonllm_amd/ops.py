@@ -601,6 +601,54 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: t
     return o.view(bs, 1, n_heads * 64)
 
 
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Tensor | None, sm_scale: float,
+              bandwidth: int | None, start_q: torch.Tensor) -> torch.Tensor:
+    """Prefill attention with sinks and an optional sliding window (attention, attention_tt.py:166-236):
+    ``q [bs, n_ctx, n_kv_heads, repeat_kv, 64]``, ``k, v [bs, n_kv_ctx, n_kv_heads, 64]``, ``sinks [n_heads]`` bf16,
+    ``start_q`` a device tensor of one int32/int64 element (query ``i`` sits at position ``start_q + i``; read on the
+    device), ``bandwidth`` the sliding window (``None`` / 0: none). Returns ``[bs, n_ctx, n_heads * 64]`` (pooled).
+
+    ``q`` may be a view into the fused QKV output and ``k`` / ``v`` views of the cache: the kernel takes batch and
+    token strides, so none of the reference's transposed, padded copies (:178-191) is made."""
+    _on_gpu(q, k, v, sinks, start_q)
+    assert len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64)
+    bs, n_ctx, n_kv_heads, repeat_kv, head_dim_q = q.shape
+    bs_k, n_kv_ctx, n_kv_heads_k, head_dim_k = k.shape
+    bs_v, n_kv_ctx_v, n_kv_heads_v, head_dim_v = v.shape
+    assert bs == bs_k == bs_v and n_kv_ctx == n_kv_ctx_v
+    assert n_kv_heads == n_kv_heads_k == n_kv_heads_v
+    assert head_dim_q == head_dim_k == head_dim_v
+    assert head_dim_q in {16, 32, 64, 128, 256}
+    if head_dim_q != 64:
+        raise NotImplementedError("attention: the HIP kernel is built for head_dim 64")
+    assert q.dtype == _BF16 and k.dtype == _BF16 and v.dtype == _BF16 and (sinks is None or sinks.dtype == _BF16)
+    n_heads = n_kv_heads * repeat_kv
+
+    def dense_q(t):
+        ok = t.stride(4) == 1 and t.stride(3) == 64 and t.stride(2) == 64 * repeat_kv and t.stride(1) % 8 == 0 and t.stride(0) % 8 == 0
+        return t if ok and t.data_ptr() % 16 == 0 else t.contiguous()
+
+    def dense_heads(t):
+        ok = t.stride(3) == 1 and t.stride(2) == 64 and t.stride(1) % 8 == 0 and t.stride(0) % 8 == 0
+        return t if ok and t.data_ptr() % 16 == 0 else t.contiguous()
+
+    q = dense_q(q)
+    k, v = dense_heads(k), dense_heads(v)
+    if k.stride() != v.stride():
+        k, v = k.contiguous(), v.contiguous()
+    if sinks is not None:
+        assert sinks.shape == (n_heads,)
+        sinks = sinks if sinks.is_contiguous() else sinks.contiguous()
+    window = int(bandwidth) if bandwidth else 0
+    o = scratch_pool.get((bs, n_ctx, n_heads * 64), q.dtype, q.device)
+    rc = lib().tllm_attention_prefill_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), sinks.data_ptr() if sinks is not None else None,
+                                           o.data_ptr(), q.stride(0), q.stride(1), o.stride(0), o.stride(1), k.stride(0), k.stride(1),
+                                           bs, n_ctx, n_kv_ctx, n_kv_heads, repeat_kv, 64, float(sm_scale), window, start_q.data_ptr(),
+                                           int(start_q.dtype == torch.int64), _stream())
+    check(rc, "attention")
+    return o
+
+
 def mxfp4_dequant(blocks: torch.Tensor, scales: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """Expand MXFP4 checkpoint data to bf16 (Checkpoint._get_mxfp4_tensor, weights.py:68-117).
 
