@@ -115,6 +115,20 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         else:
             fn = lambda i: T.unembedding_decode_forward(ux, table)
             nbytes = bytes_of["unembed"](n)
+    elif kind.startswith("attention_prefill_"):
+        # attention_prefill_ctx<T>_B<n> (T-token prompts, every earlier key visible) or attention_prefill_win<T>_B<n> (window 128)
+        mode, ctx = kind[len("attention_prefill_"):][:3], int(kind[len("attention_prefill_") + 3:])
+        qkv = [torch.empty(n, ctx, QKV_DIM, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(2)]
+        asink = torch.empty(NQ, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        astart = torch.zeros(1, dtype=torch.int64, device=dev)
+        win = 128 if mode == "win" else None
+        # q, k and v are the three column ranges of the fused projection's output, read in place
+        views = [(t[:, :, :NQ * HD].view(n, ctx, NKV, NQ // NKV, HD), t[:, :, NQ * HD:(NQ + NKV) * HD].view(n, ctx, NKV, HD),
+                  t[:, :, (NQ + NKV) * HD:].view(n, ctx, NKV, HD)) for t in qkv]
+        fn = lambda i: T.attention(*views[i % 2], asink, 0.125, win, astart)
+        pairs = sum(min(i + 1, win) if win else i + 1 for i in range(ctx))
+        flops = 4.0 * n * NQ * HD * pairs
+        nbytes = n * ctx * (QKV_DIM + NQ * HD) * 2
     elif kind.startswith("attention_decode_"):
         # attention_decode_ctx<L>_B<n> (full causal context of L keys) or attention_decode_win<L>_B<n> (window 128 inside a cache of L)
         mode, ctx = kind[len("attention_decode_"):][:3], int(kind[len("attention_decode_") + 3:])
@@ -162,7 +176,7 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
     row = {"kernel": name, "us": round(sec * 1e6, 3), "launches_per_replay": reps}
     if nbytes is not None:
         row["GB/s"] = round(nbytes / sec / 1e9, 1)
-    if flops is not None and kind.endswith("prefill"):
+    if flops is not None and "prefill" in kind:
         row["TFLOP/s"] = round(flops / sec / 1e12, 1)
         row["mfma_frac"] = round(flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
     print(json.dumps(row))

@@ -17,9 +17,12 @@
 //     per 32-key block, so the running maximum, the running sum and the rescale factor of the online softmax are
 //     lane-local apart from one exchange between the two half-wavefronts;
 //   * those accumulator registers are, pairwise, the B operand (P^T) of O^T = V^T . P^T when the MFMA's k slots are read
-//     as a permutation of the block's keys, so P never leaves the registers; V is written into LDS transposed
-//     ([d][key], keys in that permuted order, two keys per 32-bit write) so that the A operand is one 16-byte read;
-//   * both tiles are XOR-swizzled in 16-byte chunks: fragment reads are conflict-free;
+//     as a permutation of the block's keys, so P never leaves the registers; V stays row-major in LDS and the A operand
+//     (V^T: lane = d, 8 keys) comes out of two transposing reads (ds_read_b64_tr_b16: within 16 lanes, lane i receives
+//     element i % 4 of the 8 bytes addressed by lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4);
+//   * the running maximum is only raised when a block exceeds it by more than 2^8 (exponents stay far from overflow, the
+//     result is the same quotient), so the accumulator is almost never rescaled;
+//   * both tiles are XOR-swizzled in 16-byte chunks: fragment reads are conflict-free (K) or at the two-pass minimum (V);
 //   * the KV head is the fastest-varying part of the workgroup index, so with eight KV heads each XCD's L2 holds the
 //     K and V of one head; the query tiles with the most keys to visit are launched first.
 // start_q is read from device memory (int32 or int64).
@@ -44,38 +47,61 @@ namespace {
 constexpr int PBM = 128;              // queries per workgroup
 constexpr int PBN = 64;               // keys per block
 constexpr int KT_BYTES = PBN * 128;   // K tile [key][64 d]
-constexpr int VT_BYTES = 64 * 128;    // V^T tile [d][64 keys]
+constexpr int VT_BYTES = PBN * 128;   // V tile [key][64 d]
 constexpr int PSTAGE = KT_BYTES + VT_BYTES;
+constexpr int NSTG = 4;               // LDS stages: three blocks in flight behind the one being computed
 constexpr float kLog2e = 1.4426950408889634f;
 }  // namespace
 
-// 16-byte chunk swizzle of a V^T row: consecutive rows (fragment reads) and rows eight apart (the transposing writes)
-// both land on distinct chunks.
-__device__ __forceinline__ int vt_swizzle(int d) { return ((d >> 1) ^ (d >> 3)) & 7; }
+constexpr float kRaise = 8.f;         // log2 units by which a block must exceed the running maximum to move it
 
-template <int NH>
-__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a) {
-  __shared__ __align__(16) unsigned char smem[2 * PSTAGE];
+// 16-byte chunk swizzle of a V row: a transposing read touches eight consecutive keys x 64 bytes; this spreads them
+// over the banks evenly.
+__device__ __forceinline__ int v_swizzle(int key) { return (((key >> 1) & 1) << 2) | ((key >> 2) & 3); }
+
+// The value lane l ^ 32 holds: lanes l and l ^ 32 carry the two halves of one query's keys.
+__device__ __forceinline__ float other_half(float x, int high) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // r[0]: the low half's x in every lane, r[1]: the high half's
+  return __builtin_bit_cast(float, high ? r[0] : r[1]);
+}
+
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4;
+
+// NH: query heads per wavefront; HW: sets of four wavefronts, each set with its own NH heads of the same queries
+template <int NH, int HW>
+__global__ __launch_bounds__(256 * HW, HW == 1 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
+  constexpr int NT = 256 * HW;
+  constexpr int DPT = 16 / (4 * HW);              // global->LDS load instructions per wavefront and block (1 KB each)
+  __shared__ __align__(16) unsigned char smem[NSTG * PSTAGE];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qg = wave & 3, hset = wave >> 2;      // the wavefront's 32 queries; its set of heads
   const int l31 = lane & 31, h = lane >> 5;
 
-  // workgroup -> (kv head, head sub-group, batch row, query tile); kv head fastest, long tiles first
-  const int nsub = a.group / NH;
+  // workgroup -> (kv head, head sub-group, batch row, query tile); kv head fastest. Long tiles go first; when the whole
+  // launch is resident at once (two workgroups per CU), the second workgroup of each CU is taken in the opposite
+  // order, so a CU that got a long tile gets a short one next to it.
+  const int nsub = a.group / (NH * HW);
   const int ntiles = (a.n_q + PBM - 1) / PBM;
   unsigned id = blockIdx.x;
   const int kvh = id % a.n_kv_heads;
   id /= a.n_kv_heads;
+  {
+    const unsigned per_round = 256 / (a.n_kv_heads < 256 ? a.n_kv_heads : 256);      // first workgroups of the CUs, per KV head
+    const unsigned n = gridDim.x / a.n_kv_heads;
+    if (HW == 1 && per_round > 0 && n <= 2 * per_round && id >= per_round) id = n + per_round - 1 - id;
+  }
   const int sub = id % nsub;
   id /= nsub;
   const int b = id % a.batch;
   id /= a.batch;
   const int tile = ntiles - 1 - static_cast<int>(id);
-  const int head0 = kvh * a.group + sub * NH;
+  const int head0 = kvh * a.group + (sub * HW + hset) * NH;
 
   const int start = a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
   const int q0 = tile * PBM;
-  const int qw0 = q0 + wave * 32;          // the wavefront's first query
+  const int qw0 = q0 + qg * 32;            // the wavefront's first query
   const int p0 = start + qw0;              // and its position
   const int q_end = q0 + PBM < a.n_q ? q0 + PBM : a.n_q;
   int kv_hi = start + q_end < a.n_kv_ctx ? start + q_end : a.n_kv_ctx;       // keys the tile's last query sees (exclusive)
@@ -89,59 +115,55 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
   const bf16* kp = a.k + b * a.kv_bs + kvh * 64;
   const bf16* vp = a.v + b * a.kv_bs + kvh * 64;
 
-  // ---- Q fragments (B operand: lane = query, 8 d per half-wavefront and k16 step)
-  bf16x8 qf[NH][4];
-  {
-    int qrow = qw0 + l31;
-    qrow = qrow < a.n_q ? qrow : a.n_q - 1;
-    const bf16* qp = a.q + b * a.q_bs + static_cast<int64_t>(qrow) * a.q_ts + head0 * 64 + h * 8;
+  // ---- K / V block movers: global_load_lds_dwordx4 (no staging registers, no LDS writes). One instruction fills
+  // 1 KB = 8 tile rows, the lanes' 16 bytes landing at M0 + 16 * lane; the swizzle is applied by choosing which chunk of
+  // the row a lane fetches. A stage is the K tile followed by the V tile, so a wavefront's DPT instructions all belong
+  // to one of the two.
+  const bool dma_v = wave * DPT >= 8;
+  const bf16* dma_src = dma_v ? vp : kp;
+  int dma_row[DPT], dma_col[DPT];
+  const bf16* dma_ptr[DPT];                       // the lane's chunk of its row of key block 0
 #pragma unroll
-    for (int hd = 0; hd < NH; ++hd)
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) qf[hd][kk] = *reinterpret_cast<const bf16x8*>(qp + hd * 64 + kk * 16);
+  for (int j = 0; j < DPT; ++j) {
+    const int row = ((wave * DPT + j) & 7) * 8 + (lane >> 3);
+    dma_row[j] = row;
+    dma_col[j] = ((lane & 7) ^ (dma_v ? v_swizzle(row) : ((row >> 1) & 7))) * 8;
+    dma_ptr[j] = dma_src + static_cast<int64_t>(row) * a.kv_ts + dma_col[j];
   }
+  const unsigned lds0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem)) + wave * DPT * 1024;
+  const int64_t blk_stride = static_cast<int64_t>(PBN) * a.kv_ts;
+  auto issue_block = [&](int blk, int stage) {
+    const bool whole = blk * PBN + PBN - 1 <= key_max;       // no row of the block lies beyond the last visible key
+#pragma unroll
+    for (int j = 0; j < DPT; ++j) {
+      const bf16* g;
+      if (whole) {
+        g = dma_ptr[j] + blk * blk_stride;
+      } else {
+        int key = blk * PBN + dma_row[j];
+        key = key < key_max ? key : key_max;
+        g = dma_src + static_cast<int64_t>(key) * a.kv_ts + dma_col[j];
+      }
+      const unsigned m0v = lds0 + stage * PSTAGE + j * 1024;
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
+    }
+  };
+  // wait until all but the `behind` youngest blocks' loads of this wavefront have landed, then meet the others
+  auto wait_and_meet = [&](int behind) {
+    if (behind >= 2)
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * DPT) : "memory");
+    else if (behind == 1)
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(DPT) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  };
 
-  // ---- K / V block movers. K: thread -> two 16-byte chunks. V: thread -> 8 d of two keys that are neighbours in the
-  // permuted key order (keys 2p, 2p + 1), written as eight 32-bit (key pair) words into V^T.
-  bf16x8 kr[2], vr[2];
-  auto load_block = [&](int blk) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int ci = tid + 256 * j;
-      int key = blk * PBN + (ci >> 3);
-      key = key < key_max ? key : key_max;
-      kr[j] = *reinterpret_cast<const bf16x8*>(kp + static_cast<int64_t>(key) * a.kv_ts + (ci & 7) * 8);
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      int key = blk * PBN + 2 * (tid >> 3) + j;
-      key = key < key_max ? key : key_max;
-      vr[j] = *reinterpret_cast<const bf16x8*>(vp + static_cast<int64_t>(key) * a.kv_ts + (tid & 7) * 8);
-    }
-  };
-  auto store_block = [&](int stage) {
-    unsigned char* ks = smem + stage * PSTAGE;
-    unsigned char* vs = ks + KT_BYTES;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int ci = tid + 256 * j;
-      const int key = ci >> 3, ch = ci & 7;
-      *reinterpret_cast<bf16x8*>(ks + key * 128 + ((ch ^ ((key >> 1) & 7)) << 4)) = kr[j];
-    }
-    // key r of the block = kb*32 + c*16 + u*8 + hh*4 + i sits at column kb*32 + c*16 + hh*8 + u*4 + i of V^T
-    const int r0 = 2 * (tid >> 3);
-    const int chunk = (r0 >> 5) * 4 + ((r0 >> 4) & 1) * 2 + ((r0 >> 2) & 1);
-    const int within = ((r0 >> 3) & 1) * 4 + (r0 & 3);
-    const int dc = tid & 7;
-    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
-    const u32x4 w0 = __builtin_bit_cast(u32x4, vr[0]), w1 = __builtin_bit_cast(u32x4, vr[1]);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int d = dc * 8 + e;
-      const unsigned word = (e & 1) ? ((w0[e >> 1] >> 16) | (w1[e >> 1] & 0xffff0000u)) : ((w0[e >> 1] & 0xffffu) | (w1[e >> 1] << 16));
-      *reinterpret_cast<unsigned*>(vs + d * 128 + ((chunk ^ vt_swizzle(d)) << 4) + within * 2) = word;
-    }
-  };
+  // K fragment (A operand of S^T): lane = key l31 of a 32-key half, 16 bytes at d = kk*16 + h*8
+  const int k_row = l31 * 128, k_sw = (l31 >> 1) & 7;
+  // V^T fragment (A operand of O^T): lane = d; the transposing read wants from lane j of each 16 the address of
+  // four d (quad j % 4 of the lane group's 16) of key j / 4 of the four keys this half-wavefront takes
+  const int v_key = 4 * h + ((lane & 15) >> 2);                       // + 16*cc + 8*u + 32*kb
+  const int v_d = (l31 & 16) + 4 * (lane & 3);                        // + 32*db
 
   // ---- running state: lane = query; m in log2 units of the scaled logits
   const float c = a.sm_scale * kLog2e;
@@ -157,16 +179,37 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
       for (int r = 0; r < 16; ++r) o[hd][db][r] = 0.f;
   }
 
-  if (blk_lo < blk_hi) {
-    load_block(blk_lo);
-    store_block(0);
-  }
-  __syncthreads();
+  const int nblk = blk_hi - blk_lo;
+#pragma unroll
+  for (int i = 0; i < NSTG - 1; ++i)
+    if (i < nblk) issue_block(blk_lo + i, i);
 
-  for (int blk = blk_lo; blk < blk_hi; ++blk) {
-    const int stage = (blk - blk_lo) & 1;
-    const bool more = blk + 1 < blk_hi;
-    if (more) load_block(blk + 1);
+  // ---- Q fragments (B operand: lane = query, 8 d per half-wavefront and k16 step)
+  bf16x8 qf[NH][4];
+  {
+    int qrow = qw0 + l31;
+    qrow = qrow < a.n_q ? qrow : a.n_q - 1;
+    const bf16* qp = a.q + b * a.q_bs + static_cast<int64_t>(qrow) * a.q_ts + head0 * 64 + h * 8;
+#pragma unroll
+    for (int hd = 0; hd < NH; ++hd)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) qf[hd][kk] = *reinterpret_cast<const bf16x8*>(qp + hd * 64 + kk * 16);
+    // The compiler does not see the direct-to-LDS loads in its count of outstanding loads; were the fragments first
+    // used inside the loop, its wait for them there would be "nothing outstanding" and drain the blocks in flight on
+    // every step. Pin the wait here, where the first blocks have to land anyway.
+#pragma unroll
+    for (int hd = 0; hd < NH; ++hd)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) asm volatile("" : "+v"(qf[hd][kk]));
+  }
+
+  wait_and_meet(nblk - 1);                       // block 0 has landed (those behind it may still be in flight)
+
+  for (int i = 0; i < nblk; ++i) {
+    const int blk = blk_lo + i;
+    const int stage = i & (NSTG - 1);
+    // the stage this refills was read in the previous step, which every wavefront has left
+    if (i + NSTG - 1 < nblk) issue_block(blk + NSTG - 1, (i + NSTG - 1) & (NSTG - 1));
 
     const int key0 = blk * PBN;
     // does any of the wavefront's 32 queries see a key of this block?
@@ -177,18 +220,19 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
       // S^T[key, query]
       f32x16 s[NH][2];
 #pragma unroll
-      for (int hd = 0; hd < NH; ++hd)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[hd][kb][r] = 0.f;
-#pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + (kb * 32 + l31) * 128 + (((kk * 2 + h) ^ ((l31 >> 1) & 7)) << 4));
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + kb * 32 * 128 + k_row + (((kk * 2 + h) ^ k_sw) << 4));
 #pragma unroll
-          for (int hd = 0; hd < NH; ++hd) s[hd][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[hd][kk], s[hd][kb], 0, 0, 0);
+          for (int hd = 0; hd < NH; ++hd) {
+            if (kk == 0) {
+              const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              s[hd][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[hd][kk], zero, 0, 0, 0);
+            } else {
+              s[hd][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[hd][kk], s[hd][kb], 0, 0, 0);
+            }
+          }
         }
       // mask where the block crosses the causal diagonal, the window's trailing edge or the end of the keys
       const bool full = key0 + PBN - 1 <= p0 && key0 + PBN - 1 < a.n_kv_ctx && (a.window <= 0 || key0 >= p0 + 31 - a.window + 1);
@@ -206,57 +250,85 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
             for (int hd = 0; hd < NH; ++hd) s[hd][kb][r] = vis ? s[hd][kb][r] : -INFINITY;
           }
       }
-      // online softmax, P^T in bf16 straight into operand registers
-      bf16x8 pf[NH][2][2];
+      // online softmax. First the block maxima of all heads and ONE (rare) branch that raises running maxima; what
+      // follows is then a single straight-line region in which the exponentials of one (head, 32-key half) and the
+      // P.V MFMAs of the one before it can be issued in turn.
+      bool raise[NH];
+      float mx[NH];
+      bool any = false;
 #pragma unroll
       for (int hd = 0; hd < NH; ++hd) {
-        float mx = -INFINITY;
+        float t = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[hd][kb][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[hd], mx * c);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run[hd] - m_use);
-        m_run[hd] = m_new;
-        float lsum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[hd][kb][r], c, -m_use));
-            lsum += p;
-            pf[hd][kb][r >> 3][r & 7] = static_cast<bf16>(p);
-          }
-        l_run[hd] = fmaf(l_run[hd], alpha, lsum);
-#pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[hd][db][r] *= alpha;
+          for (int r = 0; r < 16; ++r) t = fmaxf(t, s[hd][kb][r]);
+        mx[hd] = fmaxf(t, other_half(t, h)) * c;
+        // the maximum moves only when this block tops it by more than kRaise: p stays below 2^kRaise otherwise
+        raise[hd] = mx[hd] > m_run[hd] + kRaise;                  // false while mx is -inf (nothing visible yet)
+        any = any || raise[hd];
       }
-      // O^T[d, query] += V^T[d, keys] . P^T[keys, query]
+      if (__builtin_amdgcn_ballot_w64(any) != 0) {
 #pragma unroll
-      for (int db = 0; db < 2; ++db)
+        for (int hd = 0; hd < NH; ++hd) {
+          const float m_new = raise[hd] ? mx[hd] : m_run[hd];
+          const float alpha = raise[hd] ? __builtin_amdgcn_exp2f(m_run[hd] - m_new) : 1.f;     // -inf - finite: 0
+          m_run[hd] = m_new;
+          l_run[hd] *= alpha;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+          for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[hd][db][r] *= alpha;
+        }
+      }
+      const bf16x2 one2 = {static_cast<bf16>(1.0f), static_cast<bf16>(1.0f)};
+#pragma unroll
+      for (int hd = 0; hd < NH; ++hd) {
+        const float m_use = m_run[hd] == -INFINITY ? 0.f : m_run[hd];
+        float lsum = l_run[hd];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          // P^T in bf16 straight into operand registers
+          bf16x8 pf[2];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) pf[r >> 3][r & 7] = static_cast<bf16>(__builtin_amdgcn_exp2f(fmaf(s[hd][kb][r], c, -m_use)));
+          // the denominator sums the rounded weights the numerator's MFMA multiplies with, two per instruction
 #pragma unroll
           for (int cc = 0; cc < 2; ++cc) {
-            const int d = db * 32 + l31;
-            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs + d * 128 + (((kb * 4 + cc * 2 + h) ^ vt_swizzle(d)) << 4));
-#pragma unroll
-            for (int hd = 0; hd < NH; ++hd) o[hd][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[hd][kb][cc], o[hd][db], 0, 0, 0);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[cc], pf[cc], 0, 1), one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[cc], pf[cc], 2, 3), one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[cc], pf[cc], 4, 5), one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[cc], pf[cc], 6, 7), one2, lsum, false);
           }
+          // O^T[d, query] += V^T[d, keys] . P^T[keys, query]
+#pragma unroll
+          for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int db = 0; db < 2; ++db) {
+              i16x4 part[2];
+#pragma unroll
+              for (int u = 0; u < 2; ++u) {
+                const int key = kb * 32 + cc * 16 + u * 8 + v_key;
+                const int d = db * 32 + v_d;
+                part[u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) i16x4*)(vs + key * 128 + (((d >> 3) ^ v_swizzle(key)) << 4) + (d & 7) * 2));
+              }
+              typedef __attribute__((__vector_size__(8 * sizeof(short)))) short i16x8;
+              const i16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
+              o[hd][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[cc], o[hd][db], 0, 0, 0);
+            }
+        }
+        l_run[hd] = lsum;
+      }
     }
-    if (more) store_block(stage ^ 1);
-    __syncthreads();
+    wait_and_meet(nblk - 2 - i);                 // block i + 1 has landed
   }
 
   // ---- the sink joins the denominator; normalise; store (lane = query: 8-byte runs of four d)
   const int qrow = qw0 + l31;
 #pragma unroll
   for (int hd = 0; hd < NH; ++hd) {
-    const float l_tot = l_run[hd] + __shfl_xor(l_run[hd], 32, 64);
+    const float l_tot = l_run[hd] + other_half(l_run[hd], h);
     const float sk = a.sinks ? static_cast<float>(a.sinks[head0 + hd]) * kLog2e : 0.f;
     const float m_f = fmaxf(m_run[hd], sk);
     const float so = __builtin_amdgcn_exp2f(m_run[hd] - m_f);
@@ -324,14 +396,14 @@ extern "C" int tllm_attention_prefill_bf16(const void* q, const void* k, const v
   a.group = group;
   a.window = window;
   a.sm_scale = sm_scale;
-  const int nh = group % 2 == 0 ? 2 : 1;
+  const int nh = group % 2 == 0 ? 2 : 1, hw = 1;
   const int64_t ntiles = (n_q + PBM - 1) / PBM;
-  const int64_t wgs = ntiles * batch * n_kv_heads * (group / nh);
+  const int64_t wgs = ntiles * batch * n_kv_heads * (group / (nh * hw));
   TLLM_REQUIRE(batch < (1ll << 24) && wgs < (1ll << 31), TLLM_E_SHAPE, "attention_prefill: %lld workgroups are too many for one launch", (long long)wgs);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (nh == 2)
-    hipLaunchKernelGGL(attn_prefill_kernel<2>, dim3((unsigned)wgs), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((attn_prefill_kernel<2, 1>), dim3((unsigned)wgs), dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((unsigned)wgs), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((attn_prefill_kernel<1, 1>), dim3((unsigned)wgs), dim3(256), 0, st, a);
   return check_launch("attention_prefill");
 }
