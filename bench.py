@@ -445,6 +445,18 @@ def main() -> int:
             bench_kernel(f"rmsnorm_T{tt}", lambda i, xp=xp, to=to: T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=to),
                          bytes_of["rmsnorm"](tt), n=96)
             del xp, qo, to
+            # prefill attention over the projection's output, q / k / v read in place as column ranges of [1, T, 5120]
+            pq = [torch.empty(1, tt, QKV_DIM, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(2)]
+            pv = [(t[:, :, :NQ * HD].view(1, tt, NKV, NQ // NKV, HD), t[:, :, NQ * HD:(NQ + NKV) * HD].view(1, tt, NKV, HD),
+                   t[:, :, (NQ + NKV) * HD:].view(1, tt, NKV, HD)) for t in pq]
+            psink = torch.empty(NQ, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            pstart = torch.zeros(1, dtype=torch.int64, device=dev)
+            for win in (None, 128):
+                pairs = sum(min(i + 1, win) if win else i + 1 for i in range(tt))
+                bench_kernel(f"attention_prefill_{'win' if win else 'ctx'}{tt}_B1",
+                             lambda i, pv=pv, win=win: T.attention(*pv[i % 2], psink, 0.125, win, pstart),
+                             flops=4.0 * NQ * HD * pairs, n=24)
+            del pq, pv
         idp = torch.randint(0, VOCAB_BENCH, (2048,), generator=g, dtype=torch.int32).to(dev)
         hp = torch.empty(2048, HIDDEN, dtype=torch.bfloat16, device=dev)
         bench_kernel("embedding_T2048", lambda i: T.embedding_forward(idp, table, out=hp), bytes_of["embedding"](2048), n=96)

@@ -11,8 +11,9 @@
 // the cache layout ([token, kv head, 64]), and writes [token, head * 64]: no copies on either side.
 //
 //   * a workgroup takes 128 consecutive queries of NH query heads that share a KV head, four wavefronts of 32 queries;
-//     K / V blocks of 64 keys pass through two LDS stages (registers -> LDS while the previous block is computed,
-//     one barrier per block) and serve all NH heads;
+//     K / V blocks of 64 keys pass through four LDS stages filled by global_load_lds_dwordx4 (no staging registers, no
+//     LDS writes; three blocks in flight behind the one being computed, one hand-spelled wait + barrier per block)
+//     and serve all NH heads;
 //   * S^T = K . Q^T on v_mfma_f32_32x32x16_bf16 with the keys on M: a lane then owns ONE query (column) and 16 keys
 //     per 32-key block, so the running maximum, the running sum and the rescale factor of the online softmax are
 //     lane-local apart from one exchange between the two half-wavefronts;
@@ -21,7 +22,8 @@
 //     (V^T: lane = d, 8 keys) comes out of two transposing reads (ds_read_b64_tr_b16: within 16 lanes, lane i receives
 //     element i % 4 of the 8 bytes addressed by lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4);
 //   * the running maximum is only raised when a block exceeds it by more than 2^8 (exponents stay far from overflow, the
-//     result is the same quotient), so the accumulator is almost never rescaled;
+//     result is the same quotient), so the accumulator is almost never rescaled; the weights are summed, as the bf16
+//     values the MFMA multiplies with, two per v_dot2c_f32_bf16;
 //   * both tiles are XOR-swizzled in 16-byte chunks: fragment reads are conflict-free (K) or at the two-pass minimum (V);
 //   * the KV head is the fastest-varying part of the workgroup index, so with eight KV heads each XCD's L2 holds the
 //     K and V of one head; the query tiles with the most keys to visit are launched first.
@@ -68,21 +70,19 @@ __device__ __forceinline__ float other_half(float x, int high) {
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4;
 
-// NH: query heads per wavefront; HW: sets of four wavefronts, each set with its own NH heads of the same queries
-template <int NH, int HW>
-__global__ __launch_bounds__(256 * HW, HW == 1 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
-  constexpr int NT = 256 * HW;
-  constexpr int DPT = 16 / (4 * HW);              // global->LDS load instructions per wavefront and block (1 KB each)
+// NH: query heads (of one KV head) per wavefront
+template <int NH>
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a) {
+  constexpr int DPT = 4;                          // global->LDS load instructions per wavefront and block (1 KB each)
   __shared__ __align__(16) unsigned char smem[NSTG * PSTAGE];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int qg = wave & 3, hset = wave >> 2;      // the wavefront's 32 queries; its set of heads
   const int l31 = lane & 31, h = lane >> 5;
 
   // workgroup -> (kv head, head sub-group, batch row, query tile); kv head fastest. Long tiles go first; when the whole
   // launch is resident at once (two workgroups per CU), the second workgroup of each CU is taken in the opposite
   // order, so a CU that got a long tile gets a short one next to it.
-  const int nsub = a.group / (NH * HW);
+  const int nsub = a.group / NH;
   const int ntiles = (a.n_q + PBM - 1) / PBM;
   unsigned id = blockIdx.x;
   const int kvh = id % a.n_kv_heads;
@@ -90,18 +90,18 @@ __global__ __launch_bounds__(256 * HW, HW == 1 ? 2 : 1) void attn_prefill_kernel
   {
     const unsigned per_round = 256 / (a.n_kv_heads < 256 ? a.n_kv_heads : 256);      // first workgroups of the CUs, per KV head
     const unsigned n = gridDim.x / a.n_kv_heads;
-    if (HW == 1 && per_round > 0 && n <= 2 * per_round && id >= per_round) id = n + per_round - 1 - id;
+    if (per_round > 0 && n <= 2 * per_round && id >= per_round) id = n + per_round - 1 - id;
   }
   const int sub = id % nsub;
   id /= nsub;
   const int b = id % a.batch;
   id /= a.batch;
   const int tile = ntiles - 1 - static_cast<int>(id);
-  const int head0 = kvh * a.group + (sub * HW + hset) * NH;
+  const int head0 = kvh * a.group + sub * NH;
 
   const int start = a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
   const int q0 = tile * PBM;
-  const int qw0 = q0 + qg * 32;            // the wavefront's first query
+  const int qw0 = q0 + wave * 32;          // the wavefront's first query
   const int p0 = start + qw0;              // and its position
   const int q_end = q0 + PBM < a.n_q ? q0 + PBM : a.n_q;
   int kv_hi = start + q_end < a.n_kv_ctx ? start + q_end : a.n_kv_ctx;       // keys the tile's last query sees (exclusive)
@@ -396,14 +396,14 @@ extern "C" int tllm_attention_prefill_bf16(const void* q, const void* k, const v
   a.group = group;
   a.window = window;
   a.sm_scale = sm_scale;
-  const int nh = group % 2 == 0 ? 2 : 1, hw = 1;
+  const int nh = group % 2 == 0 ? 2 : 1;
   const int64_t ntiles = (n_q + PBM - 1) / PBM;
-  const int64_t wgs = ntiles * batch * n_kv_heads * (group / (nh * hw));
+  const int64_t wgs = ntiles * batch * n_kv_heads * (group / nh);
   TLLM_REQUIRE(batch < (1ll << 24) && wgs < (1ll << 31), TLLM_E_SHAPE, "attention_prefill: %lld workgroups are too many for one launch", (long long)wgs);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (nh == 2)
-    hipLaunchKernelGGL((attn_prefill_kernel<2, 1>), dim3((unsigned)wgs), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_prefill_kernel<2>, dim3((unsigned)wgs), dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL((attn_prefill_kernel<1, 1>), dim3((unsigned)wgs), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((unsigned)wgs), dim3(256), 0, st, a);
   return check_launch("attention_prefill");
 }
