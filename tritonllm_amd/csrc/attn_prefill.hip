@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
 
   const int nblk = blk_hi - blk_lo;
 #pragma unroll
-  for (int i = 0; i < NSTG - 1; ++i)
+  for (int i = 0; i < 2; ++i)
     if (i < nblk) issue_block(blk_lo + i, i);
 
   // ---- Q fragments (B operand: lane = query, 8 d per half-wavefront and k16 step)
@@ -203,14 +203,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
       for (int kk = 0; kk < 4; ++kk) asm volatile("" : "+v"(qf[hd][kk]));
   }
 
-  wait_and_meet(nblk - 1);                       // block 0 has landed (those behind it may still be in flight)
+  wait_and_meet(0);                              // blocks 0 and 1 have landed
 
-  for (int i = 0; i < nblk; ++i) {
-    const int blk = blk_lo + i;
-    const int stage = i & (NSTG - 1);
-    // the stage this refills was read in the previous step, which every wavefront has left
-    if (i + NSTG - 1 < nblk) issue_block(blk + NSTG - 1, (i + NSTG - 1) & (NSTG - 1));
-
+  auto process = [&](int blk, int stage) __attribute__((always_inline)) {
     const int key0 = blk * PBN;
     // does any of the wavefront's 32 queries see a key of this block?
     const bool active = key0 <= p0 + 31 && (a.window <= 0 || key0 + PBN - 1 >= p0 - a.window + 1);
@@ -321,7 +316,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
         l_run[hd] = lsum;
       }
     }
-    wait_and_meet(nblk - 2 - i);                 // block i + 1 has landed
+  };
+
+  // Two blocks per step: the step's loads refill the two stages the previous step read (every wavefront has left it),
+  // have two blocks of arithmetic to land behind, and are met with one wait + barrier.
+  for (int i = 0; i < nblk; i += 2) {
+#pragma unroll
+    for (int j = 2; j < 4; ++j)
+      if (i + j < nblk) issue_block(blk_lo + i + j, (i + j) & (NSTG - 1));
+    process(blk_lo + i, i & (NSTG - 1));
+    if (i + 1 < nblk) process(blk_lo + i + 1, (i + 1) & (NSTG - 1));
+    wait_and_meet(0);
   }
 
   // ---- the sink joins the denominator; normalise; store (lane = query: 8-byte runs of four d)
