@@ -939,6 +939,38 @@ def test_attention_block_decode_chain(gpu):
         close(y.view(bs, 2880), yr)
 
 
+def test_attention_block_prefill_chain(gpu):
+    """The attention block of a prompt, in two chunks, as model.py:471-573 strings it together: RMSNorm, QKV + bias +
+    RoPE with k / v written straight into the cache rows of the chunk, attention of the chunk's queries (read in place
+    from the projection's output) over the cache so far, with sinks, full and windowed -- against the oracle chain."""
+    n_ctx, chunk = 512, 200
+    g = torch.Generator().manual_seed(91)
+    sinks = torch.randn(64, generator=g).bfloat16()
+    yarn = T.gpt_oss_yarn()
+    for window in (None, 128):
+        ck = torch.full((1, n_ctx, 8, 64), float("nan"), dtype=torch.bfloat16, device=gpu)     # slots never written stay NaN
+        cv = torch.full((1, n_ctx, 8, 64), float("nan"), dtype=torch.bfloat16, device=gpu)
+        rk = torch.zeros(1, 2 * chunk, 8, 64, dtype=torch.bfloat16)
+        rv = torch.zeros(1, 2 * chunk, 8, 64, dtype=torch.bfloat16)
+        for part in range(2):
+            start = part * chunk
+            d = O.make_inputs(chunk, seed=92 + part)
+            pos = torch.arange(start, start + chunk, dtype=torch.int64)
+            tn = T.rmsnorm_forward(d["x"].to(gpu), d["norm_scale"].to(gpu), 1e-5)
+            q = torch.empty(chunk, 4096, dtype=torch.bfloat16, device=gpu)
+            T.qkv_rope_forward(tn, d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=pos.to(gpu), mode="prefill",
+                               out=(q, ck[0, start:start + chunk].view(chunk, 512), cv[0, start:start + chunk].view(chunk, 512)))
+            t = T.attention(q.view(1, chunk, 8, 8, 64), ck, cv, sinks.to(gpu), 0.125, window, torch.tensor([start], dtype=torch.int64, device=gpu))
+            # oracle chain, rounding to bf16 wherever a tensor crosses from one reference kernel to the next
+            tr = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16()
+            qr, kr, vr = O.qkv_rope_ref(tr, d["w"], d["b"], pos)
+            rk[0, start:start + chunk] = kr.bfloat16().view(chunk, 8, 64)
+            rv[0, start:start + chunk] = vr.bfloat16().view(chunk, 8, 64)
+            want = O.attention_ref(qr.bfloat16().view(1, chunk, 8, 8, 64), rk[:, :start + chunk], rv[:, :start + chunk], sinks, 0.125, window, start)
+            close(ck[0, start:start + chunk].view(chunk, 512), kr)
+            close(t, want)
+
+
 # ----------------------------------------------------------------------------------- MXFP4 checkpoint expansion
 def _bits_equal_nan_aware(out, ref):
     out = out.cpu()
