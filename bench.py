@@ -534,6 +534,35 @@ def main() -> int:
                                             "tokens/s": round(r / sec, 1)}
             del ck, cv
 
+    # ---------------------------------------------------------------- the same half of the layers for a prompt
+    # per layer: RMSNorm, QKV + bias + RoPE with k / v written into the cache rows of the prompt, prefill attention
+    # reading q in place from the projection's output (window 128 on even layers). The out-projection of a prompt is a
+    # library GEMM in the reference and here (model.py:571-572) and is left out.
+    if not args.no_kernel_table:
+        for tt in (2048, 8192):
+            xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            tn = torch.empty_like(xp)
+            pp = torch.arange(tt, dtype=torch.int64, device=dev)
+            qb = torch.empty(tt, NQ * HD, dtype=torch.bfloat16, device=dev)
+            ck = [torch.empty(1, tt, NKV, HD, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+            cv = [torch.empty(1, tt, NKV, HD, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+            pstart = torch.zeros(1, dtype=torch.int64, device=dev)
+
+            def prompt_step(_i, tt=tt, xp=xp, tn=tn, pp=pp, qb=qb, ck=ck, cv=cv):
+                for l in range(N_LAYERS):
+                    T.rmsnorm_forward(xp, scales[l], 1e-5, out=tn)
+                    T.qkv_rope_forward(tn, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=pp, mode="prefill",
+                                       out=(qb, ck[l % 2][0].view(tt, NKV * HD), cv[l % 2][0].view(tt, NKV * HD)))
+                    T.attention(qb.view(1, tt, NKV, NQ // NKV, HD), ck[l % 2], cv[l % 2], asink, 0.125, 128 if l % 2 == 0 else None, pstart)
+
+            prompt_step(0)
+            gr = graph_of(prompt_step, 1)
+            gr.replay()
+            sec = min(time_graph(gr) for _ in range(3))
+            attn_stack[f"prompt_T{tt}"] = {"us_per_prompt": round(sec * 1e6, 1), "us_per_layer": round(sec * 1e6 / N_LAYERS, 2),
+                                           "tokens/s": round(tt / sec, 1)}
+            del xp, tn, qb, ck, cv
+
     # ---------------------------------------------------------------- CPU baseline (reported only)
     cpu_baseline = None
     if not args.no_cpu_baseline:
