@@ -46,7 +46,6 @@ struct AttnPrefillArgs {
 };
 
 namespace {
-constexpr int PBM = 128;              // queries per workgroup
 constexpr int PBN = 64;               // keys per block
 constexpr int KT_BYTES = PBN * 128;   // K tile [key][64 d]
 constexpr int VT_BYTES = PBN * 128;   // V tile [key][64 d]
@@ -70,9 +69,12 @@ __device__ __forceinline__ float other_half(float x, int high) {
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4;
 
-// NH: query heads (of one KV head) per wavefront
-template <int NH>
+// NH: query heads (of one KV head) per wavefront. QG: groups of 32 queries per workgroup; the four wavefronts are QG
+// query groups x 4 / QG head sets, so a workgroup covers 32 * QG queries of NH * 4 / QG heads.
+template <int NH, int QG>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a) {
+  constexpr int PBM = 32 * QG;                    // queries per workgroup
+  constexpr int HS = 4 / QG;                      // head sets
   constexpr int DPT = 4;                          // global->LDS load instructions per wavefront and block (1 KB each)
   __shared__ __align__(16) unsigned char smem[NSTG * PSTAGE];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
   // workgroup -> (kv head, head sub-group, batch row, query tile); kv head fastest. Long tiles go first; when the whole
   // launch is resident at once (two workgroups per CU), the second workgroup of each CU is taken in the opposite
   // order, so a CU that got a long tile gets a short one next to it.
-  const int nsub = a.group / NH;
+  const int nsub = a.group / (NH * HS);
   const int ntiles = (a.n_q + PBM - 1) / PBM;
   unsigned id = blockIdx.x;
   const int kvh = id % a.n_kv_heads;
@@ -97,11 +99,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
   const int b = id % a.batch;
   id /= a.batch;
   const int tile = ntiles - 1 - static_cast<int>(id);
-  const int head0 = kvh * a.group + sub * NH;
+  const int head0 = kvh * a.group + (sub * HS + wave / QG) * NH;
 
   const int start = a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
   const int q0 = tile * PBM;
-  const int qw0 = q0 + wave * 32;          // the wavefront's first query
+  const int qw0 = q0 + (wave % QG) * 32;   // the wavefront's first query
   const int p0 = start + qw0;              // and its position
   const int q_end = q0 + PBM < a.n_q ? q0 + PBM : a.n_q;
   int kv_hi = start + q_end < a.n_kv_ctx ? start + q_end : a.n_kv_ctx;       // keys the tile's last query sees (exclusive)
@@ -401,14 +403,21 @@ extern "C" int tllm_attention_prefill_bf16(const void* q, const void* k, const v
   a.group = group;
   a.window = window;
   a.sm_scale = sm_scale;
+  // Workgroup shape: 128 queries x 2 heads (two heads per wavefront) as soon as that gives every CU two workgroups;
+  // below that 64 queries x 2 heads with one head per wavefront: twice the workgroups, and the longest of them -- it
+  // sets the time of so small a launch -- takes about half as long per key block (one prompt of 1024 tokens: 28.8 ->
+  // 21.4 us; at 2048 tokens, 512 workgroups of the large shape, the two are level). Odd group sizes: 128 x 1.
   const int nh = group % 2 == 0 ? 2 : 1;
-  const int64_t ntiles = (n_q + PBM - 1) / PBM;
-  const int64_t wgs = ntiles * batch * n_kv_heads * (group / nh);
+  const int64_t wgs128 = (n_q + 127) / 128 * batch * n_kv_heads * (group / nh);
+  const bool small = nh == 2 && wgs128 < 512;
+  const int64_t wgs = small ? (n_q + 63) / 64 * batch * n_kv_heads * (group / 2) : wgs128;
   TLLM_REQUIRE(batch < (1ll << 24) && wgs < (1ll << 31), TLLM_E_SHAPE, "attention_prefill: %lld workgroups are too many for one launch", (long long)wgs);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (nh == 2)
-    hipLaunchKernelGGL(attn_prefill_kernel<2>, dim3((unsigned)wgs), dim3(256), 0, st, a);
+  if (small)
+    hipLaunchKernelGGL((attn_prefill_kernel<1, 2>), dim3((unsigned)wgs), dim3(256), 0, st, a);
+  else if (nh == 2)
+    hipLaunchKernelGGL((attn_prefill_kernel<2, 4>), dim3((unsigned)wgs), dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((unsigned)wgs), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((attn_prefill_kernel<1, 4>), dim3((unsigned)wgs), dim3(256), 0, st, a);
   return check_launch("attention_prefill");
 }
