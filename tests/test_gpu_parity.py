@@ -892,6 +892,13 @@ def test_attention_prefill_full_prompt(gpu):
     _attn_prefill_case(gpu, 1, 2048, 2048, 128, 0, seed=32)
 
 
+@pytest.mark.parametrize("sliding_window", [None, 128])
+def test_attention_prefill_large_launch_ragged(gpu, sliding_window):
+    """Enough workgroups for the 128-query x two-heads-per-wavefront shape (the library picks the workgroup shape from
+    the size of the launch), with a ragged last tile, a later chunk of the prompt and keys beyond the last query."""
+    _attn_prefill_case(gpu, 4, 600, 700, sliding_window, 77, start_dtype=torch.int64, seed=41)
+
+
 def test_attention_prefill_argument_errors(gpu):
     q = torch.zeros(1, 16, 8, 8, 64, dtype=torch.bfloat16, device=gpu)
     k = torch.zeros(1, 16, 8, 64, dtype=torch.bfloat16, device=gpu)
