@@ -158,6 +158,27 @@ def test_mxfp4_argument_errors():
     assert "aligned" in _err()
 
 
+def test_attention_prefill_argument_errors():
+    """Argument checks of the prefill attention entry point happen before anything touches the GPU."""
+    f = _lib.lib().tllm_attention_prefill_bf16
+    p = C.c_void_p(4096)
+
+    def call(q=p, k=p, v=p, out=p, q_ts=4096, kv_ts=512, batch=1, n_q=16, n_kv=16, kvh=8, group=8, hd=64, scale=0.125, window=0, start=p):
+        return f(q, k, v, None, out, n_q * q_ts, q_ts, n_q * 4096, 4096, n_kv * kv_ts, kv_ts, batch, n_q, n_kv, kvh, group, hd, scale, window,
+                 start, 0, None)
+
+    assert call(batch=0) == 0 and call(n_q=0) == 0                      # nothing to do
+    assert call(hd=128) != 0 and "head_dim" in _err()
+    assert call(scale=0.0) != 0 and "sm_scale" in _err()
+    assert call(window=-1) != 0
+    assert call(n_kv=0) != 0
+    assert call(q=None) != 0 and "NULL" in _err()
+    assert call(start=None) != 0
+    assert call(k=C.c_void_p(4104)) != 0 and "aligned" in _err()
+    assert call(q_ts=4000) != 0                                         # heads do not fit into a token's stride
+    assert call(kv_ts=256) != 0
+
+
 def test_attention_decode_shape_planning():
     """The host-side choice of workgroup shape and splits (no launch): small batches keep one KV head per workgroup."""
     hpw = _lib.lib().tllm_attention_decode_heads_per_workgroup
