@@ -534,6 +534,37 @@ def main() -> int:
                                             "tokens/s": round(r / sec, 1)}
             del ck, cv
 
+    # ---------------------------------------------------------------- the two prefill configurations as chains
+    # configs[2]: gather [2048] -> RMSNorm -> QKV + bias + RoPE;  configs[3]: RMSNorm -> QKV + bias + RoPE at T = 8192 and
+    # SwiGLU [32768, 5760]. One graph replay = the chain once, weights rotating over the 24 sets.
+    prefill_chains = {}
+    if not args.no_kernel_table:
+        for tt, with_gather, swiglu_rows in ((2048, True, 0), (8192, False, 32768)):
+            idp = torch.randint(0, VOCAB_BENCH, (tt,), generator=g, dtype=torch.int32).to(dev)
+            xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+            tn = torch.empty_like(xp)
+            pp = torch.arange(tt, dtype=torch.int64, device=dev)
+            qo = (torch.empty(tt, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(tt, NKV * HD, dtype=torch.bfloat16, device=dev),
+                  torch.empty(tt, NKV * HD, dtype=torch.bfloat16, device=dev))
+            sx = torch.empty(swiglu_rows, 2 * HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 2, generator=gg) if swiglu_rows else None
+            so = torch.empty(swiglu_rows, HIDDEN, dtype=torch.bfloat16, device=dev) if swiglu_rows else None
+
+            def chain(i, idp=idp, xp=xp, tn=tn, pp=pp, qo=qo, sx=sx, so=so, with_gather=with_gather):
+                if with_gather:
+                    T.embedding_forward(idp, table, out=xp)
+                T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=tn)
+                T.qkv_rope_forward(tn, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn, positions=pp, mode="prefill", out=qo)
+                if sx is not None:
+                    T.swiglu(sx, out=so)
+
+            chain(0)
+            gr = graph_of(chain, 24)
+            gr.replay()
+            sec = min(time_graph(gr) for _ in range(5)) / 24
+            prefill_chains[f"T{tt}"] = {"chain": ("gather + " if with_gather else "") + "RMSNorm + QKV/bias/RoPE" + (" + SwiGLU[32768,5760]" if swiglu_rows else ""),
+                                        "us": round(sec * 1e6, 2), "tokens/s": round(tt / sec, 1)}
+            del xp, tn, qo, sx, so
+
     # ---------------------------------------------------------------- the same half of the layers for a prompt
     # per layer: RMSNorm, QKV + bias + RoPE with k / v written into the cache rows of the prompt, prefill attention
     # reading q in place from the projection's output (window 128 on even layers). The out-projection of a prompt is a
@@ -606,7 +637,7 @@ def main() -> int:
                    "batch": B, "layers_rotated": N_LAYERS,
                    "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel",
                    "gather": "inside the QKV decode kernel (x = table rows)" if args.fuse_gather else "own launch (x ~ N(0,1) as the configuration states)"},
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "attention_blocks24": attn_stack,
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "prefill_chains": prefill_chains, "attention_blocks24": attn_stack,
         "wall_s_timed_region": round(wall, 4),
     }
     print(json.dumps(out))
