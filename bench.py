@@ -460,6 +460,9 @@ def main() -> int:
         idp = torch.randint(0, VOCAB_BENCH, (2048,), generator=g, dtype=torch.int32).to(dev)
         hp = torch.empty(2048, HIDDEN, dtype=torch.bfloat16, device=dev)
         bench_kernel("embedding_T2048", lambda i: T.embedding_forward(idp, table, out=hp), bytes_of["embedding"](2048), n=96)
+        hn = torch.empty_like(hp)
+        bench_kernel("embedding_rmsnorm_T2048", lambda i: T.embedding_rmsnorm_forward(idp, table, scales[i % N_LAYERS], 1e-5, x_out=hp, out=hn),
+                     bytes_of["embedding"](2048) + 2048 * HIDDEN * 2 + HIDDEN * 2, n=96)
         sx = torch.empty(32768, 2 * HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 2, generator=gg)
         so = torch.empty(32768, HIDDEN, dtype=torch.bfloat16, device=dev)
         bench_kernel("swiglu_M32768", lambda i: T.swiglu(sx, out=so), bytes_of["swiglu"](32768), n=48)
@@ -551,8 +554,9 @@ def main() -> int:
 
             def chain(i, idp=idp, xp=xp, tn=tn, pp=pp, qo=qo, sx=sx, so=so, with_gather=with_gather):
                 if with_gather:
-                    T.embedding_forward(idp, table, out=xp)
-                T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=tn)
+                    T.embedding_rmsnorm_forward(idp, table, scales[i % N_LAYERS], 1e-5, x_out=xp, out=tn)      # one launch
+                else:
+                    T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=tn)
                 T.qkv_rope_forward(tn, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn, positions=pp, mode="prefill", out=qo)
                 if sx is not None:
                     T.swiglu(sx, out=so)
@@ -561,7 +565,7 @@ def main() -> int:
             gr = graph_of(chain, 24)
             gr.replay()
             sec = min(time_graph(gr) for _ in range(5)) / 24
-            prefill_chains[f"T{tt}"] = {"chain": ("gather + " if with_gather else "") + "RMSNorm + QKV/bias/RoPE" + (" + SwiGLU[32768,5760]" if swiglu_rows else ""),
+            prefill_chains[f"T{tt}"] = {"chain": ("gather/RMSNorm (one launch)" if with_gather else "RMSNorm") + " + QKV/bias/RoPE" + (" + SwiGLU[32768,5760]" if swiglu_rows else ""),
                                         "us": round(sec * 1e6, 2), "tokens/s": round(tt / sec, 1)}
             del xp, tn, qo, sx, so
 

@@ -75,6 +75,16 @@ const char* tllm_last_error(void);
 int tllm_rmsnorm_bf16(const void* x, const void* scale, int scale_is_bf16, void* out,
                       int64_t rows, int64_t hidden, float eps, void* stream);
 
+/* Token gather and RMSNorm of the gathered rows in one launch: x_out[t, :] = table[ids[t], :] (bit-exact; the hidden
+ * state, torch.nn.Embedding at model.py:906-908, 920) and out[t, :] = RMSNorm(x_out[t, :]) (the first block's norm,
+ * model.py:476; same arithmetic as tllm_rmsnorm_bf16, so the results are identical to the two calls). ids int32 or
+ * int64; an id outside [0, vocab) gives a zero row in both outputs and sets *oob_flag (device int, may be NULL) to 1.
+ * hidden must be a multiple of 8 up to 8192, x_out and out different buffers. No counterpart in the reference (two
+ * launches there). */
+int tllm_embed_rmsnorm_bf16(const void* table, const void* ids, int ids_is_i64, void* x_out, const void* scale,
+                            int scale_is_bf16, void* out, int64_t n_tokens, int64_t hidden, int64_t vocab, float eps,
+                            int* oob_flag, void* stream);
+
 /* out[t,:] = table[ids[t],:], bit-exact row gather.
  * replaces torch.nn.Embedding forward, model.py:906-908, 920.
  * ids are int32 (the reference's token tensors, model.py:1170) or int64.

@@ -978,6 +978,46 @@ def test_attention_block_prefill_chain(gpu):
             close(t, want)
 
 
+@pytest.mark.parametrize("n_tokens", [1, 8, 300, 512, 513, 2048])
+@pytest.mark.parametrize("scale_dtype", [torch.bfloat16, torch.float32])
+def test_embedding_rmsnorm_one_launch(gpu, n_tokens, scale_dtype):
+    """Gather + RMSNorm of the gathered rows in one launch (both row-count regimes of the norm kernel): the hidden state
+    is bit-exact, the normalised rows equal the separate rmsnorm_forward bit for bit and the oracle within tolerance."""
+    g = torch.Generator().manual_seed(n_tokens)
+    table = (0.02 * torch.randn(5000, 2880, generator=g)).bfloat16()
+    scale = (1 + 0.1 * torch.randn(2880, generator=g)).to(scale_dtype)
+    for dt in (torch.int32, torch.int64):
+        ids = torch.randint(0, 5000, (1, n_tokens), generator=g).to(dt)
+        ids[0, 0], ids[0, -1] = 4999, 0
+        x, t = T.embedding_rmsnorm_forward(ids.to(gpu), table.to(gpu), scale.to(gpu), 1e-5)
+        assert x.shape == (1, n_tokens, 2880) and t.shape == x.shape
+        x_ref = O.embedding_ref(table, ids)
+        assert torch.equal(x.cpu(), x_ref)
+        assert torch.equal(t, T.rmsnorm_forward(x, scale.to(gpu), 1e-5, out=torch.empty_like(x)))
+        close(t, O.rmsnorm_ref(x_ref, scale.float(), 1e-5))
+
+
+def test_embedding_rmsnorm_bad_ids_and_other_widths(gpu):
+    g = torch.Generator().manual_seed(5)
+    table = (0.02 * torch.randn(100, 256, generator=g)).bfloat16()
+    scale = (1 + 0.1 * torch.randn(256, generator=g)).bfloat16()
+    ids = torch.tensor([3, -1, 99, 100, 7], dtype=torch.int64)
+    flag = torch.zeros(1, dtype=torch.int32, device=gpu)
+    x, t = T.embedding_rmsnorm_forward(ids.to(gpu), table.to(gpu), scale.to(gpu), 1e-5, oob_flag=flag)
+    assert flag.item() == 1
+    good = torch.tensor([0, 2, 4])
+    assert torch.equal(x.cpu()[good], table[ids[good]])
+    assert x.cpu()[1].abs().max() == 0 and x.cpu()[3].abs().max() == 0 and t.cpu()[1].abs().max() == 0 and t.cpu()[3].abs().max() == 0
+    close(t.cpu()[good], O.rmsnorm_ref(table[ids[good]], scale.float(), 1e-5))
+    # a width the fused kernel does not take: composed from the two calls, same results
+    table2 = (0.02 * torch.randn(50, 100, generator=g)).bfloat16()
+    scale2 = torch.ones(100)
+    ids2 = torch.randint(0, 50, (9,), generator=g, dtype=torch.int32)
+    x2, t2 = T.embedding_rmsnorm_forward(ids2.to(gpu), table2.to(gpu), scale2.to(gpu), 1e-5)
+    assert torch.equal(x2.cpu(), table2[ids2.long()])
+    close(t2, O.rmsnorm_ref(table2[ids2.long()], scale2, 1e-5))
+
+
 # ----------------------------------------------------------------------------------- MXFP4 checkpoint expansion
 def _bits_equal_nan_aware(out, ref):
     out = out.cpu()

@@ -8,6 +8,7 @@ from .ops import (
     attention_decode,
     embed_qkv_rope_forward,
     embedding_forward,
+    embedding_rmsnorm_forward,
     linear_qkv_forward,
     mxfp4_dequant,
     out_residual_decode_forward,
@@ -29,7 +30,7 @@ from .yarn import YarnParams, gpt_oss_yarn
 
 __all__ = [
     "Checkpoint", "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
-    "attention", "attention_decode", "embed_qkv_rope_forward", "embedding_forward", "linear_qkv_forward", "mxfp4_dequant", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
+    "attention", "attention_decode", "embed_qkv_rope_forward", "embedding_forward", "embedding_rmsnorm_forward", "linear_qkv_forward", "mxfp4_dequant", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
     "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu", "UnEmbedding", "unembedding_decode_forward", "unembedding_decode_argmax_forward",
     "unembedding_decode_fp8_forward", "unembedding_decode_fp8_argmax_forward", "unembedding_forward",
 ]

@@ -57,6 +57,7 @@ SIGNATURES = {
     "tllm_attention_decode_workspace_bytes": (_i64, [_i64, _i32, _i32, _i64, _i32]),
     "tllm_attention_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _vp,
                                           _i32, _i64, _vp, _i64, _vp]),
+    "tllm_embed_rmsnorm_bf16": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _f32, _vp, _vp]),
     "tllm_attention_prefill_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32,
                                            _f32, _i32, _vp, _i32, _vp]),
     "tllm_mxfp4_dequant_bf16": (_i32, [_vp, _vp, _vp, _i64, _vp]),

@@ -8,9 +8,32 @@
 //                      single row's latency is spread over four wavefronts;
 //                      shuffle inside each wavefront, then a 4-entry LDS exchange.
 // A scalar two-pass kernel covers hidden sizes / alignments the vector paths do not.
+//
+// GATHER form (the first layer of a prompt: x = table[ids] followed by RMSNorm(x), model.py:920 and :476): the row
+// comes from the embedding table by token id, is written out unchanged (the hidden state, bit-exact) and normalised
+// from the same registers -- one launch and one read of the row instead of two of each. An id outside the table
+// yields a zero row (and a zero normalised row) and sets a device flag, as in the gather kernel.
 #include "common.h"
 
 namespace tllm {
+
+struct GatherSrc {
+  const void* ids;        // [rows] int32 or int64
+  int ids_is_i64;
+  int64_t vocab;
+  bf16x8* x_out;          // [rows, nvec]: the gathered rows
+  int* oob;               // device flag or null
+};
+
+// row base in the table (null: id out of range)
+__device__ __forceinline__ const bf16x8* gather_row(const GatherSrc& g, const bf16x8* table, int64_t row, int nvec, bool flag_lane) {
+  const int64_t id = g.ids_is_i64 ? reinterpret_cast<const int64_t*>(g.ids)[row] : reinterpret_cast<const int*>(g.ids)[row];
+  if (id < 0 || id >= g.vocab) {
+    if (flag_lane && g.oob) *g.oob = 1;
+    return nullptr;
+  }
+  return table + id * nvec;
+}
 
 template <bool kScaleBf16>
 __device__ __forceinline__ void load_scale8(const void* scale, int vec, float s[8]) {
@@ -50,22 +73,29 @@ __device__ __forceinline__ float sumsq8(bf16x8 v) {
 }
 
 // One wavefront per row; VPL = 16-byte vectors per lane (row length <= VPL*64*8).
-template <int VPL, bool kScaleBf16>
+template <int VPL, bool kScaleBf16, bool GATHER>
 __global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const bf16x8* x, const void* __restrict__ scale,
-                                                           bf16x8* out, int64_t rows, int nvec, float hidden_f, float eps) {
+                                                           bf16x8* out, int64_t rows, int nvec, float hidden_f, float eps, GatherSrc g) {
   const int lane = threadIdx.x & 63;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
-  const bf16x8* xr = x + row * nvec;
+  const bf16x8* xr = GATHER ? gather_row(g, x, row, nvec, lane == 0) : x + row * nvec;
   bf16x8 v[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int idx = lane + i * 64;
-    if (idx < nvec) {
+    if (idx < nvec && (!GATHER || xr != nullptr)) {
       v[i] = xr[idx];
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[i][j] = static_cast<bf16>(0.f);
+    }
+  }
+  if constexpr (GATHER) {
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int idx = lane + i * 64;
+      if (idx < nvec) __builtin_nontemporal_store(v[i], g.x_out + row * nvec + idx);
     }
   }
   float ss = 0.f;
@@ -82,22 +112,29 @@ __global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const bf16x8* x, cons
 }
 
 // One 256-lane workgroup per row; VPT = 16-byte vectors per thread.
-template <int VPT, bool kScaleBf16>
+template <int VPT, bool kScaleBf16, bool GATHER>
 __global__ __launch_bounds__(256) void rmsnorm_block_kernel(const bf16x8* x, const void* __restrict__ scale,
-                                                            bf16x8* out, int nvec, float hidden_f, float eps) {
+                                                            bf16x8* out, int nvec, float hidden_f, float eps, GatherSrc g) {
   __shared__ float part[4];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
-  const bf16x8* xr = x + row * nvec;
+  const bf16x8* xr = GATHER ? gather_row(g, x, row, nvec, tid == 0) : x + row * nvec;
   bf16x8 v[VPT];
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int idx = tid + i * 256;
-    if (idx < nvec) {
+    if (idx < nvec && (!GATHER || xr != nullptr)) {
       v[i] = xr[idx];
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[i][j] = static_cast<bf16>(0.f);
+    }
+  }
+  if constexpr (GATHER) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = tid + i * 256;
+      if (idx < nvec) __builtin_nontemporal_store(v[i], g.x_out + row * nvec + idx);
     }
   }
   float ss = 0.f;
@@ -142,13 +179,13 @@ __global__ __launch_bounds__(256) void rmsnorm_scalar_kernel(const bf16* x, cons
   }
 }
 
-template <bool kScaleBf16>
+template <bool kScaleBf16, bool GATHER>
 static void launch_wave(int vpl, const bf16x8* x, const void* scale, bf16x8* out, int64_t rows, int nvec, float inv_h, float eps,
-                        hipStream_t st) {
+                        const GatherSrc& g, hipStream_t st) {
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(256);
-#define TLLM_CASE(V)                                                                                           \
-  case V:                                                                                                      \
-    hipLaunchKernelGGL((rmsnorm_wave_kernel<V, kScaleBf16>), grid, block, 0, st, x, scale, out, rows, nvec, inv_h, eps); \
+#define TLLM_CASE(V)                                                                                                             \
+  case V:                                                                                                                        \
+    hipLaunchKernelGGL((rmsnorm_wave_kernel<V, kScaleBf16, GATHER>), grid, block, 0, st, x, scale, out, rows, nvec, inv_h, eps, g); \
     break;
   switch (vpl) {
     TLLM_CASE(1) TLLM_CASE(2) TLLM_CASE(3) TLLM_CASE(4) TLLM_CASE(5) TLLM_CASE(6) TLLM_CASE(7) TLLM_CASE(8)
@@ -157,13 +194,13 @@ static void launch_wave(int vpl, const bf16x8* x, const void* scale, bf16x8* out
 #undef TLLM_CASE
 }
 
-template <bool kScaleBf16>
+template <bool kScaleBf16, bool GATHER>
 static void launch_block(int vpt, const bf16x8* x, const void* scale, bf16x8* out, int64_t rows, int nvec, float inv_h, float eps,
-                         hipStream_t st) {
+                         const GatherSrc& g, hipStream_t st) {
   dim3 grid(static_cast<unsigned>(rows)), block(256);
-#define TLLM_CASE(V)                                                                                      \
-  case V:                                                                                                 \
-    hipLaunchKernelGGL((rmsnorm_block_kernel<V, kScaleBf16>), grid, block, 0, st, x, scale, out, nvec, inv_h, eps); \
+#define TLLM_CASE(V)                                                                                                        \
+  case V:                                                                                                                   \
+    hipLaunchKernelGGL((rmsnorm_block_kernel<V, kScaleBf16, GATHER>), grid, block, 0, st, x, scale, out, nvec, inv_h, eps, g); \
     break;
   switch (vpt) { TLLM_CASE(1) TLLM_CASE(2) TLLM_CASE(3) TLLM_CASE(4) }
 #undef TLLM_CASE
@@ -176,6 +213,31 @@ using namespace tllm;
 // Rows at or below this go to the workgroup-per-row kernel (latency), above to wave-per-row (throughput).
 static constexpr int64_t kBlockPerRowMaxRows = 512;
 
+// Shared by the plain and the gather form: the two vector kernels by row count.
+template <bool GATHER>
+static bool launch_vector(const void* x, const void* scale, int scale_is_bf16, void* out, int64_t rows, int64_t hidden, float eps,
+                          const GatherSrc& g, hipStream_t st) {
+  const float inv_h = static_cast<float>(hidden);  // divisor of the mean
+  const int64_t nvec = hidden / 8;
+  if (rows <= kBlockPerRowMaxRows && nvec <= 4 * 256) {
+    const int vpt = static_cast<int>((nvec + 255) / 256);
+    if (scale_is_bf16)
+      launch_block<true, GATHER>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+    else
+      launch_block<false, GATHER>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+    return true;
+  }
+  if (nvec <= 16 * 64) {
+    const int vpl = static_cast<int>((nvec + 63) / 64);
+    if (scale_is_bf16)
+      launch_wave<true, GATHER>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+    else
+      launch_wave<false, GATHER>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+    return true;
+  }
+  return false;
+}
+
 extern "C" int tllm_rmsnorm_bf16(const void* x, const void* scale, int scale_is_bf16, void* out, int64_t rows, int64_t hidden,
                                  float eps, void* stream) {
   TLLM_REQUIRE(rows >= 0 && hidden > 0, TLLM_E_ARG, "rmsnorm: rows %lld / hidden %lld invalid", (long long)rows, (long long)hidden);
@@ -183,24 +245,28 @@ extern "C" int tllm_rmsnorm_bf16(const void* x, const void* scale, int scale_is_
   TLLM_REQUIRE(x && scale && out, TLLM_E_ARG, "rmsnorm: null pointer");
   TLLM_REQUIRE(rows < (1ll << 31), TLLM_E_SHAPE, "rmsnorm: rows %lld too large", (long long)rows);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const float inv_h = static_cast<float>(hidden);  // divisor of the mean
   const bool vec_ok = hidden % 8 == 0 && aligned16(x) && aligned16(out) && aligned16(scale);
-  const int64_t nvec = hidden / 8;
-  if (vec_ok && rows <= kBlockPerRowMaxRows && nvec <= 4 * 256) {
-    const int vpt = static_cast<int>((nvec + 255) / 256);
-    if (scale_is_bf16)
-      launch_block<true>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, st);
-    else
-      launch_block<false>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, st);
-  } else if (vec_ok && nvec <= 16 * 64) {
-    const int vpl = static_cast<int>((nvec + 63) / 64);
-    if (scale_is_bf16)
-      launch_wave<true>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, st);
-    else
-      launch_wave<false>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, st);
-  } else {
+  if (!(vec_ok && launch_vector<false>(x, scale, scale_is_bf16, out, rows, hidden, eps, GatherSrc{}, st))) {
     hipLaunchKernelGGL(rmsnorm_scalar_kernel, dim3((unsigned)rows), dim3(256), 0, st, (const bf16*)x, scale, scale_is_bf16,
-                       (bf16*)out, hidden, inv_h, eps);
+                       (bf16*)out, hidden, static_cast<float>(hidden), eps);
   }
   return check_launch("rmsnorm");
+}
+
+extern "C" int tllm_embed_rmsnorm_bf16(const void* table, const void* ids, int ids_is_i64, void* x_out, const void* scale,
+                                       int scale_is_bf16, void* out, int64_t n_tokens, int64_t hidden, int64_t vocab, float eps,
+                                       int* oob_flag, void* stream) {
+  TLLM_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, TLLM_E_ARG, "embed_rmsnorm: n_tokens %lld / hidden %lld / vocab %lld invalid",
+               (long long)n_tokens, (long long)hidden, (long long)vocab);
+  if (n_tokens == 0) return TLLM_OK;
+  TLLM_REQUIRE(table && ids && x_out && scale && out, TLLM_E_ARG, "embed_rmsnorm: null pointer");
+  TLLM_REQUIRE(n_tokens < (1ll << 31), TLLM_E_SHAPE, "embed_rmsnorm: n_tokens %lld too large", (long long)n_tokens);
+  TLLM_REQUIRE(hidden % 8 == 0 && hidden <= 8192 && aligned16(table) && aligned16(x_out) && aligned16(out) && aligned16(scale), TLLM_E_SHAPE,
+               "embed_rmsnorm: hidden %lld must be a multiple of 8 up to 8192 and all pointers 16-byte aligned (otherwise: the two "
+               "separate calls)", (long long)hidden);
+  TLLM_REQUIRE(x_out != out, TLLM_E_ARG, "embed_rmsnorm: x_out and out must be different buffers");
+  GatherSrc g{ids, ids_is_i64, vocab, (bf16x8*)x_out, oob_flag};
+  const bool ok = launch_vector<true>(table, scale, scale_is_bf16, out, n_tokens, hidden, eps, g, static_cast<hipStream_t>(stream));
+  TLLM_REQUIRE(ok, TLLM_E_SHAPE, "embed_rmsnorm: hidden %lld not covered", (long long)hidden);
+  return check_launch("embed_rmsnorm");
 }

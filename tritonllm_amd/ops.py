@@ -134,6 +134,43 @@ def embedding_forward(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor 
     return out
 
 
+def embedding_rmsnorm_forward(ids: torch.Tensor, table: torch.Tensor, scale: torch.Tensor, eps: float,
+                              x_out: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                              oob_flag: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """``x = table[ids]`` (model.py:906-908, 920) and ``RMSNorm(x)`` of the first block (model.py:476) in one launch.
+    Returns ``(x, normed)``, both ``[*ids.shape, hidden]``: ``x`` bit-exact like ``embedding_forward`` (a fresh tensor
+    unless ``x_out`` is given), ``normed`` identical to ``rmsnorm_forward(x, scale, eps)`` (pooled unless ``out`` is given).
+    Hidden sizes the fused kernel does not cover take the two separate calls."""
+    _on_gpu(ids, table, scale, x_out, out, oob_flag)
+    assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
+    assert ids.dtype in (torch.int32, torch.int64)
+    assert scale.dtype in (torch.float32, _BF16), "embedding_rmsnorm_forward: scale must be float32 or bfloat16"
+    vocab, hidden = table.shape
+    assert scale.shape == (hidden,)
+    if hidden % 8 != 0 or hidden > 8192:
+        x = embedding_forward(ids, table, out=x_out, oob_flag=oob_flag)
+        return x, rmsnorm_forward(x, scale, eps, out=out)
+    if not ids.is_contiguous():
+        ids = ids.contiguous()
+    if not scale.is_contiguous():
+        scale = scale.contiguous()
+    shape = (*ids.shape, hidden)
+    if x_out is None:
+        x_out = torch.empty(shape, dtype=table.dtype, device=table.device)
+    if out is None:
+        out = scratch_pool.get(shape, table.dtype, table.device)
+    for t in (x_out, out):
+        assert tuple(t.shape) == shape and t.dtype == table.dtype and t.is_contiguous()
+    assert x_out.data_ptr() != out.data_ptr()
+    if oob_flag is not None:
+        assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
+    rc = lib().tllm_embed_rmsnorm_bf16(table.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64), x_out.data_ptr(), scale.data_ptr(),
+                                       int(scale.dtype == _BF16), out.data_ptr(), ids.numel(), hidden, vocab, float(eps),
+                                       oob_flag.data_ptr() if oob_flag is not None else None, _stream())
+    check(rc, "embedding_rmsnorm_forward")
+    return x_out, out
+
+
 # --------------------------------------------------------------------------------------- SwiGLU
 def swiglu(x: torch.Tensor, alpha: float = 1.702, limit: float | None = 7.0, interleaved: bool = True,
            out: torch.Tensor | None = None) -> torch.Tensor:
