@@ -11,7 +11,10 @@ in one HIP graph and replayed, which is how the reference runs its decode loop.
 Prints ONE JSON line: whole-job tokens/s, plus `roofline` for the dominant kernel (the
 decode QKV stream), `cpu_baseline` (the eager bf16 PyTorch restatement of the reference
 chain timed on the host cores) and a `kernels` table with every kernel at its decode and
-prefill sizes (GB/s against 8 TB/s, or TFLOP/s against 2.5 PFLOP/s bf16 for prefill QKV).
+prefill sizes (GB/s against 8 TB/s, or TFLOP/s against 2.5 PFLOP/s bf16 for the prefill QKV and
+prefill attention kernels), `stack24` (the 24-layer per-token stack at B = 1, 8, 32), `prefill_chains`
+(the two prefill configurations as chains) and `attention_blocks24` (the attention half of the
+layers for a decode token and for a whole prompt).
 """
 from __future__ import annotations
 
