@@ -899,6 +899,38 @@ def test_attention_prefill_large_launch_ragged(gpu, sliding_window):
     _attn_prefill_case(gpu, 4, 600, 700, sliding_window, 77, start_dtype=torch.int64, seed=41)
 
 
+def test_attention_graph_replay_follows_device_start(gpu):
+    """Both attention kernels read start_q on the device: a graph captured once follows the tensor's new value on every
+    replay (decode: the growing context; prefill: the next chunk of a prompt), with eager work between the replays."""
+    g = torch.Generator().manual_seed(61)
+    bs, n_ctx, chunk = 2, 700, 150
+    k = torch.randn(bs, n_ctx, 8, 64, generator=g).bfloat16()
+    v = torch.randn(bs, n_ctx, 8, 64, generator=g).bfloat16()
+    q1 = torch.randn(bs, 1, 8, 8, 64, generator=g).bfloat16()
+    qn = torch.randn(bs, chunk, 8, 8, 64, generator=g).bfloat16()
+    sinks = torch.randn(64, generator=g).bfloat16()
+    kg, vg, q1g, qng, sg = k.to(gpu), v.to(gpu), q1.to(gpu), qn.to(gpu), sinks.to(gpu)
+    start = torch.zeros(1, dtype=torch.int64, device=gpu)
+    outs = {}
+
+    def both():
+        outs["dec"] = T.attention_decode(q1g, kg, vg, sg, 0.125, None, start)
+        outs["pre"] = T.attention(qng, kg, vg, sg, 0.125, 128, start)
+
+    both()                                        # warm up (allocates pool buffers)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        both()
+    for p in (0, 37, 300, 549, 37):
+        start.fill_(p)
+        graph.replay()
+        torch.cuda.synchronize()
+        close(outs["dec"], O.attention_decode_ref(q1, k, v, sinks, 0.125, None, p))
+        close(outs["pre"], O.attention_ref(qn, k, v, sinks, 0.125, 128, p))
+        T.rmsnorm_forward(qng.view(-1, 4096)[:4], torch.ones(4096, device=gpu), 1e-5)   # eager work between the replays
+
+
 def test_attention_prefill_argument_errors(gpu):
     q = torch.zeros(1, 16, 8, 8, 64, dtype=torch.bfloat16, device=gpu)
     k = torch.zeros(1, 16, 8, 64, dtype=torch.bfloat16, device=gpu)
