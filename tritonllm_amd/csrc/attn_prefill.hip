@@ -101,10 +101,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
   const int tile = ntiles - 1 - static_cast<int>(id);
   const int head0 = kvh * a.group + (sub * HS + wave / QG) * NH;
 
-  const int start = a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
+  // ---- Q fragments (B operand: lane = query, 8 d per half-wavefront and k16 step), requested before the start
+  // position is read: their addresses do not depend on it, so they travel while that (dependent) load is on its way
   const int q0 = tile * PBM;
   const int qw0 = q0 + (wave % QG) * 32;   // the wavefront's first query
-  const int p0 = start + qw0;              // and its position
+  bf16x8 qf[NH][4];
+  {
+    int qrow = qw0 + l31;
+    qrow = qrow < a.n_q ? qrow : a.n_q - 1;
+    const bf16* qp = a.q + b * a.q_bs + static_cast<int64_t>(qrow) * a.q_ts + head0 * 64 + h * 8;
+#pragma unroll
+    for (int hd = 0; hd < NH; ++hd)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) qf[hd][kk] = *reinterpret_cast<const bf16x8*>(qp + hd * 64 + kk * 16);
+  }
+
+  const int start = a.start_is_i64 ? static_cast<int>(*reinterpret_cast<const int64_t*>(a.start_q)) : *reinterpret_cast<const int*>(a.start_q);
+  const int p0 = start + qw0;              // the position of the wavefront's first query
   const int q_end = q0 + PBM < a.n_q ? q0 + PBM : a.n_q;
   int kv_hi = start + q_end < a.n_kv_ctx ? start + q_end : a.n_kv_ctx;       // keys the tile's last query sees (exclusive)
   kv_hi = kv_hi > 0 ? kv_hi : 0;
@@ -186,16 +199,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
   for (int i = 0; i < 2; ++i)
     if (i < nblk) issue_block(blk_lo + i, i);
 
-  // ---- Q fragments (B operand: lane = query, 8 d per half-wavefront and k16 step)
-  bf16x8 qf[NH][4];
   {
-    int qrow = qw0 + l31;
-    qrow = qrow < a.n_q ? qrow : a.n_q - 1;
-    const bf16* qp = a.q + b * a.q_bs + static_cast<int64_t>(qrow) * a.q_ts + head0 * 64 + h * 8;
-#pragma unroll
-    for (int hd = 0; hd < NH; ++hd)
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) qf[hd][kk] = *reinterpret_cast<const bf16x8*>(qp + hd * 64 + kk * 16);
     // The compiler does not see the direct-to-LDS loads in its count of outstanding loads; were the fragments first
     // used inside the loop, its wait for them there would be "nothing outstanding" and drain the blocks in flight on
     // every step. Pin the wait here, where the first blocks have to land anyway.
