@@ -259,7 +259,7 @@ int tllm_attention_decode_bf16(const void* q, const void* k, const void* v, cons
                                int64_t kv_len_hint, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Prefill attention with sinks and an optional sliding window: n_q query positions per batch row against the keys
- * written so far. Replaces attention (attention_tt.py:166-236, kernel :17-164; definition attention_ref.py:4-42).
+ * written so far. Replaces attention (attention_tt.py:167-242, kernel :17-164; definition attention_ref.py:4-42).
  * q [batch, n_q, n_kv_heads * group, 64] with batch / token strides in elements (heads adjacent: the layout the QKV
  * projection writes), k / v [batch, n_kv_ctx, n_kv_heads, 64] with batch / token strides (a view of the KV cache
  * will do), sinks [n_kv_heads * group] bf16 or NULL (logit 0, :103-106), out [batch, n_q, n_kv_heads * group * 64].

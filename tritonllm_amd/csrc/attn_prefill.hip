@@ -1,5 +1,5 @@
 // Prefill attention with learned sinks and an optional sliding window: many query positions per batch row against
-// the keys written so far (attention, attention_tt.py:166-236; kernel :17-164; definition attention_ref.py:4-42):
+// the keys written so far (attention, attention_tt.py:167-242; kernel :17-164; definition attention_ref.py:4-42):
 //
 //   query i of a batch row sits at position p = start_q + i and sees the keys n with
 //       n <= p,   n < n_kv_ctx,   n > p - window (when a window is set)
@@ -36,7 +36,7 @@ struct AttnPrefillArgs {
   const bf16* q;          // [B, n_q, n_heads, 64]: batch stride q_bs, token stride q_ts (elements), heads adjacent
   const bf16* k;          // [B, n_kv_ctx, n_kv_heads, 64]: batch stride kv_bs, token stride kv_ts
   const bf16* v;
-  const bf16* sinks;      // [n_heads] or null (logit 0, attention_tt.py:103-106)
+  const bf16* sinks;      // [n_heads] or null (logit 0, attention_tt.py:100-104)
   bf16* out;              // [B, n_q, n_heads * 64]: batch stride out_bs, token stride out_ts
   const void* start_q;    // device scalar
   int start_is_i64;

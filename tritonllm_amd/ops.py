@@ -640,7 +640,7 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: t
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Tensor | None, sm_scale: float,
               bandwidth: int | None, start_q: torch.Tensor) -> torch.Tensor:
-    """Prefill attention with sinks and an optional sliding window (attention, attention_tt.py:166-236):
+    """Prefill attention with sinks and an optional sliding window (attention, attention_tt.py:167-242):
     ``q [bs, n_ctx, n_kv_heads, repeat_kv, 64]``, ``k, v [bs, n_kv_ctx, n_kv_heads, 64]``, ``sinks [n_heads]`` bf16,
     ``start_q`` a device tensor of one int32/int64 element (query ``i`` sits at position ``start_q + i``; read on the
     device), ``bandwidth`` the sliding window (``None`` / 0: none). Returns ``[bs, n_ctx, n_heads * 64]`` (pooled).
