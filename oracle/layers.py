@@ -187,9 +187,9 @@ def attention_ref(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, s
     ``[bs, n_queries, heads*hd]``.
 
     query ``[bs, n_queries, kv_heads, groups, hd]``, key/value ``[bs, n_keys, kv_heads, hd]``, sinks ``[kv_heads*groups]``
-    (``None``: logit 0, attention_tt.py:100-104). Query ``i`` sits at position ``start_q + i`` (:20); keys after that
-    position are masked (:21-22), keys older than ``position - sliding_window + 1`` too (:24-26); the sink joins the
-    softmax denominator but contributes no value (:31-36). A query that sees no key yields zeros."""
+    (``None``: logit 0, attention_tt.py:100-104). Query ``i`` sits at position ``start_q + i`` (:21); keys after that
+    position are masked (:22-23), keys older than ``position - sliding_window + 1`` too (:25-27); the sink joins the
+    softmax denominator but contributes no value (:31-37). A query that sees no key yields zeros."""
     bs, nq, n_kv, groups, hd = query.shape
     n_keys = key.shape[1]
     sink = torch.zeros(n_kv * groups) if sinks is None else sinks.to(torch.float32)

@@ -646,7 +646,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Te
     device), ``bandwidth`` the sliding window (``None`` / 0: none). Returns ``[bs, n_ctx, n_heads * 64]`` (pooled).
 
     ``q`` may be a view into the fused QKV output and ``k`` / ``v`` views of the cache: the kernel takes batch and
-    token strides, so none of the reference's transposed, padded copies (:178-191) is made."""
+    token strides, so none of the reference's transposed, padded copies (:180-191) is made."""
     _on_gpu(q, k, v, sinks, start_q)
     assert len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64)
     bs, n_ctx, n_kv_heads, repeat_kv, head_dim_q = q.shape
