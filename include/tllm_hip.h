@@ -168,7 +168,7 @@ int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int sc
  * feeding the first block's RMSNorm + QKV + bias + rotary (model.py:476, 489-503). x_out[r, :] = table[ids[r], :]
  * (bit-exact, [rows, hidden] dense: the residual stream the following layers read), and q / k / v as
  * tllm_norm_qkv_rope_decode_bf16 computes them from x_out. ids: int32 or int64 [rows]; an id outside [0, vocab)
- * reads row 0 or vocab - 1 and sets *oob_flag (may be NULL) -- unlike tllm_embedding_bf16, which writes zeros for it.
+ * gives a zero row in x_out (and q / k / v computed from it) and sets *oob_flag (may be NULL), as tllm_embedding_bf16 does.
  * w_scale: NULL for a bf16 W, else W holds fp8 bytes as in tllm_qkv_rope_decode_w8_bf16. norm_scale must not be
  * NULL; hidden 2880, head_dim 64, rows <= 16 (larger batches: gather, then the QKV entry point). */
 int tllm_embed_norm_qkv_rope_decode_bf16(const void* ids, int ids_is_i64, const void* table, int64_t vocab, void* x_out,

@@ -197,6 +197,43 @@ def test_rope_module_tables_and_per_row_positions(gpu, yarn):
     close(kg, O.rope_rotate_ref(k.view(-1, 8, 64), cos, sin).view(k.shape))
 
 
+@pytest.mark.parametrize("scaling_factor", [32.0, 1.0])
+def test_yarn_table_whole_context(gpu, scaling_factor):
+    """The device's sin/cos routine (the one every rotary kernel uses in registers) over ALL 131072 positions x 32
+    frequencies, in fp32, against the oracle's tables (model.py:307-313 restated): absolute error within
+    4e-7 x concentration, i.e. a few units in the last place of values of magnitude ~1. YaRN and plain RoPE."""
+    yp = T.YarnParams(head_dim=64, base=150000.0, initial_context_length=4096, scaling_factor=scaling_factor, ntk_alpha=1.0, ntk_beta=32.0)
+    cos = torch.empty(O.MAX_CTX, 32, dtype=torch.float32, device=gpu)
+    sin = torch.empty(O.MAX_CTX, 32, dtype=torch.float32, device=gpu)
+    import ctypes
+    from tritonllm_amd import _lib
+    rc = _lib.lib().tllm_yarn_table_f32(cos.data_ptr(), sin.data_ptr(), 0, O.MAX_CTX, ctypes.byref(yp.c_struct()),
+                                        torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    cos_ref, sin_ref = O.yarn_cos_sin(torch.arange(O.MAX_CTX), scaling_factor=scaling_factor)
+    conc = 0.1 * __import__("math").log(scaling_factor) + 1.0 if scaling_factor > 1 else 1.0
+    assert abs(yp.concentration - conc) < 1e-12
+    torch.testing.assert_close(cos.cpu(), cos_ref, rtol=0, atol=4e-7 * conc)
+    torch.testing.assert_close(sin.cpu(), sin_ref, rtol=0, atol=4e-7 * conc)
+    # a table requested from the middle of the context is the same numbers
+    c2 = torch.empty(1000, 32, dtype=torch.float32, device=gpu)
+    s2 = torch.empty(1000, 32, dtype=torch.float32, device=gpu)
+    rc = _lib.lib().tllm_yarn_table_f32(c2.data_ptr(), s2.data_ptr(), 130000, 1000, ctypes.byref(yp.c_struct()), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(c2, cos[130000:131000]) and torch.equal(s2, sin[130000:131000])
+
+
+def test_rope_positions_must_cover_every_row(gpu, yarn):
+    """The kernels read positions[row] for every row; a shorter tensor is refused on the host."""
+    q, k = _qk(4, 1, seed=14)
+    with pytest.raises(AssertionError):
+        T.rope_forward(q.to(gpu), k.to(gpu), None, None, O.MAX_CTX, None, yarn=yarn, positions=torch.zeros(3, dtype=torch.int64, device=gpu))
+    d = O.make_inputs(8, seed=15)
+    with pytest.raises(AssertionError):
+        T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"][:7].to(gpu))
+    with pytest.raises((AssertionError, RuntimeError)):
+        T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"])   # CPU positions
+
+
 def test_rope_norm_property_full_size(gpu, yarn):
     q, k = _qk(1, 8192, seed=13)
     qg, kg = q.to(gpu), k.to(gpu)
@@ -296,7 +333,7 @@ def test_embed_norm_qkv_fp8_weight_and_bad_ids(gpu, yarn):
     q2, k2, v2 = T.qkv_rope_forward(x, w8, d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), mode="decode",
                                     norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5, weight_scale=ws)
     assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
-    # ids outside the table: clamped to the nearest row, flag raised, no fault
+    # ids outside the table: a zero row (as the stand-alone gather gives), flag raised, no fault
     bad = ids.clone()
     bad[2], bad[5] = -7, 64
     flag = torch.zeros(1, dtype=torch.int32, device=gpu)
@@ -304,12 +341,46 @@ def test_embed_norm_qkv_fp8_weight_and_bad_ids(gpu, yarn):
                                           yarn=yarn, positions=d["positions"].to(gpu), oob_flag=flag)
     assert flag.item() == 1
     want = table[bad.clamp(0, 63)]
+    want[2] = 0
+    want[5] = 0
     assert torch.equal(x.cpu(), want)
     # pooled outputs and a caller-provided x_out
     xo = torch.empty(8, 2880, dtype=torch.bfloat16, device=gpu)
     x, *_ = T.embed_qkv_rope_forward(ids.to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64,
                                      yarn=yarn, positions=d["positions"].to(gpu), x_out=xo)
     assert x.data_ptr() == xo.data_ptr() and torch.equal(xo.cpu(), table[ids])
+
+
+@pytest.mark.parametrize("id_dtype", [torch.int32, torch.int64])
+def test_embed_qkv_bad_ids_same_policy_either_side_of_16_rows(gpu, yarn, id_dtype):
+    """One launch (<= 16 rows) and gather + QKV (> 16 rows) behind the same call treat an id outside the table alike: a
+    zero row of x, the q / k / v that follow from a zero row (the rotated bias), the flag raised -- and every other row
+    untouched by it."""
+    g = torch.Generator().manual_seed(41)
+    vocab = 300
+    table = torch.randn(vocab, 2880, generator=g).bfloat16()
+    for rows in (16, 17):
+        d = O.make_inputs(rows, seed=500 + rows)
+        ids = torch.randint(0, vocab, (rows,), generator=g, dtype=id_dtype)
+        ids[0], ids[rows // 2], ids[rows - 1] = -1, vocab, vocab + 12345
+        flag = torch.zeros(1, dtype=torch.int32, device=gpu)
+        x, q, k, v = T.embed_qkv_rope_forward(ids.to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, d["w"].to(gpu), d["b"].to(gpu),
+                                              64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), oob_flag=flag)
+        assert flag.item() == 1
+        ok = (ids >= 0) & (ids < vocab)
+        want_x = torch.where(ok[:, None], table[ids.long().clamp(0, vocab - 1)], torch.zeros((), dtype=torch.bfloat16))
+        assert torch.equal(x.cpu(), want_x), rows
+        t_ref = O.rmsnorm_ref(want_x, d["norm_scale"].float(), 1e-5).bfloat16()
+        assert (t_ref[~ok] == 0).all()
+        qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"])
+        close(q, qr)
+        close(k, kr)
+        close(v, vr)
+        # no bad id: the flag stays down
+        flag.zero_()
+        T.embed_qkv_rope_forward(ids.clamp(0, vocab - 1).to(gpu), table.to(gpu), d["norm_scale"].to(gpu), 1e-5, d["w"].to(gpu), d["b"].to(gpu),
+                                 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu), oob_flag=flag)
+        assert flag.item() == 0
 
 
 @pytest.mark.parametrize("rows", [17, 32, 50])
@@ -1126,3 +1197,140 @@ def test_checkpoint_mxfp4_on_gpu(gpu, tmp_path):
     assert b.is_cuda and torch.equal(b.cpu(), bias)
     dst = torch.empty(4, 96, 192, dtype=torch.bfloat16, device=gpu)
     assert ck.get("block.2.mlp.mlp2_weight", out=dst) is dst and torch.equal(dst, w)
+
+
+# ----------------------------------------------------------------------------------- pooled outputs vs inputs
+def test_pooled_outputs_never_alias_the_activations(gpu):
+    """hidden == n_q_heads * head_dim: the normalised activations (a borrowed pool buffer of shape [rows, hidden]) and q
+    have the same size. The projection must not be handed the buffer it is still reading as its output, neither when
+    it normalises by a preceding launch itself nor when the caller passes a pooled rmsnorm result as x."""
+    rows, hidden, nq, nkv, hd = 12, 4096, 64, 8, 64
+    d = O.make_inputs(rows, seed=61, hidden=hidden, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd)
+    yarn = T.gpt_oss_yarn()
+    t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"], n_q_heads=nq, n_kv_heads=nkv, head_dim=hd)
+    xg, wg, bg, sg, pg = d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), d["norm_scale"].to(gpu), d["positions"].to(gpu)
+    scratch_pool.clear()
+    # (a) the call normalises by a preceding launch (this shape has no fused norm)
+    q, k, v = T.qkv_rope_forward(xg, wg, bg, nq, nkv, hd, yarn=yarn, positions=pg, mode="decode", norm_scale=sg, norm_eps=1e-5)
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    # (b) the caller passes the pooled 2-D output of rmsnorm_forward as x
+    t = T.rmsnorm_forward(xg, sg, 1e-5)
+    assert t.data_ptr() == scratch_pool.get((rows, hidden), torch.bfloat16, gpu).data_ptr()
+    q, k, v = T.qkv_rope_forward(t, wg, bg, nq, nkv, hd, yarn=yarn, positions=pg, mode="decode")
+    assert q.data_ptr() != t.data_ptr()
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    # (c) the reference-signature decode call with a pooled [B, hidden] buffer viewed as [B, 1, hidden]
+    t = T.rmsnorm_forward(xg, sg, 1e-5)
+    q3, k3, v3 = T.qkv_decode_forward(t.view(rows, 1, hidden), wg, bg, nq * hd, nkv * hd)
+    assert q3.data_ptr() != t.data_ptr()
+    lin = O.linear_ref(t_ref, d["w"], d["b"])
+    close(q3.view(rows, -1), lin[:, :nq * hd])
+    close(k3.view(rows, -1), lin[:, nq * hd:(nq + nkv) * hd])
+    close(v3.view(rows, -1), lin[:, (nq + nkv) * hd:])
+    scratch_pool.clear()
+
+
+# ----------------------------------------------------------------------------------- 24-layer per-token stack
+N_STACK_LAYERS = 24
+
+
+@pytest.fixture(scope="module")
+def stack_weights(gpu):
+    """24 distinct layer weight sets (bf16 N(0, 0.02), norm scales 1 + 0.1 N), seeded on the CPU; the GPU copies are made once."""
+    g = torch.Generator().manual_seed(2024)
+    cpu = {
+        "w": [(0.02 * torch.randn(5120, 2880, generator=g)).bfloat16() for _ in range(N_STACK_LAYERS)],
+        "b": [(0.02 * torch.randn(5120, generator=g)).bfloat16() for _ in range(N_STACK_LAYERS)],
+        "attn": [(1 + 0.1 * torch.randn(2880, generator=g)).bfloat16() for _ in range(N_STACK_LAYERS)],
+        "mlp": [(1 + 0.1 * torch.randn(2880, generator=g)).bfloat16() for _ in range(N_STACK_LAYERS)],
+        "final": (1 + 0.1 * torch.randn(2880, generator=g)).bfloat16(),
+    }
+    dev = {key: ([t.to(gpu) for t in val] if isinstance(val, list) else val.to(gpu)) for key, val in cpu.items()}
+    return cpu, dev
+
+
+def _stack_inputs(batch, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(batch, 2880, generator=g).bfloat16()
+    pos = torch.randint(0, 8192, (batch,), generator=g, dtype=torch.int64)
+    sx = (2.0 * torch.randn(4 * batch, 5760, generator=g)).bfloat16()
+    return x, pos, sx
+
+
+def _check_stack(stack, final, cpu, x, pos, sx, what):
+    """Every layer's q / k / v, MLP-norm output and SwiGLU output, and the final norm, against the oracle."""
+    sw_ref = O.swiglu_ref(sx)
+    for l in range(N_STACK_LAYERS):
+        t_ref = O.rmsnorm_ref(x, cpu["attn"][l].float(), 1e-5).bfloat16()
+        qr, kr, vr = O.qkv_rope_ref(t_ref, cpu["w"][l], cpu["b"][l], pos)
+        for name, got, want in (("q", stack.q[l], qr), ("k", stack.k[l], kr), ("v", stack.v[l], vr),
+                                ("mlp norm", stack.mlp_normed[l], O.rmsnorm_ref(x, cpu["mlp"][l].float(), 1e-5)),
+                                ("swiglu", stack.swiglu_out[l], sw_ref)):
+            try:
+                close(got, want)
+            except AssertionError as e:
+                raise AssertionError(f"{what}: layer {l} {name}: {e}") from None
+    close(final, O.rmsnorm_ref(x, cpu["final"].float(), 1e-5))
+
+
+@pytest.mark.parametrize("batch", [1, 8, 32])
+def test_layer_stack24_token_step(gpu, stack_weights, batch):
+    """The whole per-token layer-kernel stack of a 24-layer gpt-oss-20b-shaped model -- per layer attention RMSNorm + QKV
+    + bias + YaRN rotary (inside one kernel up to 16 rows, two launches at 32), MLP RMSNorm, SwiGLU on [4B, 5760]; then
+    the final RMSNorm (model.py:471-526, 751-757, 918-923) -- with 24 distinct weight sets, run eagerly and as a
+    captured HIP graph replayed with new inputs, every layer's outputs against the oracle."""
+    from tritonllm_amd.stack import LayerKernelStack
+
+    cpu, dev = stack_weights
+    stack = LayerKernelStack(dev["w"], dev["b"], dev["attn"], dev["mlp"], dev["final"], T.gpt_oss_yarn(), batch, keep_layers=True)
+    assert stack.launches_per_step() == N_STACK_LAYERS * (3 if batch <= 16 else 4) + 1
+    x, pos, sx = _stack_inputs(batch, seed=700 + batch)
+    xg, pg, sg = x.to(gpu), pos.to(gpu), sx.to(gpu)
+    final = stack.token_step(xg, pg, sg)
+    torch.cuda.synchronize()
+    _check_stack(stack, final, cpu, x, pos, sx, f"eager B={batch}")
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        final_g = stack.token_step(xg, pg, sg)
+    for rep in range(3):
+        x, pos, sx = _stack_inputs(batch, seed=800 + 10 * batch + rep)
+        for buf in (stack.q, stack.k, stack.v, stack.mlp_normed, stack.swiglu_out, stack.final):
+            buf.fill_(float("nan"))                                    # nothing of the previous run may pass for a result
+        xg.copy_(x.to(gpu))
+        pg.copy_(pos.to(gpu))
+        sg.copy_(sx.to(gpu))
+        graph.replay()
+        torch.cuda.synchronize()
+        _check_stack(stack, final_g, cpu, x, pos, sx, f"graph replay {rep} B={batch}")
+
+
+def test_layer_stack24_shared_buffers_and_unfused_norm(gpu, stack_weights):
+    """The form the benchmark times (one output set reused by all layers) leaves the LAST layer's results behind, and the
+    stack with the attention norm as its own launch agrees with the fused one."""
+    from tritonllm_amd.stack import LayerKernelStack
+
+    cpu, dev = stack_weights
+    batch = 8
+    x, pos, sx = _stack_inputs(batch, seed=900)
+    outs = []
+    for fuse in (True, False):
+        stack = LayerKernelStack(dev["w"], dev["b"], dev["attn"], dev["mlp"], dev["final"], T.gpt_oss_yarn(), batch, fuse_norm=fuse)
+        assert stack.launches_per_step() == N_STACK_LAYERS * (3 if fuse else 4) + 1
+        final = stack.token_step(x.to(gpu), pos.to(gpu), sx.to(gpu))
+        l = N_STACK_LAYERS - 1
+        t_ref = O.rmsnorm_ref(x, cpu["attn"][l].float(), 1e-5).bfloat16()
+        qr, kr, vr = O.qkv_rope_ref(t_ref, cpu["w"][l], cpu["b"][l], pos)
+        close(stack.q[0], qr)
+        close(stack.k[0], kr)
+        close(stack.v[0], vr)
+        close(stack.mlp_normed[0], O.rmsnorm_ref(x, cpu["mlp"][l].float(), 1e-5))
+        close(final, O.rmsnorm_ref(x, cpu["final"].float(), 1e-5))
+        outs.append((stack.q[0].clone(), stack.k[0].clone(), stack.v[0].clone()))
+    for a, b in zip(*outs):
+        close(a, b.float().cpu())

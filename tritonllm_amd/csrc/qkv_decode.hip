@@ -217,8 +217,8 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 // row scale multiplies the finished sum.
 // EMB: the activation rows are gathered from an embedding table by token id (the first layer of a decode step:
 // model.py:906-920 feeds the gather straight into the first block's norm + QKV); the workgroup with blockIdx.x == 0
-// also writes the gathered rows out, as the residual stream. An id outside the table reads row 0 or vocab - 1 and
-// raises the flag.
+// also writes the gathered rows out, as the residual stream. An id outside the table gives a zero row (its loads are
+// clamped to a real row and the values discarded) and raises the flag, as the stand-alone gather does.
 template <int XR, int CH, int NORM, bool W8, bool EMB = false>
 __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   static_assert(!EMB || NORM != 0, "the fused gather exists with the fused norm only");
@@ -287,6 +287,7 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   if constexpr (NORM == 2) sc16 = reinterpret_cast<const bf16x8*>(a.norm_scale)[wave * (SPW * 4) + (lane < SPW * 4 ? lane : SPW * 4 - 1)];
   // EMB: where each of this lane's activation rows starts in the table (one id per load slot, fetched first)
   const bf16x8* xsrc[XL];
+  bool xok[XL];
   if constexpr (EMB) {
     int64_t id[XL];
 #pragma unroll
@@ -301,6 +302,7 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 #pragma unroll
     for (int i = 0; i < XL; ++i) {
       const bool ok = id[i] >= 0 && id[i] < a.emb_vocab;
+      xok[i] = ok;
       if (!ok && a.emb_oob) *a.emb_oob = 1;
       const int64_t idc = id[i] < 0 ? 0 : (id[i] < a.emb_vocab ? id[i] : a.emb_vocab - 1);
       xsrc[i] = reinterpret_cast<const bf16x8*>(a.emb_table) + idc * KV + wave * (SPW * 4);
@@ -374,6 +376,15 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
   if constexpr (NORM != 0) {
     float* tmp = reinterpret_cast<float*>(lds + wave * PATCH);
     float* wscale = tmp + NCH * XR * CPR;
+    if constexpr (EMB) {                      // an id outside the table stands for a zero row (the load itself read a real one)
+#pragma unroll
+      for (int c = 0; c < NCH * XL; ++c) {
+        if (!xok[c % XL]) {
+#pragma unroll
+          for (int q = 0; q < 8; ++q) xr[c][q] = static_cast<bf16>(0.f);
+        }
+      }
+    }
     if constexpr (NORM == 1) {
       if (lane < SPW * 8) reinterpret_cast<f32x4*>(wscale)[lane] = sc32;
     } else {

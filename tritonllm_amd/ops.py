@@ -47,13 +47,31 @@ def _on_gpu(*tensors: torch.Tensor) -> None:
             raise RuntimeError("tritonllm_amd ops run on the GPU only (got a CPU tensor); there is no CPU fallback")
 
 
+def _overlaps(a: torch.Tensor, b: torch.Tensor) -> bool:
+    a0, b0 = a.data_ptr(), b.data_ptr()
+    return a0 < b0 + b.numel() * b.element_size() and b0 < a0 + a.numel() * a.element_size()
+
+
+def _pooled_output(shape: tuple, dtype, device, *inputs) -> torch.Tensor:
+    """A scratch-pool buffer for an output the kernel writes while other workgroups still read ``inputs``. The pool
+    hands out one buffer per (shape, dtype, device), so an input that is itself a borrowed pool buffer of the same
+    shape (the normalised activations, when hidden == n_q_heads * head_dim) would be that very memory: then the
+    output is a fresh tensor instead."""
+    buf = scratch_pool.get(shape, dtype, device)
+    for t in inputs:
+        if t is not None and t.numel() and buf.numel() and _overlaps(buf, t):
+            return torch.empty(shape, dtype=dtype, device=device)
+    return buf
+
+
 def _yarn_of(t) -> YarnParams | None:
     return getattr(t, "_tllm_yarn", None)
 
 
-def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, keep: list) -> TllmRope:
+def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, keep: list, rows: int) -> TllmRope:
     """Fill the C descriptor of where the rotary angles come from. ``keep`` collects
-    objects that must stay alive until the launch call has returned."""
+    objects that must stay alive until the launch call has returned. ``rows`` is the number of rows the kernel
+    will rotate: it reads ``positions[row]`` for each of them, and only the host can check that they exist."""
     r = TllmRope()
     if yarn is None and cos is not None:
         yarn = _yarn_of(cos)
@@ -77,10 +95,11 @@ def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, kee
         r.sin_table = sin.data_ptr()
         r.table_row_stride = cos.stride(0)
     if positions is not None:
-        assert positions.dtype == torch.int64 and positions.is_contiguous()
+        assert positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous()
+        assert positions.numel() == rows, f"positions holds {positions.numel()} entries for {rows} rows"
         r.positions = positions.data_ptr()
     if offset is not None:
-        assert offset.dtype == torch.int64 and offset.numel() == 1
+        assert offset.is_cuda and offset.dtype == torch.int64 and offset.numel() == 1
         r.offset = offset.data_ptr()
     r.tokens_per_batch = int(tokens_per_batch)
     r.max_ctx = int(max_ctx)
@@ -215,7 +234,7 @@ def rope_forward(query: torch.Tensor, key: torch.Tensor, sin: torch.Tensor | Non
     assert query.dtype == _BF16 and key.dtype == _BF16
     assert query.is_contiguous() and key.is_contiguous(), "rope_forward rotates in place and needs dense q/k"
     keep: list = []
-    desc = _rope_desc(cos, sin, yarn, positions, offset, num_tokens, max_context_length, keep)
+    desc = _rope_desc(cos, sin, yarn, positions, offset, num_tokens, max_context_length, keep, batch_size * num_tokens)
     rc = lib().tllm_rope_bf16(query.data_ptr(), key.data_ptr(), batch_size * num_tokens, num_heads, num_key_value_heads, head_dim,
                               C.byref(desc), _stream())
     check(rc, "rope_forward")
@@ -320,8 +339,9 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     x, weight, bias = _prep_linear(x, weight, bias)
     q_dim, kv_dim = num_q_heads * head_dim, num_kv_heads * head_dim
     if out is None:
-        q = scratch_pool.get((rows, q_dim), x.dtype, x.device)
-        kv = scratch_pool.get((2, rows, kv_dim), x.dtype, x.device)   # k and v share a shape: one buffer, two halves
+        # keyed by the 3-D shape the reference's pool uses for q (triton_kernels.py:1196-1199), never a [rows, hidden] key
+        q = _pooled_output((rows, num_q_heads, head_dim), x.dtype, x.device, x).view(rows, q_dim)
+        kv = _pooled_output((2, rows, kv_dim), x.dtype, x.device, x)   # k and v share a shape: one buffer, two halves
         k, v = kv[0], kv[1]
     else:
         q, k, v = out
@@ -331,7 +351,7 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     desc = None
     if rotate:
         desc = _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch if tokens_per_batch else max(rows, 1),
-                          max_context_length, keep)
+                          max_context_length, keep, rows)
     if mode == "auto":
         mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
     assert mode in ("decode", "prefill")
@@ -356,8 +376,8 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
     the gathered rows (bit-exact; the residual stream), q / k / v as ``qkv_rope_forward(x, ..., norm_scale=...)`` gives them.
 
     Up to 16 ids at the gpt-oss shape this is ONE launch (the gather rides in the QKV kernel's activation loads);
-    otherwise it is the gather followed by ``qkv_rope_forward``. In the single launch an id outside the table reads
-    row 0 / vocab - 1 instead of producing a zero row; ``oob_flag`` is set either way."""
+    otherwise it is the gather followed by ``qkv_rope_forward``. Either way an id outside the table produces a zero
+    row of ``x`` (and the q / k / v that follow from it) and sets ``oob_flag``."""
     _on_gpu(ids, table, norm_scale, weight, bias, positions, offset, cos, sin, weight_scale, x_out, oob_flag)
     assert ids.ndim == 1 and ids.dtype in (torch.int32, torch.int64)
     assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
@@ -386,8 +406,8 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
     w_scale = None if weight_scale is None else _prep_weight_scale(weight, weight_scale)
     q_dim, kv_dim = num_q_heads * head_dim, num_kv_heads * head_dim
     if out is None:
-        q = scratch_pool.get((rows, q_dim), _BF16, table.device)
-        kv = scratch_pool.get((2, rows, kv_dim), _BF16, table.device)
+        q = _pooled_output((rows, num_q_heads, head_dim), _BF16, table.device, x_out).view(rows, q_dim)
+        kv = _pooled_output((2, rows, kv_dim), _BF16, table.device, x_out)
         k, v = kv[0], kv[1]
     else:
         q, k, v = out
@@ -396,7 +416,7 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
     keep: list = []
     desc = None
     if rotate:
-        desc = _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch if tokens_per_batch else rows, max_context_length, keep)
+        desc = _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch if tokens_per_batch else rows, max_context_length, keep, rows)
     ptr = lambda t: t.data_ptr() if t is not None else None
     rc = lib().tllm_embed_norm_qkv_rope_decode_bf16(
         ids.data_ptr(), int(ids.dtype == torch.int64), table.data_ptr(), vocab, x_out.data_ptr(), ptr(oob_flag), norm_scale.data_ptr(),
@@ -428,8 +448,8 @@ def qkv_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias: torch.T
     assert weight.dtype == _BF16
     x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
     hd = _split_head_dim(q_dim, kv_dim)
-    q = scratch_pool.get((batch, q_dim), hidden.dtype, hidden.device)
-    kv = scratch_pool.get((2, batch, kv_dim), hidden.dtype, hidden.device)
+    q = _pooled_output((batch, q_dim), hidden.dtype, hidden.device, x2)
+    kv = _pooled_output((2, batch, kv_dim), hidden.dtype, hidden.device, x2)
     k, v = kv[0], kv[1]
     _launch_qkv("decode", x2, weight, bias, q, k, v, q_dim, kv_dim, kv_dim, 0, q_dim // hd, kv_dim // hd, hd, None)
     return q[:, None, :], k[:, None, :], v[:, None, :]
@@ -461,9 +481,9 @@ def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_le
     assert cache_k.stride() == cache_v.stride()
     assert cache_k.stride(3) == 1 and cache_k.stride(2) == head_dim, "KV cache must be dense over (heads, head_dim)"
     x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
-    q = scratch_pool.get((batch, num_q_heads, head_dim), hidden.dtype, hidden.device)
+    q = _pooled_output((batch, num_q_heads, head_dim), hidden.dtype, hidden.device, x2)
     keep: list = []
-    desc = _rope_desc(cos, sin, yarn, positions, offset, 1, max_context_length, keep)
+    desc = _rope_desc(cos, sin, yarn, positions, offset, 1, max_context_length, keep, batch)
     _launch_qkv("decode", x2, weight, bias, q, cache_k, cache_v, num_q_heads * head_dim, cache_k.stride(0), cache_v.stride(0),
                 cache_k.stride(1), num_q_heads, num_kv_heads, head_dim, desc,
                 norm=None if norm_scale is None else (norm_scale, norm_eps),
