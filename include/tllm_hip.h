@@ -229,6 +229,18 @@ int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_sc
                                  int64_t workspace_bytes, int32_t* token_ids, int64_t rows, int64_t hidden,
                                  int64_t vocab, void* stream);
 
+/* The same greedy sampling for callers that cannot allocate device memory or hand over a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference, which takes
+ * its partial_max / partial_idx buffers from its scratch pool. The per-wavefront candidates pass through a
+ * 512 KiB device array owned by the library (one copy per GPU, held until the process ends), so rows is limited to
+ * tllm_unembedding_argmax_noalloc_max_rows() = 16; more rows return TLLM_E_SHAPE. The call allocates nothing and
+ * gives the same token_ids as tllm_unembedding_argmax_bf16. All calls on one GPU share the array: calls that may run
+ * concurrently on one GPU (different streams without ordering between them) race on it and must be serialised by the
+ * caller. Nothing in the array needs clearing between calls. */
+int64_t tllm_unembedding_argmax_noalloc_max_rows(void);
+int tllm_unembedding_argmax_noalloc_bf16(const void* x, const void* W, const float* w_scale, int32_t* token_ids,
+                                         int64_t rows, int64_t hidden, int64_t vocab, void* stream);
+
 /* Decode attention with learned sinks and an optional sliding window: one new token per batch row against the KV
  * cache; replaces attention_decode(q, k, v, sinks, sm_scale, bandwidth, start_q), attention_tt_decode.py:290-408
  * (kernels :9-287), whose definition is attention_ref.py:4-42:

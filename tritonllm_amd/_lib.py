@@ -52,6 +52,8 @@ SIGNATURES = {
     "tllm_unembedding_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "tllm_unembedding_argmax_workspace_bytes": (_i64, [_i64]),
     "tllm_unembedding_argmax_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
+    "tllm_unembedding_argmax_noalloc_max_rows": (_i64, []),
+    "tllm_unembedding_argmax_noalloc_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "tllm_attention_decode_splits": (_i32, [_i64, _i32, _i64, _i32]),
     "tllm_attention_decode_heads_per_workgroup": (_i32, [_i64, _i32, _i64, _i32]),
     "tllm_attention_decode_workspace_bytes": (_i64, [_i64, _i32, _i32, _i64, _i32]),

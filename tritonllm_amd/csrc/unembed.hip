@@ -22,6 +22,8 @@
 //
 // W8: fp8 (OCP e4m3) weight with one fp32 scale per vocabulary row (triton_kernels.py:261-268): widened to bf16
 // on the way into the patch, the row scale multiplies the finished sum. Half the bytes.
+#include <mutex>
+
 #include "common.h"
 
 namespace tllm {
@@ -331,15 +333,11 @@ extern "C" int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows) {
   return chunks * kUnembedGrid * 16 * xr * 8;      // one (float, int) pair per wavefront (at most 16 per workgroup) and batch-row slot
 }
 
-extern "C" int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_scale, void* workspace, int64_t workspace_bytes,
-                                            int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
-  int rc = unembed_check("unembedding_argmax", x, W, w_scale != nullptr, rows, hidden, vocab);
-  if (rc != TLLM_OK || rows == 0) return rc;
-  const int64_t need = tllm_unembedding_argmax_workspace_bytes(rows);
-  TLLM_REQUIRE(token_ids != nullptr, TLLM_E_ARG, "unembedding_argmax: token_ids is NULL");
-  TLLM_REQUIRE(workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 4 == 0, TLLM_E_ARG,
-               "unembedding_argmax: workspace of %lld bytes needed (tllm_unembedding_argmax_workspace_bytes), got %lld", (long long)need,
-               (long long)workspace_bytes);
+// Both argmax entry points: the stream kernel leaves one candidate per wavefront and batch row in `workspace`, the
+// reduce kernel picks the winners. Every slot the reduce kernel reads is written by the stream kernel of the same
+// call, so the workspace needs no clearing.
+static int unembed_argmax_run(const char* who, const void* x, const void* W, const float* w_scale, void* workspace, int64_t need,
+                              int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
   const int xr = unembed_xr(rows);
   UnembedArgs a{};
   a.x = (const bf16*)x;
@@ -351,9 +349,75 @@ extern "C" int tllm_unembedding_argmax_bf16(const void* x, const void* W, const 
   a.hidden = (int)hidden;
   a.vocab = (int)vocab;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  rc = unembed_launch<true>("unembedding_argmax", a, w_scale != nullptr, st);
+  int rc = unembed_launch<true>(who, a, w_scale != nullptr, st);
   if (rc != TLLM_OK) return rc;
   hipLaunchKernelGGL(unembed_argmax_reduce_kernel, dim3((unsigned)rows), dim3(256), 0, st, a.part_max, a.part_idx, token_ids,
                      kUnembedGrid * unembed_nw(xr, w_scale != nullptr), xr);
-  return check_launch("unembedding_argmax(reduce)");
+  return check_launch(who);
+}
+
+extern "C" int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_scale, void* workspace, int64_t workspace_bytes,
+                                            int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
+  int rc = unembed_check("unembedding_argmax", x, W, w_scale != nullptr, rows, hidden, vocab);
+  if (rc != TLLM_OK || rows == 0) return rc;
+  const int64_t need = tllm_unembedding_argmax_workspace_bytes(rows);
+  TLLM_REQUIRE(token_ids != nullptr, TLLM_E_ARG, "unembedding_argmax: token_ids is NULL");
+  TLLM_REQUIRE(workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 4 == 0, TLLM_E_ARG,
+               "unembedding_argmax: workspace of %lld bytes needed (tllm_unembedding_argmax_workspace_bytes), got %lld", (long long)need,
+               (long long)workspace_bytes);
+  return unembed_argmax_run("unembedding_argmax", x, W, w_scale, workspace, need, token_ids, rows, hidden, vocab, stream);
+}
+
+// ---- the allocation-free form -----------------------------------------------------------------------------------
+// The candidates travel through a buffer the library owns: a file-scope device array, present on every GPU the code
+// object is loaded on from then until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress; the kernels get the device address that call returns, looked up once per device.
+namespace {
+constexpr int kNoAllocMaxRows = 16;
+constexpr int64_t kNoAllocScratchBytes = static_cast<int64_t>(kUnembedGrid) * 16 * kNoAllocMaxRows * 8;   // 512 KiB
+constexpr int kMaxDevices = 64;
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int noalloc_scratch(const char* who, void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  TLLM_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, TLLM_E_LAUNCH, "%s: hipGetDevice: %s (device %d)", who,
+               hipGetErrorString(e), dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    TLLM_REQUIRE(e == hipSuccess && p != nullptr, TLLM_E_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", who, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return TLLM_OK;
+}
+}  // namespace
+
+extern "C" int64_t tllm_unembedding_argmax_noalloc_max_rows(void) { return kNoAllocMaxRows; }
+
+extern "C" int tllm_unembedding_argmax_noalloc_bf16(const void* x, const void* W, const float* w_scale, int32_t* token_ids, int64_t rows,
+                                                    int64_t hidden, int64_t vocab, void* stream) {
+  TLLM_REQUIRE(rows <= kNoAllocMaxRows, TLLM_E_SHAPE,
+               "unembedding_argmax_noalloc: at most %d rows (got %lld): the library-owned scratch holds the candidates of %d batch rows; "
+               "use tllm_unembedding_argmax_bf16 with a workspace for more",
+               kNoAllocMaxRows, (long long)rows, kNoAllocMaxRows);
+  int rc = unembed_check("unembedding_argmax_noalloc", x, W, w_scale != nullptr, rows, hidden, vocab);
+  if (rc != TLLM_OK || rows == 0) return rc;
+  TLLM_REQUIRE(token_ids != nullptr, TLLM_E_ARG, "unembedding_argmax_noalloc: token_ids is NULL");
+  const int64_t need = tllm_unembedding_argmax_workspace_bytes(rows);
+  TLLM_REQUIRE(need <= kNoAllocScratchBytes, TLLM_E_SHAPE, "unembedding_argmax_noalloc: %lld bytes of candidates exceed the scratch",
+               (long long)need);
+  void* ws = nullptr;
+  rc = noalloc_scratch("unembedding_argmax_noalloc", &ws);
+  if (rc != TLLM_OK) return rc;
+  return unembed_argmax_run("unembedding_argmax_noalloc", x, W, w_scale, ws, need, token_ids, rows, hidden, vocab, stream);
 }

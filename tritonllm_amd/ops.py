@@ -593,6 +593,21 @@ def unembedding_decode_argmax_forward(hidden: torch.Tensor, weight: torch.Tensor
     return ids
 
 
+def unembedding_decode_argmax_noalloc(hidden: torch.Tensor, weight: torch.Tensor, token_ids: torch.Tensor,
+                                      weight_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """``unembedding_decode_argmax_forward`` for callers that must not allocate: the caller passes ``token_ids``
+    (int32 ``[B]``), the candidates go through a device array the library owns, and nothing is taken from the scratch
+    pool or from PyTorch's allocator. At most ``tllm_unembedding_argmax_noalloc_max_rows()`` (16) batch rows. Calls on
+    one GPU share that array: do not overlap them on different streams. No counterpart in the reference."""
+    x2, weight, ws, batch, hidden_size, vocab_size = _unembed_prep(hidden, weight, weight_scale)
+    _on_gpu(token_ids)
+    assert token_ids.dtype == torch.int32 and token_ids.shape == (batch,) and token_ids.is_contiguous()
+    rc = lib().tllm_unembedding_argmax_noalloc_bf16(x2.data_ptr(), weight.data_ptr(), ws.data_ptr() if ws is not None else None,
+                                                    token_ids.data_ptr(), batch, hidden_size, vocab_size, _stream())
+    check(rc, "unembedding_decode_argmax_noalloc")
+    return token_ids
+
+
 def unembedding_forward(hidden: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """triton_kernels.py:515-525: the stream kernel for one bf16 token per batch row on the GPU, the library GEMM otherwise."""
     if hidden.is_cuda and hidden.ndim == 3 and hidden.shape[1] == 1 and hidden.dtype == _BF16 and weight.dtype == _BF16:
