@@ -51,6 +51,8 @@ def algorithmic_bytes():
         "embedding": lambda t: t * (2 * HIDDEN * 2 + 4),
         "swiglu": lambda m: m * (2 * HIDDEN * 2 + HIDDEN * 2),
         "mxfp4": lambda blocks: blocks * (16 + 1 + 64),
+        # stand-alone rotary: q [R, 4096] and k [R, 512] read and written in place
+        "rope": lambda r: 2 * r * (NQ + NKV) * HD * 2,
         "qkv": lambda r: w + QKV_DIM * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
         "norm_qkv": lambda r: w + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
         # fp8 weight: one byte per element + one fp32 scale per output row
@@ -64,6 +66,46 @@ def algorithmic_bytes():
         "unembed_w8": lambda r: VOCAB_BENCH * HIDDEN + VOCAB_BENCH * 4 + r * (HIDDEN * 2 + VOCAB_BENCH * 2),
         "norm_qkv_w8": lambda r: w // 2 + QKV_DIM * 4 + QKV_DIM * 2 + HIDDEN * 2 + r * (HIDDEN * 2 + QKV_DIM * 2),
     }
+
+
+def host_cpu_info() -> dict:
+    """CPU model and core counts of the host, and how many threads the CPU-baseline leg uses: every physical core this
+    process may run on, capped by OMP_NUM_THREADS when the environment sets it (a shared box grants a share of its cores)."""
+    model, cores, logical = "unknown", set(), 0
+    try:
+        phys = core = None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                key, _, val = line.partition(":")
+                key, val = key.strip(), val.strip()
+                if key == "model name" and model == "unknown":
+                    model = val
+                elif key == "processor":
+                    logical += 1
+                elif key == "physical id":
+                    phys = val
+                elif key == "core id":
+                    core = val
+                elif not key and phys is not None and core is not None:
+                    cores.add((phys, core))
+                    phys = core = None
+        if phys is not None and core is not None:
+            cores.add((phys, core))
+    except OSError:
+        pass
+    logical = logical or (os.cpu_count() or 1)
+    physical = len(cores) or logical
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        usable = logical
+    threads = min(physical, usable)
+    note = "all physical cores this process may run on"
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    if cap.isdigit() and 0 < int(cap) < threads:
+        threads = int(cap)
+        note = f"capped by OMP_NUM_THREADS={cap} (the box's CPU share) of {physical} physical cores"
+    return {"model": model, "physical": physical, "logical": logical, "usable": usable, "threads_used": max(threads, 1), "note": note}
 
 
 def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg) -> int:
@@ -145,6 +187,12 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         fn = lambda i: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart, kv_len_hint=hint)
         keys = min(ctx, 128) if win else ctx
         nbytes = n * NKV * keys * HD * 2 * 2 + n * NQ * HD * 2 * 2
+    elif kind == "rope":
+        rq = torch.empty(1, n, NQ, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        rk = torch.empty(1, n, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        roff = torch.zeros(1, dtype=torch.int64, device=dev)
+        fn = lambda i: T.rope_forward(rq, rk, None, None, 131072, roff, yarn=yarn)
+        nbytes = bytes_of["rope"](n)
     elif kind == "rmsnorm":
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         to = torch.empty_like(xp)
@@ -191,13 +239,14 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--samples", type=int, default=31, help="how often the --steps steps are timed; the median sample is reported")
     ap.add_argument("--fuse-gather", action="store_true",
                     help="the step's embedding gather rides in the QKV kernel too (2 launches per step instead of 3)")
     ap.add_argument("--unfused", action="store_true",
                     help="run RMSNorm as its own launch in front of the QKV kernel (default: normalised inside the QKV decode kernel)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="seconds of CPU work per CPU-baseline leg (all cores, one thread)")
     ap.add_argument("--only", default=None,
                     help="run just one entry of the kernel table (e.g. qkv_rope_prefill_T2048) and print its row; for profiling")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -213,6 +262,7 @@ def main() -> int:
 
     import tritonllm_amd as T
     from tritonllm_amd import _lib
+    from tritonllm_amd.stack import LayerKernelStack
 
     if not os.path.exists(_lib.LIB_PATH):
         from tritonllm_amd.build import build_library
@@ -279,15 +329,24 @@ def main() -> int:
         return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg)
 
     # ---------------------------------------------------------------- the timed job
+    # One sample = EXACTLY --steps steps, captured as one HIP graph and timed with HIP events between two
+    # synchronisations. The sample is repeated (>= 25 times) and the median reported. A graph's weight pointers are
+    # fixed, so there is one graph per starting layer: sample s starts at layer (s * steps) % 24, i.e. where the
+    # previous sample stopped, and all 24 weight sets keep rotating whatever --steps is.
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    job = graph_of(step, args.steps)
-    job.replay()                                   # one untimed replay: graph upload / first-touch
+    n_samples = max(args.samples, 1)
+    starts = sorted({(s * args.steps) % N_LAYERS for s in range(n_samples)})
+    jobs = {st: graph_of(lambda i, st=st: step(st + i), args.steps) for st in starts}
+    for gr in jobs.values():
+        gr.replay()                                # one untimed replay each: graph upload / first-touch
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    elapsed = time_graph(job)
+    samples = [time_graph(jobs[(s * args.steps) % N_LAYERS]) for s in range(n_samples)]
     wall = time.perf_counter() - t0
+    samples.sort()
+    elapsed = samples[len(samples) // 2]           # median sample: seconds for --steps steps
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = B * args.steps / elapsed
 
@@ -434,6 +493,11 @@ def main() -> int:
         uw8, uws = T.quantize_fp8_rows(table)
         bench_kernel("unembedding_decode_w8_B8", lambda i, ux=ux: T.unembedding_decode_forward(ux, uw8, uws), bytes_of["unembed_w8"](8), n=10)
         del uw8, uws
+        # stand-alone rotary at the decode size (one token per batch row, independent positions)
+        rope_off = torch.zeros(1, dtype=torch.int64, device=dev)
+        bench_kernel("rope_B8", lambda i: T.rope_forward(q.view(B, 1, NQ, HD), k.view(B, 1, NKV, HD), None, None, 131072, None, yarn=yarn,
+                                                         positions=positions),
+                     bytes_of["rope"](B))
         # prefill sizes
         for tt in (2048, 8192):
             xp = torch.empty(tt, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
@@ -447,6 +511,10 @@ def main() -> int:
                          flops=2.0 * tt * HIDDEN * QKV_DIM, n=48)
             bench_kernel(f"rmsnorm_T{tt}", lambda i, xp=xp, to=to: T.rmsnorm_forward(xp, scales[i % N_LAYERS], 1e-5, out=to),
                          bytes_of["rmsnorm"](tt), n=96)
+            # stand-alone rotary (the reference's prefill path, model.py:521-522): q and k rotated in place
+            bench_kernel(f"rope_T{tt}", lambda i, qo=qo, tt=tt: T.rope_forward(qo[0].view(1, tt, NQ, HD), qo[1].view(1, tt, NKV, HD), None, None,
+                                                                              131072, rope_off, yarn=yarn),
+                         bytes_of["rope"](tt), n=96)
             del xp, qo, to
             # prefill attention over the projection's output, q / k / v read in place as column ranges of [1, T, 5120]
             pq = [torch.empty(1, tt, QKV_DIM, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(2)]
@@ -483,30 +551,15 @@ def main() -> int:
         for r in (1, 8, 32):
             xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
             pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
-            qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),
-                  torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev))
-            tr = torch.empty_like(xr)
             sx = (2.0 * torch.randn(4 * r, 2 * HIDDEN, generator=g)).bfloat16().to(dev)
-            so = torch.empty(4 * r, HIDDEN, dtype=torch.bfloat16, device=dev)
-
-            def token_step(_i, xr=xr, pr=pr, qo=qo, tr=tr, sx=sx, so=so):
-                for l in range(N_LAYERS):
-                    if args.unfused:
-                        T.rmsnorm_forward(xr, scales[l], 1e-5, out=tr)
-                        T.qkv_rope_forward(tr, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=pr, mode="decode", out=qo)
-                    else:
-                        T.qkv_rope_forward(xr, weights[l], biases[l], NQ, NKV, HD, yarn=yarn, positions=pr, mode="decode", out=qo,
-                                           norm_scale=scales[l], norm_eps=1e-5)
-                    T.rmsnorm_forward(xr, mlp_scales[l], 1e-5, out=tr)
-                    T.swiglu(sx, out=so)
-                T.rmsnorm_forward(xr, mlp_scales[N_LAYERS], 1e-5, out=tr)
-
+            # the same object the parity test drives (tests/test_gpu_parity.py::test_layer_stack24_token_step)
+            st = LayerKernelStack(weights, biases, scales, mlp_scales[:N_LAYERS], mlp_scales[N_LAYERS], yarn, r, fuse_norm=not args.unfused)
+            token_step = lambda _i, st=st, xr=xr, pr=pr, sx=sx: st.token_step(xr, pr, sx)
             token_step(0)
             gr = graph_of(token_step, 4)
             gr.replay()
             sec = min(time_graph(gr) for _ in range(5)) / 4
-            launches = N_LAYERS * (4 if args.unfused else 3) + 1
-            stack[f"B{r}"] = {"us_per_token_step": round(sec * 1e6, 2), "tokens/s": round(r / sec, 1), "launches": launches,
+            stack[f"B{r}"] = {"us_per_token_step": round(sec * 1e6, 2), "tokens/s": round(r / sec, 1), "launches": st.launches_per_step(),
                               "weight_GB/s": round(N_LAYERS * QKV_DIM * HIDDEN * 2 / sec / 1e9, 1)}
 
     # ---------------------------------------------------------------- attention blocks of a 24-layer decode step
@@ -602,36 +655,55 @@ def main() -> int:
             del xp, tn, qb, ck, cv
 
     # ---------------------------------------------------------------- CPU baseline (reported only)
+    # The oracle's eager-bf16 PyTorch twin of the reference chain on the host cores: the same B = 8 step, the same 24
+    # rotating weight sets (708 MB, beyond the host's caches), timed with perf_counter on all the cores this process may
+    # use and on one thread (timing convention of the reference's examples/bench_moe.py:53-77: warm-up, then a timed loop).
     cpu_baseline = None
     if not args.no_cpu_baseline:
         from oracle import layers as O
 
-        cores = min(os.cpu_count() or 1, 16)
-        torch.set_num_threads(cores)
-        cx, cw, cb, cs = x.cpu(), weights[0].cpu(), biases[0].cpu(), scales[0].cpu()
-        cids, cpos, csw = ids.cpu().long(), positions.cpu(), swiglu_x.cpu()
+        host = host_cpu_info()
+        cw, cb, cs = [w.cpu() for w in weights], [b_.cpu() for b_ in biases], [s_.cpu() for s_ in scales]
+        cx, cids, cpos, csw = x.cpu(), ids.cpu().long(), positions.cpu(), swiglu_x.cpu()
         ctable = table[:65536].cpu()                      # the gather touches 8 rows; a 377 MB slice keeps host memory modest
         cids = cids % 65536
         cos_t, sin_t = O.yarn_cos_sin(torch.arange(8192))
 
-        def cpu_step():
+        def cpu_step(i):
+            l = i % N_LAYERS
             O.embedding_eager(ctable, cids)
-            tt = O.rmsnorm_eager(cx, cs)
-            O.qkv_rope_eager(tt, cw, cb, cos_t, sin_t, cpos)
+            tt = O.rmsnorm_eager(cx, cs[l])
+            O.qkv_rope_eager(tt, cw[l], cb[l], cos_t, sin_t, cpos)
             O.swiglu_eager(csw)
 
-        for _ in range(3):
-            cpu_step()
-        n_cpu, t_start = 0, time.perf_counter()
-        while True:
-            cpu_step()
-            n_cpu += 1
-            dt = time.perf_counter() - t_start
-            if dt > args.cpu_seconds:
-                break
+        def time_cpu(threads, seconds):
+            torch.set_num_threads(threads)
+            for i in range(3):
+                cpu_step(i)
+            per_step, n, t_start = [], 0, time.perf_counter()
+            while True:
+                t1 = time.perf_counter()
+                cpu_step(n)
+                t2 = time.perf_counter()
+                per_step.append(t2 - t1)
+                n += 1
+                if t2 - t_start > seconds and n >= 10:
+                    break
+            per_step.sort()
+            med = per_step[len(per_step) // 2]
+            return {"tokens/s": round(B / med, 1), "ms_per_step_median": round(med * 1e3, 3), "steps": n, "threads": threads,
+                    "weight_GB/s": round(QKV_DIM * HIDDEN * 2 / med / 1e9, 2), "seconds": round(t2 - t_start, 1)}
+
+        many = time_cpu(host["threads_used"], args.cpu_seconds)
+        one = time_cpu(1, args.cpu_seconds)
+        torch.set_num_threads(host["threads_used"])
         cpu_baseline = {
-            "value": round(B * n_cpu / dt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{n_cpu} steps of the same B=8 step (eager bf16 PyTorch restatement of the reference chain, one weight set) in {dt:.1f} s",
+            "value": many["tokens/s"], "unit": "tokens/s", "cores": host["threads_used"], "kind": "port",
+            "sample": f"{many['steps']} steps of the same B=8 step in {many['seconds']} s (eager bf16 PyTorch restatement of the reference chain, "
+                      f"24 rotating weight sets, median step), then {one['steps']} steps on one thread in {one['seconds']} s",
+            "cpu_model": host["model"], "cores_physical": host["physical"], "cores_logical": host["logical"],
+            "cores_usable": host["usable"], "threads_note": host["note"],
+            "all_cores": many, "single_thread": one,
         }
 
     out = {
@@ -645,7 +717,8 @@ def main() -> int:
                    "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel",
                    "gather": "inside the QKV decode kernel (x = table rows)" if args.fuse_gather else "own launch (x ~ N(0,1) as the configuration states)"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "prefill_chains": prefill_chains, "attention_blocks24": attn_stack,
-        "wall_s_timed_region": round(wall, 4),
+        "samples": n_samples, "sample_ms_min_median_max": [round(samples[0] * 1e3, 4), round(elapsed * 1e3, 4), round(samples[-1] * 1e3, 4)],
+        "wall_s_all_samples": round(wall, 4),
     }
     print(json.dumps(out))
     return 0
