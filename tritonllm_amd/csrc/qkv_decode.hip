@@ -4,9 +4,10 @@
 // kernels are HBM-bound. All of them use the matrix core with the weight rows on the M side and
 // the activation rows on the N side -- the MFMA does the K reduction across lanes for free and
 // leaves the VALU to the rotary epilogue -- and keep a rotation pair (row d and row d+32 of a
-// head) inside one workgroup so the rotation needs no second pass. Three kernels:
-//   qkv_decode_cu_kernel   hidden == 2880 (gpt-oss): one workgroup per CU, coalesced loads,
-//                          LDS-transposed operands. The fast path; see its comment.
+// head) inside one workgroup so the rotation needs no second pass. The kernels:
+//   qkv_decode_r8_kernel   hidden == 2880 (gpt-oss), up to 8 rows, bf16 weight: qkv_decode_r8.hip, the fastest.
+//   qkv_decode_cu_kernel   hidden == 2880, 9 rows and more, or an fp8 weight: one workgroup per CU, coalesced
+//                          loads, LDS-transposed operands; see its comment.
 //   qkv_decode_kernel      head_dim == 64, hidden % 32 == 0: operands loaded straight into MFMA
 //                          layout (simple, ~1.8x slower: every lane is its own cache-line request).
 //   qkv_generic_kernel     anything else: shuffle-reduced dot products.
@@ -624,7 +625,9 @@ static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, 
   const int64_t chunks = (rows + xr - 1) / xr;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
   const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
-  if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
+  const bool fits32 = (a.emb_ids ? a.emb_vocab : rows) * 5760 < (1ll << 32);   // the kernel addresses activation rows with 32-bit byte offsets
+  if (xr == 8 && !w8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, grid, st, a, ra, fr);
+  else if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
   else launch_cu(xr, norm, w8, grid, st, a, ra, fr);
   return check_launch(what);
 }

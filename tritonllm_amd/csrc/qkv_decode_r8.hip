@@ -1,0 +1,429 @@
+// Decode-size fused (RMSNorm +) QKV projection + bias + rotary for hidden == 2880 and up to 8 activation rows per
+// workgroup: the weight-streaming kernel of the gpt-oss decode step (B <= 8).
+//
+// Work per CU. The 2560 rotation pairs are dealt ten at a time to 256 workgroups, each needing most of a CU's LDS, so
+// exactly one lands on every CU and every CU streams 1/256 of the weight: 20 rows of 5760 bytes. The rows form two
+// 16-row MFMA tiles (v_mfma_f32_16x16x32_bf16: weight rows on M, activation rows on N): tile 0 = pairs 0..5, tile 1 =
+// pairs 6..9, two adjacent pairs (2i, 2i+1) occupying four tile rows [lo(2i), lo(2i+1), hi(2i), hi(2i+1)], so that one
+// lane ends up with both halves of two adjacent rotation pairs.
+//
+// What was measured on the machine and what the kernel does about it:
+//   * A CU returns vector loads in the order it took them, across wavefronts, and takes only so many at a time. A
+//     barrier that waits for staged activations therefore waits for every weight load queued ahead of them. Here no
+//     wavefront ever waits for another one's loads: each of the six streaming wavefronts owns one K slice of 480
+//     (fifteen k32 steps) and brings in its own slice of the activations, then its slice of the 20 weight rows.
+//   * Passing the stream through registers and ds_write into operand layout costs as much time as the stream
+//     itself (loads, LDS writes and LDS reads all cross the same register-file port). Here everything goes from
+//     global memory straight into LDS (global_load_lds_dwordx4: a wavefront's 64 x 16 bytes land at consecutive LDS
+//     addresses; which global chunk a lane fetches is free, and that freedom carries the XOR swizzle that makes the
+//     fragment reads conflict-free) and is read back once, as MFMA fragments.
+//   * The weight slice of a wavefront arrives in four phases (4 + 4 + 4 + 3 k32 steps) through a ring of three
+//     5 KB regions; a phase is multiplied as soon as it has landed, so three steps remain when the stream ends.
+//   * The six partial tiles meet in LDS; two further wavefronts (one per tile), which loaded position, bias and
+//     scales and computed cos/sin while the stream ran, add them in a fixed order, add the bias, rotate, round once
+//     and store two adjacent dims at a time.
+// The loads of the streaming wavefronts are inline asm (the compiler cannot express "to LDS"), so their
+// s_waitcnt vmcnt are spelled by hand; those wavefronts issue no other vector load once the first asm load is out.
+//
+// NORM: 0 = x is used as it is; 1 / 2 = x is first RMS-normalised with an fp32 / bf16 scale: the wavefronts sum the
+// squares of their slices from the fragments, exchange them (one barrier) and scale the fragments in registers --
+// fp32 arithmetic, one rounding to bf16: the operand the separate rmsnorm launch would hand over.
+// EMB: the activation rows are gathered from an embedding table by token id (model.py:906-920 feeding the first
+// block); workgroup 0 also writes the gathered rows out. An id outside the table gives a zero row and raises the flag.
+#include "qkv_common.h"
+
+namespace tllm {
+
+namespace r8 {
+constexpr int XR = 8;             // activation rows per workgroup
+constexpr int NS = 6;             // streaming wavefronts = K slices
+constexpr int NE = 2;             // epilogue wavefronts = tiles
+constexpr int STEPS = 15;         // k32 steps per slice
+constexpr int PAIRS = 10;         // rotation pairs per workgroup
+constexpr int RING = 3;           // resident phases per wavefront
+constexpr int REGION = 20 * 256;  // one phase: 20 weight rows x four k32 steps
+constexpr int XBLOCK = 1024;      // one activation row of a slice: 60 chunks of 16 bytes (+ 4 spare)
+}  // namespace r8
+
+#ifdef TLLM_R8_STAMPS
+__device__ unsigned long long g_r8_stamps[256 * 8 * 8];
+#define R8_STAMP(i) do { if (lane == 0 && blockIdx.y == 0 && blockIdx.x < 256) g_r8_stamps[(blockIdx.x * 8 + wave) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define R8_STAMP(i) do { } while (0)
+#endif
+
+template <int NORM, bool EMB>
+__global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int out4) {
+  using namespace r8;
+  static_assert(!EMB || NORM != 0, "the fused gather exists with the fused norm only");
+  __shared__ __align__(1024) unsigned char xw[NS * XR * XBLOCK];
+  __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
+  __shared__ __align__(1024) unsigned char scw[NORM ? NS * 2048 : 16];
+  __shared__ float s_part[NORM ? NS * XR : 1];
+  __shared__ unsigned s_flag[NORM ? NS : 1];              // s_part[w][*] of streaming wavefront w is complete
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int total_pairs = (a.n_q_heads + 2 * a.n_kv_heads) * 32;
+  const int pair0 = blockIdx.x * PAIRS;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
+  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+  R8_STAMP(0);
+
+  if (wave >= NS) {
+    // ======================================================================= epilogue wavefront of tile `tile`
+    const int tile = wave - NS;
+    // the streaming wavefronts' rendezvous between their activation and weight loads (it also publishes their
+    // cleared flags): met here at once, before this wavefront has anything to wait for
+    if constexpr (NORM != 0) __syncthreads();
+    const int en = lane & 15, eg = lane >> 4;               // activation row, quad of the tile
+    const int epair = pair0 + (tile ? 6 : 0) + 2 * eg;      // even; its neighbour epair + 1 shares head and quad
+    const bool evalid = eg < (tile ? 2 : 3) && epair < total_pairs && en < nvalid;
+    const int egp = evalid ? epair : 0;
+    const int ehead = egp >> 5, ed = egp & 31;
+    const int64_t erow = row0 + (evalid ? en : 0);
+    const bool erot = a.has_rope && ehead < a.n_q_heads + a.n_kv_heads;
+    const int64_t* pos_ptr = ra.positions ? ra.positions + erow : reinterpret_cast<const int64_t*>(a.W);
+    const int64_t* off_ptr = ra.offset ? ra.offset : reinterpret_cast<const int64_t*>(a.W);
+    const unsigned* bias_ptr = reinterpret_cast<const unsigned*>(a.bias ? a.bias : a.W);   // two bf16 per load; ed is even
+    const int64_t pos_ld = *pos_ptr;
+    const int64_t off_ld = *off_ptr;
+    const unsigned b_lo = bias_ptr[(ehead * 64 + ed) >> 1];
+    const unsigned b_hi = bias_ptr[(ehead * 64 + 32 + ed) >> 1];
+    const float freq0 = fr.v[ed], freq1 = fr.v[ed + 1];
+    float cs0 = 1.f, sn0 = 0.f, cs1 = 1.f, sn1 = 0.f;
+    const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
+    if (erot) {
+      int64_t pos = ra.positions ? pos_ld : (erow % ra.tokens_per_batch) + (ra.offset ? off_ld : 0);
+      pos = rope_wrap(pos, ra.max_ctx);
+      if (ra.use_yarn) {
+        yarn_cos_sin(pos, freq0, ra.concentration, &cs0, &sn0);
+        yarn_cos_sin(pos, freq1, ra.concentration, &cs1, &sn1);
+      } else {
+        rope_cos_sin(ra, fr, pos, ed, &cs0, &sn0);
+        rope_cos_sin(ra, fr, pos, ed + 1, &cs1, &sn1);
+      }
+    }
+    float bl0 = 0.f, bl1 = 0.f, bh0 = 0.f, bh1 = 0.f;
+    if (a.bias) {
+      bl0 = __uint_as_float(b_lo << 16);
+      bl1 = __uint_as_float(b_lo & 0xffff0000u);
+      bh0 = __uint_as_float(b_hi << 16);
+      bh1 = __uint_as_float(b_hi & 0xffff0000u);
+    }
+    bf16* out = qkv_out_ptr(a, slot, erow, ehead) + ed;
+    unsigned red_o = static_cast<unsigned>(REGION + tile * 1024 + lane * 16);
+    // One wavefront runs alone from the last barrier to the stores, so every instruction after that barrier is
+    // latency: all of the above is forced to exist here (left to itself the compiler moves it to its first use,
+    // behind the barrier).
+    asm volatile("" : "+v"(cs0), "+v"(sn0), "+v"(cs1), "+v"(sn1), "+v"(bl0), "+v"(bl1), "+v"(bh0), "+v"(bh1), "+v"(out), "+v"(red_o));
+    __syncthreads();                                        // partial tiles are in LDS
+    R8_STAMP(6);
+    f32x4 t[NS];
+#pragma unroll
+    for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(ring + w * (RING * REGION) + red_o);
+    f32x4 acc = t[0];
+#pragma unroll
+    for (int w = 1; w < NS; ++w) {                          // fixed order: the result does not depend on timing
+      acc[0] += t[w][0];
+      acc[1] += t[w][1];
+      acc[2] += t[w][2];
+      acc[3] += t[w][3];
+    }
+    if (!evalid) return;
+    float lo0 = acc[0] + bl0, lo1 = acc[1] + bl1, hi0 = acc[2] + bh0, hi1 = acc[3] + bh1;   // [lo(d), lo(d+1), hi(d), hi(d+1)] of row en
+    if (erot) {
+      const float r0 = lo0 * cs0 - hi0 * sn0, r2 = hi0 * cs0 + lo0 * sn0;
+      const float r1 = lo1 * cs1 - hi1 * sn1, r3 = hi1 * cs1 + lo1 * sn1;
+      lo0 = r0;
+      lo1 = r1;
+      hi0 = r2;
+      hi1 = r3;
+    }
+    bf16x2 plo, phi;
+    plo[0] = static_cast<bf16>(lo0);
+    plo[1] = static_cast<bf16>(lo1);
+    phi[0] = static_cast<bf16>(hi0);
+    phi[1] = static_cast<bf16>(hi1);
+    R8_STAMP(7);
+    if (out4) {
+      *reinterpret_cast<bf16x2*>(out) = plo;
+      *reinterpret_cast<bf16x2*>(out + 32) = phi;
+    } else {
+      out[0] = plo[0];
+      out[1] = plo[1];
+      out[32] = phi[0];
+      out[33] = phi[1];
+    }
+    return;
+  }
+
+  // ========================================================================= streaming wavefront of K slice `kq`
+  const int kq = wave;
+  const int m = lane & 15, g = lane >> 4, m1 = m & 7;
+  unsigned char* myx = xw + wave * (XR * XBLOCK);
+  unsigned char* myring = ring + wave * (RING * REGION);
+
+  // activations: row n of the slice -> 1 KB block n; lane i fetches chunk i ^ 2n (60 real chunks, the rest re-read
+  // chunk 59), the swizzle that spreads the eight rows of a fragment read over the banks
+  unsigned xoff[XR];
+  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(EMB ? a.emb_table : a.x);
+  bool xok_m1 = true;                                       // EMB: is the id of the row this lane's fragments belong to inside the table?
+  {
+    int64_t src_row[XR];
+#pragma unroll
+    for (int n = 0; n < XR; ++n) src_row[n] = row0 + (n < nvalid ? n : nvalid - 1);
+    if constexpr (EMB) {
+      int64_t id[XR];
+#pragma unroll
+      for (int n = 0; n < XR; ++n) {                        // all eight ids first: nothing between these loads that could order them
+        id[n] = a.emb_ids_i64 ? reinterpret_cast<const int64_t*>(a.emb_ids)[src_row[n]]
+                              : static_cast<int64_t>(reinterpret_cast<const int*>(a.emb_ids)[src_row[n]]);
+      }
+      bool any_bad = false;
+#pragma unroll
+      for (int n = 0; n < XR; ++n) {
+        const bool ok = id[n] >= 0 && id[n] < a.emb_vocab;
+        any_bad |= !ok;
+        if (n == m1) xok_m1 = ok;
+        src_row[n] = id[n] < 0 ? 0 : (id[n] < a.emb_vocab ? id[n] : a.emb_vocab - 1);
+      }
+      if (any_bad && a.emb_oob && lane == 0) *a.emb_oob = 1;
+    }
+#pragma unroll
+    for (int n = 0; n < XR; ++n) {
+      int c = lane ^ (2 * n);
+      c = c < 60 ? c : 59;
+      xoff[n] = static_cast<unsigned>(src_row[n] * 5760 + kq * 960 + c * 16);
+    }
+  }
+  // weight: lane -> (row r4 of a 4-row block, position pos): it fetches chunk pos ^ (tile row & 15) of that row
+  unsigned goff[5], goff3[5];                               // phases 0-2 / the three-step phase 3 (chunks 0..11 only)
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    const int row20 = 4 * j + (lane >> 4);                  // 0..11 tile 0, 12..19 tile 1
+    const int tile = row20 >= 12, trow = tile ? row20 - 12 : row20;
+    const int quad = trow >> 2, q = trow & 3;
+    int gp = pair0 + (tile ? 6 : 0) + 2 * quad + (q & 1);
+    gp = gp < total_pairs ? gp : total_pairs - 1;
+    const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + ((q & 2) ? 32u : 0u);
+    const int cc = (lane & 15) ^ (trow & 15);
+    goff[j] = wrow * 5760u + kq * 960u + cc * 16u;
+    goff3[j] = wrow * 5760u + kq * 960u + (cc < 12 ? cc : 11) * 16u;
+  }
+  const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
+  auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
+  // Phases 0..2 land in the wavefront's three ring regions, phase 3 in its activation blocks, which are free as soon
+  // as the activation fragments are in registers -- so no weight load ever waits for an MFMA.
+  auto phase_region = [&](int p) -> unsigned char* { return p < RING ? myring + p * REGION : myx; };
+  auto issue_phase = [&](int p) {
+    const unsigned char* sb = wbase + p * 256;
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const unsigned dst = lds_addr(phase_region(p) + j * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == 3 ? goff3[j] : goff[j]), "s"(sb) : "memory", "m0");
+    }
+  };
+
+  // ---- every load of this wavefront, oldest first: activations, norm scale, then the weight
+#pragma unroll
+  for (int n = 0; n < XR; ++n) {
+    const unsigned dst = lds_addr(myx + n * XBLOCK);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+  }
+  constexpr int NSC = NORM == 1 ? 2 : (NORM == 2 ? 1 : 0);   // scale loads: 480 fp32 = 120 chunks, 480 bf16 = 60 chunks
+  if constexpr (NORM != 0) {
+    const unsigned char* sbase = reinterpret_cast<const unsigned char*>(a.norm_scale) + kq * (NORM == 1 ? 1920 : 960);
+#pragma unroll
+    for (int t = 0; t < NSC; ++t) {
+      int c = 64 * t + lane;
+      const int cmax = NORM == 1 ? 119 : 59;
+      c = c < cmax ? c : cmax;
+      const unsigned dst = lds_addr(scw + wave * 2048 + t * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(static_cast<unsigned>(c * 16)), "s"(sbase) : "memory", "m0");
+    }
+  }
+  // A CU takes only so many loads at a time; a wavefront that issues one more simply stalls until the queue has
+  // drained that far. Without the norm that costs nothing: everything is requested at once. With it, the wavefronts
+  // must see their activations, exchange sums and scale before the first MFMA, and one stuck issuing weight loads
+  // would hold the others up at the barrier: so all activation loads go first (the rendezvous puts them at the head
+  // of the CU's queue, which returns loads in the order it took them), one phase of weight keeps the memory system
+  // busy meanwhile, and the other three phases are requested after the norm.
+  constexpr int EARLY = NORM != 0 ? 1 : RING;
+  if constexpr (NORM != 0) {
+    if (lane == 0) s_flag[wave] = 0;
+    __syncthreads();
+  }
+#pragma unroll
+  for (int p = 0; p < EARLY; ++p) issue_phase(p);
+  R8_STAMP(1);
+
+  // ---- activation fragments into registers (the weight loads issued so far are younger and stay outstanding)
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(EARLY * 5) : "memory");
+  R8_STAMP(2);
+  bf16x8 fb[STEPS];
+  auto xfrag = [&](int s) { return *reinterpret_cast<const bf16x8*>(myx + m1 * XBLOCK + (((4 * s + g) ^ (2 * m1)) << 4)); };
+  if constexpr (NORM == 0) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) fb[s] = xfrag(s);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    issue_phase(3);
+  } else {
+    // Columns 8..15 of the MFMA are never stored, so lanes m >= 8 are free to do half of the norm's arithmetic: a
+    // lane fetches and scales the fragments of the steps of its own parity (h = bit 3 of the lane), and the lanes
+    // m < 8 then take the other parity's from their partner 8 lanes up (one DPP move per register).
+    const int h = (lane >> 3) & 1;
+    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+    bf16x8 own[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int sj = 2 * j + h;
+      own[j] = xfrag(sj < STEPS ? sj : STEPS - 2);            // (h = 1, j = 7) has no step: re-reads step 13, masked below
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the activation blocks are free from here on
+    if constexpr (EMB) {
+      if (!xok_m1) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+#pragma unroll
+          for (int q = 0; q < 8; ++q) own[j][q] = static_cast<bf16>(0.f);
+        }
+      }
+      if (blockIdx.x == 0 && m1 < nvalid) {                 // the gathered rows, as the residual stream: every lane its own fragments
+        bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + (row0 + m1) * 360 + kq * 60 + g;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (2 * j + h < STEPS) xo[4 * (2 * j + h)] = own[j];
+        }
+      }
+    }
+    float ssq = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float part = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float f = static_cast<float>(own[j][q]);
+        part = fmaf(f, f, part);
+      }
+      ssq += (j == 7 && h == 1) ? 0.f : part;
+    }
+    ssq += __shfl_xor(ssq, 8, 64);
+    ssq += __shfl_xor(ssq, 16, 64);
+    ssq += __shfl_xor(ssq, 32, 64);
+    // The six slices' sums meet through LDS, but not at a barrier: a wavefront publishes its eight sums, raises
+    // its flag and goes on to request the rest of its weight (where it may sit for a microsecond until the CU's
+    // queue takes the loads); only then does it wait for the other five flags, which by that time are long up.
+    if (lane < XR) s_part[wave * XR + lane] = ssq;          // lanes 0..7: row m1 == lane
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the loads in flight are none of its business
+    if (lane == 0) __hip_atomic_store(&s_flag[wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+    for (int p = EARLY; p < 4; ++p) issue_phase(p);
+    for (;;) {                                              // every streaming wavefront raises its flag before it gets here or exits
+      const unsigned f = lane < NS ? __hip_atomic_load(&s_flag[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : 1u;
+      if (__all(f != 0u)) break;
+      __builtin_amdgcn_s_sleep(2);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#ifdef TLLM_R8_STAMPS
+    R8_STAMP(3);
+#endif
+    float ss = 0.f;
+#pragma unroll
+    for (int w = 0; w < NS; ++w) ss += s_part[w * XR + m1];
+    const float rinv = rsqrtf(ss * (1.0f / 2880.0f) + a.norm_eps);
+    const unsigned char* sc = scw + wave * 2048;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int sj = 2 * j + h < STEPS ? 2 * j + h : STEPS - 2;
+      f32x4 s_lo, s_hi;
+      if constexpr (NORM == 1) {
+        s_lo = *reinterpret_cast<const f32x4*>(sc + (4 * sj + g) * 32);
+        s_hi = *reinterpret_cast<const f32x4*>(sc + (4 * sj + g) * 32 + 16);
+      } else {
+        const bf16x8 t = *reinterpret_cast<const bf16x8*>(sc + (4 * sj + g) * 16);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          s_lo[q] = static_cast<float>(t[q]);
+          s_hi[q] = static_cast<float>(t[4 + q]);
+        }
+      }
+      bf16x8 t;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) t[q] = static_cast<bf16>(static_cast<float>(own[j][q]) * rinv * (q < 4 ? s_lo[q] : s_hi[q - 4]));
+      own[j] = t;
+    }
+    // lanes m < 8 (h = 0): even steps are their own, odd steps come from lane + 8; lanes m >= 8 end up with a mix
+    // that only feeds the unused columns
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      fb[2 * j] = own[j];
+      if (2 * j + 1 < STEPS) {
+        const u32x4 mine = __builtin_bit_cast(u32x4, own[j]);
+        u32x4 theirs;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) theirs[q] = __builtin_amdgcn_update_dpp(0u, mine[q], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+        fb[2 * j + 1] = __builtin_bit_cast(bf16x8, theirs);
+      }
+    }
+#ifdef TLLM_R8_STAMPS
+    R8_STAMP(4);
+#endif
+  }
+
+  // ---- the stream: phase by phase out of LDS into the matrix core
+  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  const int arow0 = m < 12 ? m : m - 12;                    // tile rows past the last real one re-read a real one (their sums are dropped)
+  const unsigned a0_o = arow0 * 256, a1_o = (12 + m1) * 256;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    // five loads per phase, all four phases requested by now: phase p has landed when 5 * (3 - p) are outstanding
+    if (p == 0) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+    else if (p == 1) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+    else if (p == 2) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (NORM == 0 && p == 0) R8_STAMP(3);
+    if (NORM == 0 && p == 3) R8_STAMP(4);
+    const unsigned char* reg = phase_region(p);
+    constexpr int kMaxSt = 4;
+    bf16x8 fa0[kMaxSt], fa1[kMaxSt];
+    const int nst = p == 3 ? 3 : 4;
+#pragma unroll
+    for (int st = 0; st < nst; ++st) {                      // all fragment reads of the phase in one go, then its MFMAs
+      fa0[st] = *reinterpret_cast<const bf16x8*>(reg + a0_o + (((4 * st + g) ^ arow0) << 4));
+      fa1[st] = *reinterpret_cast<const bf16x8*>(reg + a1_o + (((4 * st + g) ^ m1) << 4));
+    }
+#pragma unroll
+    for (int st = 0; st < nst; ++st) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[st], fb[4 * p + st], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[st], fb[4 * p + st], acc1, 0, 0, 0);
+    }
+  }
+
+  // ---- partial tiles -> LDS (the wavefront's own region 1, long since consumed), then the epilogue wavefronts take over
+  *reinterpret_cast<f32x4*>(myring + REGION + lane * 16) = acc0;
+  *reinterpret_cast<f32x4*>(myring + REGION + 1024 + lane * 16) = acc1;
+  R8_STAMP(5);
+  __syncthreads();
+}
+
+// Host side: pick the instantiation. norm = 0 / 1 (fp32 scale) / 2 (bf16 scale).
+void launch_qkv_decode_r8(int norm, bool emb, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+  auto even = [](int64_t v) { return (v & 1) == 0; };
+  const int out4 = (reinterpret_cast<uintptr_t>(a.q) % 4 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 4 == 0) &&
+                   (reinterpret_cast<uintptr_t>(a.v) % 4 == 0) && even(a.q_rs) && even(a.k_rs) && even(a.v_rs) && even(a.kv_slot_stride);
+#define TLLM_R8(NORM, EMBF) hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF>), grid, dim3(512), 0, st, a, ra, fr, out4)
+  if (emb) {
+    if (norm == 1) TLLM_R8(1, true);
+    else TLLM_R8(2, true);
+  } else if (norm == 0) TLLM_R8(0, false);
+  else if (norm == 1) TLLM_R8(1, false);
+  else TLLM_R8(2, false);
+#undef TLLM_R8
+}
+
+}  // namespace tllm
+
+#ifdef TLLM_R8_STAMPS
+extern "C" int tllm_debug_r8_stamps(void* host, size_t bytes) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tllm::g_r8_stamps), bytes); }
+#endif
