@@ -6,7 +6,8 @@
 // leaves the VALU to the rotary epilogue -- and keep a rotation pair (row d and row d+32 of a
 // head) inside one workgroup so the rotation needs no second pass. The kernels:
 //   qkv_decode_r8_kernel   hidden == 2880 (gpt-oss), up to 8 rows, bf16 weight: qkv_decode_r8.hip, the fastest.
-//   qkv_decode_cu_kernel   hidden == 2880, 9 rows and more, or an fp8 weight: one workgroup per CU, coalesced
+//   qkv_decode_r32_kernel  hidden == 2880, 9..32 rows per workgroup, bf16 weight, no fused norm: qkv_decode_r32.hip.
+//   qkv_decode_cu_kernel   hidden == 2880, the other cases (fused norm beyond 8 rows, fp8 weight): one workgroup per CU, coalesced
 //                          loads, LDS-transposed operands; see its comment.
 //   qkv_decode_kernel      head_dim == 64, hidden % 32 == 0: operands loaded straight into MFMA
 //                          layout (simple, ~1.8x slower: every lane is its own cache-line request).
@@ -621,12 +622,15 @@ static void launch_cu(int xr, int norm, bool w8, dim3 grid, hipStream_t st, cons
 static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, int norm, bool w8, int64_t rows,
                               int heads, hipStream_t st) {
   TLLM_REQUIRE(static_cast<int64_t>(heads) * 64 * 2880 < (1ll << 31), TLLM_E_SHAPE, "%s: weight too large", what);
-  const int xr = rows <= 8 ? 8 : (rows <= 16 ? 16 : 32);
+  // the activations are addressed with 32-bit byte offsets in the two kernels that load straight into LDS
+  const bool fits32 = (a.emb_ids ? a.emb_vocab : rows) * 5760 < (1ll << 32);
+  const bool r32 = rows > 8 && !w8 && norm == 0 && !a.emb_ids && fits32;   // 9..32 rows per workgroup, normalised activations
+  const int xr = rows <= 8 ? 8 : ((rows <= 16 && !r32) ? 16 : 32);
   const int64_t chunks = (rows + xr - 1) / xr;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
   const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
-  const bool fits32 = (a.emb_ids ? a.emb_vocab : rows) * 5760 < (1ll << 32);   // the kernel addresses activation rows with 32-bit byte offsets
-  if (xr == 8 && !w8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, grid, st, a, ra, fr);
+  if (r32) launch_qkv_decode_r32(grid, st, a, ra, fr);
+  else if (xr == 8 && !w8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, grid, st, a, ra, fr);
   else if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
   else launch_cu(xr, norm, w8, grid, st, a, ra, fr);
   return check_launch(what);

@@ -1,0 +1,223 @@
+// Decode-size fused QKV projection + bias + rotary for hidden == 2880 and 9..32 activation rows per workgroup (bf16
+// weight, activations already normalised): the companion of qkv_decode_r8.hip for the larger decode batches.
+//
+// Same skeleton: 256 workgroups of ten rotation pairs (20 weight rows, two 16-row MFMA tiles with the quad layout
+// [lo(2i), lo(2i+1), hi(2i), hi(2i+1)]), six streaming wavefronts that each own one K slice of 480 (fifteen k32
+// steps in phases of 4 + 4 + 4 + 3), everything loaded from global memory straight into LDS with the XOR swizzle
+// chosen on the global side, fragments read back once, partial tiles reduced in a fixed order by epilogue wavefronts.
+// What differs: 32 activation rows are 184 KB per workgroup, more than the LDS holds, so the activations arrive in the
+// same four phases as the weight -- a phase is 8 KB of activations (32 rows x 256 bytes) and 5 KB of weight -- through
+// a ring of two 13 KB regions per wavefront; a phase is multiplied (two tiles x two column blocks of 16 rows) as soon
+// as it has landed and its region is then refilled with the phase after next. Four epilogue wavefronts, one per
+// (tile, column block).
+#include "qkv_common.h"
+
+namespace tllm {
+
+namespace r32 {
+constexpr int XR = 32;            // activation rows per workgroup
+constexpr int NS = 6;             // streaming wavefronts = K slices
+constexpr int NE = 4;             // epilogue wavefronts = (tile, column block)
+constexpr int PAIRS = 10;         // rotation pairs per workgroup
+constexpr int RING = 2;           // resident phases per wavefront
+constexpr int XPH = 8 * 1024;     // activations of one phase: 32 rows x four k32 steps
+constexpr int WPH = 5 * 1024;     // weight of one phase: 20 rows x four k32 steps
+constexpr int REGION = XPH + WPH;
+constexpr int LPP = 13;           // load instructions per phase
+}  // namespace r32
+
+__global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int out4) {
+  using namespace r32;
+  __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int total_pairs = (a.n_q_heads + 2 * a.n_kv_heads) * 32;
+  const int pair0 = blockIdx.x * PAIRS;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
+  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+
+  if (wave >= NS) {
+    // ======================================================================= epilogue wavefront of (tile, column block)
+    const int tile = (wave - NS) & 1, cb = (wave - NS) >> 1;
+    const int en = 16 * cb + (lane & 15), eg = lane >> 4;   // activation row, quad of the tile
+    const int epair = pair0 + (tile ? 6 : 0) + 2 * eg;      // even; its neighbour epair + 1 shares head and quad
+    const bool evalid = eg < (tile ? 2 : 3) && epair < total_pairs && en < nvalid;
+    const int egp = evalid ? epair : 0;
+    const int ehead = egp >> 5, ed = egp & 31;
+    const int64_t erow = row0 + (evalid ? en : 0);
+    const bool erot = a.has_rope && ehead < a.n_q_heads + a.n_kv_heads;
+    const int64_t* pos_ptr = ra.positions ? ra.positions + erow : reinterpret_cast<const int64_t*>(a.W);
+    const int64_t* off_ptr = ra.offset ? ra.offset : reinterpret_cast<const int64_t*>(a.W);
+    const unsigned* bias_ptr = reinterpret_cast<const unsigned*>(a.bias ? a.bias : a.W);   // two bf16 per load; ed is even
+    const int64_t pos_ld = *pos_ptr;
+    const int64_t off_ld = *off_ptr;
+    const unsigned b_lo = bias_ptr[(ehead * 64 + ed) >> 1];
+    const unsigned b_hi = bias_ptr[(ehead * 64 + 32 + ed) >> 1];
+    const float freq0 = fr.v[ed], freq1 = fr.v[ed + 1];
+    float cs0 = 1.f, sn0 = 0.f, cs1 = 1.f, sn1 = 0.f;
+    const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
+    if (erot) {
+      int64_t pos = ra.positions ? pos_ld : (erow % ra.tokens_per_batch) + (ra.offset ? off_ld : 0);
+      pos = rope_wrap(pos, ra.max_ctx);
+      if (ra.use_yarn) {
+        yarn_cos_sin(pos, freq0, ra.concentration, &cs0, &sn0);
+        yarn_cos_sin(pos, freq1, ra.concentration, &cs1, &sn1);
+      } else {
+        rope_cos_sin(ra, fr, pos, ed, &cs0, &sn0);
+        rope_cos_sin(ra, fr, pos, ed + 1, &cs1, &sn1);
+      }
+    }
+    float bl0 = 0.f, bl1 = 0.f, bh0 = 0.f, bh1 = 0.f;
+    if (a.bias) {
+      bl0 = __uint_as_float(b_lo << 16);
+      bl1 = __uint_as_float(b_lo & 0xffff0000u);
+      bh0 = __uint_as_float(b_hi << 16);
+      bh1 = __uint_as_float(b_hi & 0xffff0000u);
+    }
+    bf16* out = qkv_out_ptr(a, slot, erow, ehead) + ed;
+    unsigned red_o = static_cast<unsigned>((2 * tile + cb) * 1024 + lane * 16);
+    // everything that does not need the sums exists before the barrier (see qkv_decode_r8.hip)
+    asm volatile("" : "+v"(cs0), "+v"(sn0), "+v"(cs1), "+v"(sn1), "+v"(bl0), "+v"(bl1), "+v"(bh0), "+v"(bh1), "+v"(out), "+v"(red_o));
+    __syncthreads();                                        // partial tiles are in LDS
+    f32x4 t[NS];
+#pragma unroll
+    for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(ring + w * (RING * REGION) + red_o);
+    f32x4 acc = t[0];
+#pragma unroll
+    for (int w = 1; w < NS; ++w) {                          // fixed order: the result does not depend on timing
+      acc[0] += t[w][0];
+      acc[1] += t[w][1];
+      acc[2] += t[w][2];
+      acc[3] += t[w][3];
+    }
+    if (!evalid) return;
+    float lo0 = acc[0] + bl0, lo1 = acc[1] + bl1, hi0 = acc[2] + bh0, hi1 = acc[3] + bh1;   // [lo(d), lo(d+1), hi(d), hi(d+1)] of row en
+    if (erot) {
+      const float r0 = lo0 * cs0 - hi0 * sn0, r2 = hi0 * cs0 + lo0 * sn0;
+      const float r1 = lo1 * cs1 - hi1 * sn1, r3 = hi1 * cs1 + lo1 * sn1;
+      lo0 = r0;
+      lo1 = r1;
+      hi0 = r2;
+      hi1 = r3;
+    }
+    bf16x2 plo, phi;
+    plo[0] = static_cast<bf16>(lo0);
+    plo[1] = static_cast<bf16>(lo1);
+    phi[0] = static_cast<bf16>(hi0);
+    phi[1] = static_cast<bf16>(hi1);
+    if (out4) {
+      *reinterpret_cast<bf16x2*>(out) = plo;
+      *reinterpret_cast<bf16x2*>(out + 32) = phi;
+    } else {
+      out[0] = plo[0];
+      out[1] = plo[1];
+      out[32] = phi[0];
+      out[33] = phi[1];
+    }
+    return;
+  }
+
+  // ========================================================================= streaming wavefront of K slice `kq`
+  const int kq = wave;
+  const int m = lane & 15, g = lane >> 4, m1 = m & 7;
+  unsigned char* myring = ring + wave * (RING * REGION);
+
+  // lane -> (row r4 of a 4-row block, position pos): it fetches chunk pos ^ (row & 15) of that row, so that the 16 rows
+  // a fragment read touches lie in 16 different bank groups. Phase 3 has three steps: chunks 0..11 only.
+  unsigned xoff[8], xoff3[8], goff[5], goff3[5];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int r = 4 * j + (lane >> 4);
+    const int64_t src = row0 + (r < nvalid ? r : nvalid - 1);
+    const int cc = (lane & 15) ^ (r & 15);
+    xoff[j] = static_cast<unsigned>(src * 5760 + kq * 960 + cc * 16);
+    xoff3[j] = static_cast<unsigned>(src * 5760 + kq * 960 + (cc < 12 ? cc : 11) * 16);
+  }
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    const int row20 = 4 * j + (lane >> 4);                  // 0..11 tile 0, 12..19 tile 1
+    const int tile = row20 >= 12, trow = tile ? row20 - 12 : row20;
+    const int quad = trow >> 2, q = trow & 3;
+    int gp = pair0 + (tile ? 6 : 0) + 2 * quad + (q & 1);
+    gp = gp < total_pairs ? gp : total_pairs - 1;
+    const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + ((q & 2) ? 32u : 0u);
+    const int cc = (lane & 15) ^ (trow & 15);
+    goff[j] = wrow * 5760u + kq * 960u + cc * 16u;
+    goff3[j] = wrow * 5760u + kq * 960u + (cc < 12 ? cc : 11) * 16u;
+  }
+  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
+  const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
+  auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
+  auto issue_phase = [&](int p) {                           // thirteen loads: the activations of the phase, then its weight
+    unsigned char* reg = myring + (p % RING) * REGION;
+    const unsigned char* xb = xbase + p * 256;
+    const unsigned char* wb = wbase + p * 256;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const unsigned dst = lds_addr(reg + j * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(p == 3 ? xoff3[j] : xoff[j]), "s"(xb) : "memory", "m0");
+    }
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const unsigned dst = lds_addr(reg + XPH + j * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == 3 ? goff3[j] : goff[j]), "s"(wb) : "memory", "m0");
+    }
+  };
+  issue_phase(0);
+  issue_phase(1);
+
+  f32x4 acc[2][2];                                          // [tile][column block]
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) acc[t][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int arow0 = m < 12 ? m : m - 12;                    // tile rows past the last real one re-read a real one (their sums are dropped)
+  const unsigned a0_o = XPH + arow0 * 256, a1_o = XPH + (12 + m1) * 256;
+  const unsigned b0_o = m * 256, b1_o = (16 + m) * 256;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    // phase p has landed when only the loads of the phase after it (if requested) are outstanding
+    if (p < 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPP) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned char* reg = myring + (p % RING) * REGION;
+    const int nst = p == 3 ? 3 : 4;
+    bf16x8 fa0[4], fa1[4], fb0[4], fb1[4];
+#pragma unroll
+    for (int st = 0; st < nst; ++st) {
+      fb0[st] = *reinterpret_cast<const bf16x8*>(reg + b0_o + (((4 * st + g) ^ m) << 4));
+      fb1[st] = *reinterpret_cast<const bf16x8*>(reg + b1_o + (((4 * st + g) ^ m) << 4));
+      fa0[st] = *reinterpret_cast<const bf16x8*>(reg + a0_o + (((4 * st + g) ^ arow0) << 4));
+      fa1[st] = *reinterpret_cast<const bf16x8*>(reg + a1_o + (((4 * st + g) ^ m1) << 4));
+    }
+    if (p + RING < 4) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the region's fragments are in registers: it may be refilled
+      issue_phase(p + RING);
+    }
+#pragma unroll
+    for (int st = 0; st < nst; ++st) {
+      acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[st], fb0[st], acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[st], fb1[st], acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[st], fb0[st], acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[st], fb1[st], acc[1][1], 0, 0, 0);
+    }
+  }
+
+  // ---- partial tiles -> LDS: the wavefront's own region 0 (phase 2, consumed; phase 3 sat in region 1)
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) *reinterpret_cast<f32x4*>(myring + (2 * t + c) * 1024 + lane * 16) = acc[t][c];
+  }
+  __syncthreads();
+}
+
+void launch_qkv_decode_r32(dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+  auto even = [](int64_t v) { return (v & 1) == 0; };
+  const int out4 = (reinterpret_cast<uintptr_t>(a.q) % 4 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 4 == 0) &&
+                   (reinterpret_cast<uintptr_t>(a.v) % 4 == 0) && even(a.q_rs) && even(a.k_rs) && even(a.v_rs) && even(a.kv_slot_stride);
+  hipLaunchKernelGGL(qkv_decode_r32_kernel, grid, dim3(640), 0, st, a, ra, fr, out4);
+}
+
+}  // namespace tllm
