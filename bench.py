@@ -30,9 +30,10 @@ if ROOT not in sys.path:
 
 # HBM bytes per launch of the decode QKV kernel at B=8, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch), FETCH_SIZE scaled by the 2.000 a 256 MiB copy of known size reads on the same counter:
-# 14691.9 x 2.000 + 192.0 KiB with the fused norm, 14644.9 x 2.000 + 192.0 KiB without.
-# Summary and commands: profiles/qkv_decode_cu_kernel_B8_decode_step.md. Not re-measured by this script.
-QKV_DECODE_TRAFFIC_BYTES = {"fused": int((14691.9 * 2.000 + 192.0) * 1024), "unfused": int((14644.9 * 2.000 + 192.0) * 1024)}
+# 14715.8 x 2.000 + 192.0 KiB with the fused norm, 14668.1 x 2.000 + 192.0 KiB without.
+# Summary and commands: profiles/qkv_decode_r8_kernel_B8_decode_step.md. Not re-measured by this script: when the
+# kernel changes, the profile has to be taken again.
+QKV_DECODE_TRAFFIC_BYTES = {"fused": int((14715.8 * 2.000 + 192.0) * 1024), "unfused": int((14668.1 * 2.000 + 192.0) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published (no sparsity)
 
@@ -372,7 +373,7 @@ def main() -> int:
         "bound": "hbm", "achieved": round(qkv_bytes / qkv_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(qkv_bytes / qkv_s / 1e9 / HBM_PEAK_GBS, 4),
         "traffic": QKV_DECODE_TRAFFIC_BYTES["unfused" if args.unfused else "fused"],
-        "traffic_source": "rocprofv3 --pmc FETCH_SIZE (x2.000 copy calibration) + WRITE_SIZE, profiles/qkv_decode_cu_kernel_B8_decode_step.md",
+        "traffic_source": "rocprofv3 --pmc FETCH_SIZE (x2.000 copy calibration) + WRITE_SIZE, profiles/qkv_decode_r8_kernel_B8_decode_step.md",
         "bytes_per_launch": qkv_bytes, "avg_launch_us": round(qkv_s * 1e6, 3),
     }
 

@@ -180,12 +180,12 @@ __global__ __launch_bounds__(256) void rmsnorm_scalar_kernel(const bf16* x, cons
 }
 
 template <bool kScaleBf16, bool GATHER>
-static void launch_wave(int vpl, const bf16x8* x, const void* scale, bf16x8* out, int64_t rows, int nvec, float inv_h, float eps,
+static void launch_wave(int vpl, const bf16x8* x, const void* scale, bf16x8* out, int64_t rows, int nvec, float hidden_f, float eps,
                         const GatherSrc& g, hipStream_t st) {
   dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(256);
 #define TLLM_CASE(V)                                                                                                             \
   case V:                                                                                                                        \
-    hipLaunchKernelGGL((rmsnorm_wave_kernel<V, kScaleBf16, GATHER>), grid, block, 0, st, x, scale, out, rows, nvec, inv_h, eps, g); \
+    hipLaunchKernelGGL((rmsnorm_wave_kernel<V, kScaleBf16, GATHER>), grid, block, 0, st, x, scale, out, rows, nvec, hidden_f, eps, g); \
     break;
   switch (vpl) {
     TLLM_CASE(1) TLLM_CASE(2) TLLM_CASE(3) TLLM_CASE(4) TLLM_CASE(5) TLLM_CASE(6) TLLM_CASE(7) TLLM_CASE(8)
@@ -195,12 +195,12 @@ static void launch_wave(int vpl, const bf16x8* x, const void* scale, bf16x8* out
 }
 
 template <bool kScaleBf16, bool GATHER>
-static void launch_block(int vpt, const bf16x8* x, const void* scale, bf16x8* out, int64_t rows, int nvec, float inv_h, float eps,
+static void launch_block(int vpt, const bf16x8* x, const void* scale, bf16x8* out, int64_t rows, int nvec, float hidden_f, float eps,
                          const GatherSrc& g, hipStream_t st) {
   dim3 grid(static_cast<unsigned>(rows)), block(256);
 #define TLLM_CASE(V)                                                                                                        \
   case V:                                                                                                                   \
-    hipLaunchKernelGGL((rmsnorm_block_kernel<V, kScaleBf16, GATHER>), grid, block, 0, st, x, scale, out, nvec, inv_h, eps, g); \
+    hipLaunchKernelGGL((rmsnorm_block_kernel<V, kScaleBf16, GATHER>), grid, block, 0, st, x, scale, out, nvec, hidden_f, eps, g); \
     break;
   switch (vpt) { TLLM_CASE(1) TLLM_CASE(2) TLLM_CASE(3) TLLM_CASE(4) }
 #undef TLLM_CASE
@@ -217,22 +217,22 @@ static constexpr int64_t kBlockPerRowMaxRows = 512;
 template <bool GATHER>
 static bool launch_vector(const void* x, const void* scale, int scale_is_bf16, void* out, int64_t rows, int64_t hidden, float eps,
                           const GatherSrc& g, hipStream_t st) {
-  const float inv_h = static_cast<float>(hidden);  // divisor of the mean
+  const float hidden_f = static_cast<float>(hidden);  // divisor of the mean
   const int64_t nvec = hidden / 8;
   if (rows <= kBlockPerRowMaxRows && nvec <= 4 * 256) {
     const int vpt = static_cast<int>((nvec + 255) / 256);
     if (scale_is_bf16)
-      launch_block<true, GATHER>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+      launch_block<true, GATHER>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, hidden_f, eps, g, st);
     else
-      launch_block<false, GATHER>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+      launch_block<false, GATHER>(vpt, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, hidden_f, eps, g, st);
     return true;
   }
   if (nvec <= 16 * 64) {
     const int vpl = static_cast<int>((nvec + 63) / 64);
     if (scale_is_bf16)
-      launch_wave<true, GATHER>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+      launch_wave<true, GATHER>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, hidden_f, eps, g, st);
     else
-      launch_wave<false, GATHER>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, inv_h, eps, g, st);
+      launch_wave<false, GATHER>(vpl, (const bf16x8*)x, scale, (bf16x8*)out, rows, (int)nvec, hidden_f, eps, g, st);
     return true;
   }
   return false;
