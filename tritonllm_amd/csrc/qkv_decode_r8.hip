@@ -11,7 +11,8 @@
 //   * A CU returns vector loads in the order it took them, across wavefronts, and takes only so many at a time. A
 //     barrier that waits for staged activations therefore waits for every weight load queued ahead of them. Here no
 //     wavefront ever waits for another one's loads: each of the six streaming wavefronts owns one K slice of 480
-//     (fifteen k32 steps) and brings in its own slice of the activations, then its slice of the 20 weight rows.
+//     (fifteen k32 steps, taken as its share of four phases so that the six together read contiguous memory) and
+//     brings in its own slice of the activations, then its slice of the 20 weight rows.
 //   * Passing the stream through registers and ds_write into operand layout costs as much time as the stream
 //     itself (loads, LDS writes and LDS reads all cross the same register-file port). Here everything goes from
 //     global memory straight into LDS (global_load_lds_dwordx4: a wavefront's 64 x 16 bytes land at consecutive LDS
@@ -160,6 +161,11 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
 
   // ========================================================================= streaming wavefront of K slice `kq`
   const int kq = wave;
+  // The K slice of a wavefront is not one run of 480 but its share of each phase: in phase p < 3 the six wavefronts
+  // together read 24 consecutive k32 steps (1536 contiguous bytes of every weight row), wavefront kq steps
+  // 24 p + 4 kq .. + 4; in phase 3, 18 steps, wavefront kq steps 72 + 3 kq .. + 3. What a CU requests within a short
+  // time is then contiguous in memory. kb(c): byte offset inside a bf16 row of this wavefront's 16-byte chunk c (0..59).
+  auto kb = [&](int c) { return c < 48 ? (c >> 4) * 1536 + kq * 256 + (c & 15) * 16 : 4608 + kq * 192 + (c - 48) * 16; };
   const int m = lane & 15, g = lane >> 4, m1 = m & 7;
   unsigned char* myx = xw + wave * (XR * XBLOCK);
   unsigned char* myring = ring + wave * (RING * REGION);
@@ -194,7 +200,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     for (int n = 0; n < XR; ++n) {
       int c = lane ^ (2 * n);
       c = c < 60 ? c : 59;
-      xoff[n] = static_cast<unsigned>(src_row[n] * 5760 + kq * 960 + c * 16);
+      xoff[n] = static_cast<unsigned>(src_row[n] * 5760 + kb(c));
     }
   }
   // weight: lane -> (row r4 of a 4-row block, position pos): it fetches chunk pos ^ (tile row & 15) of that row
@@ -208,8 +214,8 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     gp = gp < total_pairs ? gp : total_pairs - 1;
     const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + ((q & 2) ? 32u : 0u);
     const int cc = (lane & 15) ^ (trow & 15);
-    goff[j] = wrow * 5760u + kq * 960u + cc * 16u;
-    goff3[j] = wrow * 5760u + kq * 960u + (cc < 12 ? cc : 11) * 16u;
+    goff[j] = wrow * 5760u + kq * 256u + cc * 16u;
+    goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
   }
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // as the activation fragments are in registers -- so no weight load ever waits for an MFMA.
   auto phase_region = [&](int p) -> unsigned char* { return p < RING ? myring + p * REGION : myx; };
   auto issue_phase = [&](int p) {
-    const unsigned char* sb = wbase + p * 256;
+    const unsigned char* sb = wbase + (p < 3 ? p * 1536 : 4608);
 #pragma unroll
     for (int j = 0; j < 5; ++j) {
       const unsigned dst = lds_addr(phase_region(p) + j * 1024);
@@ -233,14 +239,15 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   }
   constexpr int NSC = NORM == 1 ? 2 : (NORM == 2 ? 1 : 0);   // scale loads: 480 fp32 = 120 chunks, 480 bf16 = 60 chunks
   if constexpr (NORM != 0) {
-    const unsigned char* sbase = reinterpret_cast<const unsigned char*>(a.norm_scale) + kq * (NORM == 1 ? 1920 : 960);
+    const unsigned char* sbase = reinterpret_cast<const unsigned char*>(a.norm_scale);
 #pragma unroll
     for (int t = 0; t < NSC; ++t) {
-      int c = 64 * t + lane;
+      int c = 64 * t + lane;                                // 16-byte chunk of the slice's scale: 4 fp32 or 8 bf16 values
       const int cmax = NORM == 1 ? 119 : 59;
       c = c < cmax ? c : cmax;
+      const unsigned off = NORM == 1 ? 2u * kb(c >> 1) + (c & 1) * 16u : static_cast<unsigned>(kb(c));
       const unsigned dst = lds_addr(scw + wave * 2048 + t * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(static_cast<unsigned>(c * 16)), "s"(sbase) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(sbase) : "memory", "m0");
     }
   }
   // A CU takes only so many loads at a time; a wavefront that issues one more simply stalls until the queue has
@@ -290,10 +297,10 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
         }
       }
       if (blockIdx.x == 0 && m1 < nvalid) {                 // the gathered rows, as the residual stream: every lane its own fragments
-        bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + (row0 + m1) * 360 + kq * 60 + g;
+        bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + (row0 + m1) * 360;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          if (2 * j + h < STEPS) xo[4 * (2 * j + h)] = own[j];
+          if (2 * j + h < STEPS) xo[kb(4 * (2 * j + h) + g) >> 4] = own[j];
         }
       }
     }
