@@ -3,7 +3,8 @@
 //
 // Same skeleton: 256 workgroups of ten rotation pairs (20 weight rows, two 16-row MFMA tiles with the quad layout
 // [lo(2i), lo(2i+1), hi(2i), hi(2i+1)]), six streaming wavefronts that each own one K slice of 480 (fifteen k32
-// steps in phases of 4 + 4 + 4 + 3), everything loaded from global memory straight into LDS with the XOR swizzle
+// steps in phases of 4 + 4 + 4 + 3, a wavefront's steps being its share of each phase so that the six together read
+// contiguous memory), everything loaded from global memory straight into LDS with the XOR swizzle
 // chosen on the global side, fragments read back once, partial tiles reduced in a fixed order by epilogue wavefronts.
 // What differs: 32 activation rows are 184 KB per workgroup, more than the LDS holds, so the activations arrive in the
 // same four phases as the weight -- a phase is 8 KB of activations (32 rows x 256 bytes) and 5 KB of weight -- through
@@ -131,8 +132,8 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     const int r = 4 * j + (lane >> 4);
     const int64_t src = row0 + (r < nvalid ? r : nvalid - 1);
     const int cc = (lane & 15) ^ (r & 15);
-    xoff[j] = static_cast<unsigned>(src * 5760 + kq * 960 + cc * 16);
-    xoff3[j] = static_cast<unsigned>(src * 5760 + kq * 960 + (cc < 12 ? cc : 11) * 16);
+    xoff[j] = static_cast<unsigned>(src * 5760 + kq * 256 + cc * 16);
+    xoff3[j] = static_cast<unsigned>(src * 5760 + kq * 192 + (cc < 12 ? cc : 11) * 16);
   }
 #pragma unroll
   for (int j = 0; j < 5; ++j) {
@@ -143,16 +144,18 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     gp = gp < total_pairs ? gp : total_pairs - 1;
     const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + ((q & 2) ? 32u : 0u);
     const int cc = (lane & 15) ^ (trow & 15);
-    goff[j] = wrow * 5760u + kq * 960u + cc * 16u;
-    goff3[j] = wrow * 5760u + kq * 960u + (cc < 12 ? cc : 11) * 16u;
+    goff[j] = wrow * 5760u + kq * 256u + cc * 16u;
+    goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
   }
   const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
   auto issue_phase = [&](int p) {                           // thirteen loads: the activations of the phase, then its weight
     unsigned char* reg = myring + (p % RING) * REGION;
-    const unsigned char* xb = xbase + p * 256;
-    const unsigned char* wb = wbase + p * 256;
+    // phase p < 3: the six wavefronts together take 24 consecutive k32 steps (1536 contiguous bytes of every row),
+    // wavefront kq steps 24 p + 4 kq .. + 4; phase 3: 18 steps, wavefront kq steps 72 + 3 kq .. + 3
+    const unsigned char* xb = xbase + (p < 3 ? p * 1536 : 4608);
+    const unsigned char* wb = wbase + (p < 3 ? p * 1536 : 4608);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const unsigned dst = lds_addr(reg + j * 1024);
