@@ -109,7 +109,11 @@ def host_cpu_info() -> dict:
     return {"model": model, "physical": physical, "logical": logical, "usable": usable, "threads_used": max(threads, 1), "note": note}
 
 
-def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg) -> int:
+def name_of_stamps(fused: bool) -> str:
+    return "qkv_decode_r8_kernel<2,false>" if fused else "qkv_decode_r8_kernel<0,false>"
+
+
+def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg, _lib) -> int:
     """One kernel-table entry on its own (a clean target for rocprofv3)."""
     name = args.only
     kind, _, size = name.rpartition("_")
@@ -188,6 +192,48 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         fn = lambda i: T.attention_decode(aq, ak[i % 4], av[i % 4], asink, 0.125, win, astart, kv_len_hint=hint)
         keys = min(ctx, 128) if win else ctx
         nbytes = n * NKV * keys * HD * 2 * 2 + n * NQ * HD * 2 * 2
+    elif kind in ("r8_stamps", "norm_r8_stamps"):
+        # Time stamps the decode kernel for up to 8 rows writes itself (a build with the stamps compiled in:
+        # TLLM_EXTRA_HIPCC_FLAGS=-DTLLM_R8_STAMPS python -m tritonllm_amd.build): wall_clock64() at eight points of every
+        # wavefront of every workgroup, read back after the last launch of a replayed 48-launch graph.
+        import ctypes
+
+        import numpy as np
+
+        L = _lib.lib()
+        if not hasattr(L, "tllm_debug_r8_stamps"):
+            print("bench.py: the library has no stamps (rebuild with TLLM_EXTRA_HIPCC_FLAGS=-DTLLM_R8_STAMPS)", file=sys.stderr)
+            return 2
+        L.tllm_debug_r8_stamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+        fused = kind.startswith("norm_")
+        xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
+        pp = torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
+        qo = (torch.empty(n, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev),
+              torch.empty(n, NKV * HD, dtype=torch.bfloat16, device=dev))
+        fn = lambda i: T.qkv_rope_forward(xp, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn, positions=pp, mode="decode",
+                                          out=qo, norm_scale=scales[i % N_LAYERS] if fused else None)
+        fn(0)
+        gr = graph_of(fn, 48)
+        acc = []
+        for rep in range(30):
+            gr.replay()
+            torch.cuda.synchronize()
+            buf = np.zeros(256 * 8 * 8, dtype=np.uint64)
+            assert L.tllm_debug_r8_stamps(buf.ctypes.data, buf.nbytes) == 0
+            if rep >= 6:
+                st = buf.reshape(256, 8, 8).astype(np.int64)
+                acc.append((st - st[:, :, 0].min()) * 10.0)       # ns: the counter runs at 100 MHz
+        arr = np.stack(acc)                                        # [replay, workgroup, wavefront, stamp]
+        names = ["wavefront started", "first loads issued", "activations landed",
+                 "other wavefronts' sums seen" if fused else "weight phase 0 landed",
+                 "activations scaled" if fused else "weight phase 3 landed",
+                 "partial tiles written", "epilogue: past the last barrier", "epilogue: before the stores"]
+        table = {}
+        for i, name in enumerate(names):
+            v = arr[:, :, 6:, i] if i >= 6 else (arr[:, :, :6, i] if i > 0 else arr[..., i])
+            table[name] = [round(float(v.min(axis=(1, 2)).mean())), round(float(v.mean())), round(float(v.max(axis=(1, 2)).mean()))]
+        print(json.dumps({"kernel": name_of_stamps(fused), "rows": n, "ns_since_first_wavefront_started_min_mean_max": table}))
+        return 0
     elif kind == "rope":
         rq = torch.empty(1, n, NQ, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         rk = torch.empty(1, n, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
@@ -327,7 +373,7 @@ def main() -> int:
         return e0.elapsed_time(e1) * 1e-3
 
     if args.only:
-        return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg)
+        return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg, _lib)
 
     # ---------------------------------------------------------------- the timed job
     # One sample = EXACTLY --steps steps, captured as one HIP graph and timed with HIP events between two
