@@ -1,0 +1,22 @@
+// Argument block shared by the decode out-projection kernels (out_decode.hip, out_decode_r8.hip).
+#pragma once
+#include "common.h"
+
+namespace tllm {
+
+struct OutArgs {
+  const bf16* x;          // [rows, in_dim]
+  const void* W;          // [out_dim, in_dim] bf16, or fp8 bytes when w_scale != null
+  const float* w_scale;   // [out_dim] or null
+  const bf16* bias;       // [out_dim] or null
+  const bf16* res;        // [rows, out_dim] with row stride res_rs, or null
+  bf16* out;              // [rows, out_dim] with row stride out_rs
+  int64_t res_rs, out_rs;
+  int64_t rows;
+  int in_dim, out_dim;
+};
+
+// in_dim 4096, out_dim % 12 == 0, rows <= 8, bf16 weight; grid = (out_dim / 12)
+void launch_out_decode_r8(dim3 grid, hipStream_t st, const OutArgs& a);
+
+}  // namespace tllm

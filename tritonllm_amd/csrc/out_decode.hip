@@ -2,7 +2,8 @@
 // (out_residual_decode_forward, triton_kernels.py:1470-1517; split-K kernel :1340-1416 + reduce :1419-1467).
 // One launch, no partial-sum workspace; `out` may be the residual buffer itself, as in the reference.
 //
-//   out_decode_cu_kernel    in_dim == 4096, out_dim % 12 == 0 (gpt-oss: [2880, 4096]): the weight-streaming layout
+//   out_decode_r8_kernel    (out_decode_r8.hip) in_dim == 4096, out_dim % 12 == 0, up to 8 rows, bf16 weight
+//   out_decode_cu_kernel    in_dim == 4096, out_dim % 12 == 0 (gpt-oss: [2880, 4096]), more rows or fp8 weight: the weight-streaming layout
 //                           of the decode QKV kernel -- one workgroup per CU-sized share of the output features,
 //                           sixteen wavefronts splitting K, every load unconditional and issued up front, operands
 //                           through wavefront-private LDS patches into v_mfma_f32_32x32x16_bf16, one reduction.
@@ -11,21 +12,9 @@
 // W8: fp8 (OCP e4m3) weight with one fp32 scale per output row, as the reference's ATTN_FP8 option
 // (triton_kernels.py:1385-1408); the values are widened to bf16 (exact) on their way into LDS and the row scale
 // multiplies the finished sum.
-#include "common.h"
+#include "out_common.h"
 
 namespace tllm {
-
-struct OutArgs {
-  const bf16* x;          // [rows, in_dim]
-  const void* W;          // [out_dim, in_dim] bf16, or fp8 bytes when w_scale != null
-  const float* w_scale;   // [out_dim] or null
-  const bf16* bias;       // [out_dim] or null
-  const bf16* res;        // [rows, out_dim] with row stride res_rs, or null
-  bf16* out;              // [rows, out_dim] with row stride out_rs
-  int64_t res_rs, out_rs;
-  int64_t rows;
-  int in_dim, out_dim;
-};
 
 template <int XR, int CH, bool W8>
 __global__ __launch_bounds__(1024) void out_decode_cu_kernel(OutArgs a) {
@@ -230,6 +219,10 @@ extern "C" int tllm_out_residual_decode_bf16(const void* x, const void* W, const
     const int64_t chunks = (rows + xr - 1) / xr;
     TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "out_residual_decode: rows %lld too many for the decode kernel", (long long)rows);
     dim3 grid((unsigned)(out_dim / 12), (unsigned)chunks);
+    if (rows <= 8 && !w8) {
+      launch_out_decode_r8(grid, st, a);
+      return check_launch("out_residual_decode");
+    }
 #define TLLM_OUT(XR, CH)                                                                                   \
   do {                                                                                                     \
     if (w8) hipLaunchKernelGGL((out_decode_cu_kernel<XR, CH, true>), grid, dim3(1024), 0, st, a);         \
