@@ -16,7 +16,7 @@ struct OutArgs {
   int in_dim, out_dim;
 };
 
-// in_dim 4096, out_dim % 12 == 0, rows <= 8, bf16 weight; grid = (out_dim / 12)
+// in_dim 4096, out_dim % 12 == 0, rows <= 8, bf16 weight or (a.w_scale != null) fp8; grid = (out_dim / 12)
 void launch_out_decode_r8(dim3 grid, hipStream_t st, const OutArgs& a);
 
 }  // namespace tllm

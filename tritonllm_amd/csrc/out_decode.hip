@@ -2,8 +2,8 @@
 // (out_residual_decode_forward, triton_kernels.py:1470-1517; split-K kernel :1340-1416 + reduce :1419-1467).
 // One launch, no partial-sum workspace; `out` may be the residual buffer itself, as in the reference.
 //
-//   out_decode_r8_kernel    (out_decode_r8.hip) in_dim == 4096, out_dim % 12 == 0, up to 8 rows, bf16 weight
-//   out_decode_cu_kernel    in_dim == 4096, out_dim % 12 == 0 (gpt-oss: [2880, 4096]), more rows or fp8 weight: the weight-streaming layout
+//   out_decode_r8_kernel    (out_decode_r8.hip) in_dim == 4096, out_dim % 12 == 0, up to 8 rows, bf16 or fp8 weight
+//   out_decode_cu_kernel    in_dim == 4096, out_dim % 12 == 0 (gpt-oss: [2880, 4096]), more rows: the weight-streaming layout
 //                           of the decode QKV kernel -- one workgroup per CU-sized share of the output features,
 //                           sixteen wavefronts splitting K, every load unconditional and issued up front, operands
 //                           through wavefront-private LDS patches into v_mfma_f32_32x32x16_bf16, one reduction.
@@ -219,7 +219,7 @@ extern "C" int tllm_out_residual_decode_bf16(const void* x, const void* W, const
     const int64_t chunks = (rows + xr - 1) / xr;
     TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "out_residual_decode: rows %lld too many for the decode kernel", (long long)rows);
     dim3 grid((unsigned)(out_dim / 12), (unsigned)chunks);
-    if (rows <= 8 && !w8) {
+    if (rows <= 8) {
       launch_out_decode_r8(grid, st, a);
       return check_launch("out_residual_decode");
     }

@@ -1,4 +1,4 @@
-// Decode-size attention out-projection + bias + residual for in_dim == 4096 and up to 8 activation rows (bf16 weight):
+// Decode-size attention out-projection + bias + residual for in_dim == 4096 and up to 8 activation rows (bf16 or fp8 weight):
 //   out[r, n] = sum_k x[r, k] * W[n, k] + b[n] + res[r, n]        (out_residual_decode_forward, triton_kernels.py:1470-1517)
 // in the weight-streaming form of qkv_decode_r8.hip:
 //   * one workgroup per twelve output features (gpt-oss: 240 workgroups, one per CU -- it needs most of a CU's LDS),
@@ -17,6 +17,10 @@
 //   * a ninth wavefront loads bias and residual while the stream runs, then adds the eight partial tiles in a fixed
 //     order and stores four adjacent features of a row per lane (8-byte stores where the alignment allows).
 // `out` may be the residual buffer itself: an element is read and written by the same lane.
+// W8: fp8 (OCP e4m3) weight with one fp32 scale per output row (the reference's ATTN_FP8 option,
+// triton_kernels.py:1385-1408): a wavefront's 512 bytes of a row arrive in two phases of eight k32 steps (256-byte
+// pieces again, the same LDS layout), fragments are widened to bf16 (exact) between the LDS read and the MFMA, the row
+// scale multiplies the finished sum.
 #include "out_common.h"
 
 namespace tllm {
@@ -30,8 +34,13 @@ constexpr int REGION = RW * 256;  // one phase: twelve weight rows x four k32 st
 constexpr int XBLOCK = 1024;      // one activation row of a slice: 64 chunks of 16 bytes
 }  // namespace r8o
 
+template <bool W8>
 __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8) {
   using namespace r8o;
+  constexpr int NPH = W8 ? 2 : 4;                           // phases of PSTEPS k32 steps
+  constexpr int PSTEPS = 16 / NPH;
+  constexpr int RPH = W8 ? 2 : RING;                        // phases that land in the ring (the last bf16 phase lands in the activation blocks)
+  constexpr int WPITCH = W8 ? 4096 : 8192;                  // bytes per weight row
   __shared__ __align__(1024) unsigned char xw[NS * XR * XBLOCK];
   __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
 
@@ -77,6 +86,12 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
       if (!a.bias) bv[i] = 0.f;
       if (!a.res) rv[i] = 0.f;
     }
+    float ws[4] = {1.f, 1.f, 1.f, 1.f};                    // W8: the row scales of the lane's four features
+    if constexpr (W8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ws[i] = a.w_scale[efeat + i];
+      asm volatile("" : "+v"(ws[0]), "+v"(ws[1]), "+v"(ws[2]), "+v"(ws[3]));
+    }
     unsigned red_o = static_cast<unsigned>(REGION + lane * 16);
     // one wavefront runs alone from the barrier to the stores: everything that does not need the sums exists before it
     asm volatile("" : "+v"(bv[0]), "+v"(bv[1]), "+v"(bv[2]), "+v"(bv[3]), "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]), "+v"(out), "+v"(red_o));
@@ -95,7 +110,7 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
     if (!evalid) return;
     bf16x4 o;                                               // features efeat .. efeat + 3 of row en
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] + bv[i] + rv[i]);
+    for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] * ws[i] + bv[i] + rv[i]);
     if (vec8) {
       *reinterpret_cast<bf16x4*>(out) = o;
     } else {
@@ -111,7 +126,8 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
   unsigned char* myx = xw + wave * (XR * XBLOCK);
   unsigned char* myring = ring + wave * (RING * REGION);
   // byte offset inside a bf16 row of this wavefront's 16-byte chunk c (0..63): phase c / 16, chunk c % 16 of its 256 bytes
-  auto kb = [&](int c) { return (c >> 4) * 2048 + kq * 256 + (c & 15) * 16; };
+  // (of an activation row; with the fp8 weight a phase is eight steps: phase c / 32, chunk c % 32 of its 512 bytes)
+  auto kb = [&](int c) { return W8 ? (c >> 5) * 4096 + kq * 512 + (c & 31) * 16 : (c >> 4) * 2048 + kq * 256 + (c & 15) * 16; };
 
   // activations: row n of the slice -> 1 KB block n; lane i fetches chunk i ^ 2n, the swizzle that spreads the eight
   // rows of a fragment read over the banks
@@ -127,7 +143,7 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
   for (int j = 0; j < 3; ++j) {
     const int r = 4 * j + (lane >> 4);
     const int cc = (lane & 15) ^ r;
-    goff[j] = static_cast<unsigned>(n0 + r) * 8192u + kq * 256u + cc * 16u;
+    goff[j] = static_cast<unsigned>(n0 + r) * static_cast<unsigned>(WPITCH) + kq * 256u + cc * 16u;
   }
   const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
@@ -149,33 +165,53 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
   }
 #pragma unroll
-  for (int p = 0; p < RING; ++p) issue_phase(p);
+  for (int p = 0; p < RPH; ++p) issue_phase(p);
 
   // ---- activation fragments into registers (the weight loads are younger and stay outstanding)
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RING * 3) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPH * 3) : "memory");
   bf16x8 fb[16];
 #pragma unroll
   for (int s = 0; s < 16; ++s) fb[s] = *reinterpret_cast<const bf16x8*>(myx + m1 * XBLOCK + (((4 * s + g) ^ (2 * m1)) << 4));
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the activation blocks are free from here on
-  issue_phase(3);
+  if constexpr (NPH > RPH) issue_phase(NPH - 1);
 
   // ---- the stream: phase by phase out of LDS into the matrix core
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   const int arow = m < RW ? m : m - RW;                     // tile rows past the twelfth re-read a real one (their sums are dropped)
   const unsigned a_o = arow * 256;
+  // W8: the lane's eight fp8 of step st are bytes 32 st + 8 g of the row's 256-byte piece: half g & 1 of chunk
+  // 2 st + g / 2, which sits at position chunk ^ row
+  auto w8frag = [&](const unsigned char* reg, int st) {
+    typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+    typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+    const u32x2 raw = *reinterpret_cast<const u32x2*>(reg + a_o + (((2 * st + (g >> 1)) ^ arow) << 4) + (g & 1) * 8);
+    u32x4 o;
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    // three loads per phase, all four phases requested by now: phase p has landed when 3 * (3 - p) are outstanding
-    if (p == 0) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-    else if (p == 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-    else if (p == 2) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int d = 0; d < 2; ++d) {
+      const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
+      // e4m3 -> fp32 has at most four significant bits: the upper halves are the bf16 values, exactly
+      o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
+      o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
+    }
+    return __builtin_bit_cast(bf16x8, o);
+  };
+#pragma unroll
+  for (int p = 0; p < NPH; ++p) {
+    // three loads per phase, every phase requested by now: phase p has landed when 3 * (NPH - 1 - p) are outstanding
+    if (p == NPH - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (p == NPH - 2) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    else if (p == NPH - 3) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     const unsigned char* reg = phase_region(p);
-    bf16x8 fa[4];
+    bf16x8 fa[PSTEPS];
 #pragma unroll
-    for (int st = 0; st < 4; ++st) fa[st] = *reinterpret_cast<const bf16x8*>(reg + a_o + (((4 * st + g) ^ arow) << 4));
+    for (int st = 0; st < PSTEPS; ++st) {
+      if constexpr (W8) fa[st] = w8frag(reg, st);
+      else fa[st] = *reinterpret_cast<const bf16x8*>(reg + a_o + (((4 * st + g) ^ arow) << 4));
+    }
 #pragma unroll
-    for (int st = 0; st < 4; ++st) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[st], fb[4 * p + st], acc, 0, 0, 0);
+    for (int st = 0; st < PSTEPS; ++st) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[st], fb[PSTEPS * p + st], acc, 0, 0, 0);
   }
 
   // ---- partial tile -> LDS (the wavefront's own region 1, long since consumed), then the epilogue wavefront takes over
@@ -186,7 +222,8 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
 void launch_out_decode_r8(dim3 grid, hipStream_t st, const OutArgs& a) {
   auto al8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
   const int vec8 = al8(a.out) && a.out_rs % 4 == 0 && (a.res == nullptr || (al8(a.res) && a.res_rs % 4 == 0)) && (a.bias == nullptr || al8(a.bias));
-  hipLaunchKernelGGL(out_decode_r8_kernel, grid, dim3(576), 0, st, a, vec8);
+  if (a.w_scale) hipLaunchKernelGGL(out_decode_r8_kernel<true>, grid, dim3(576), 0, st, a, vec8);
+  else hipLaunchKernelGGL(out_decode_r8_kernel<false>, grid, dim3(576), 0, st, a, vec8);
 }
 
 }  // namespace tllm

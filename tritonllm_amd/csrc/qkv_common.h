@@ -53,7 +53,7 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
 // Any hidden size, any even head_dim: one workgroup per (head, row); each wavefront takes
 // rotation pairs (d, d + hd/2) in turn and reduces the two dot products by shuffle.
 // The hidden-2880 decode kernel for up to 8 rows per workgroup, bf16 weight (qkv_decode_r8.hip).
-void launch_qkv_decode_r8(int norm, bool emb, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
+void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 // ... and for 9..32 rows per workgroup, activations already normalised (qkv_decode_r32.hip).
 void launch_qkv_decode_r32(dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 

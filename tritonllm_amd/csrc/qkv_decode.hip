@@ -630,7 +630,7 @@ static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, 
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
   const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
   if (r32) launch_qkv_decode_r32(grid, st, a, ra, fr);
-  else if (xr == 8 && !w8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, grid, st, a, ra, fr);
+  else if (xr == 8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, w8, grid, st, a, ra, fr);
   else if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
   else launch_cu(xr, norm, w8, grid, st, a, ra, fr);
   return check_launch(what);

@@ -31,6 +31,10 @@
 // fp32 arithmetic, one rounding to bf16: the operand the separate rmsnorm launch would hand over.
 // EMB: the activation rows are gathered from an embedding table by token id (model.py:906-920 feeding the first
 // block); workgroup 0 also writes the gathered rows out. An id outside the table gives a zero row and raises the flag.
+// W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (triton_kernels.py:261-268, 927-965). A
+// wavefront's 480 bytes of a row arrive in two phases of 8 + 7 k32 steps (256 + 224 bytes, so a row piece is as long
+// as in the bf16 form and the LDS layout is the same), fragments are widened to bf16 (exact) between the LDS read and
+// the MFMA, the row scale multiplies the finished sum.
 #include "qkv_common.h"
 
 namespace tllm {
@@ -53,10 +57,14 @@ __device__ unsigned long long g_r8_stamps[256 * 8 * 8];
 #define R8_STAMP(i) do { } while (0)
 #endif
 
-template <int NORM, bool EMB>
+template <int NORM, bool EMB, bool W8>
 __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int out4) {
   using namespace r8;
   static_assert(!EMB || NORM != 0, "the fused gather exists with the fused norm only");
+  constexpr int LPW = 5;                                    // weight load instructions per phase and wavefront
+  constexpr int NPH = W8 ? 2 : 4;                           // phases: bf16 4 + 4 + 4 + 3 k32 steps, fp8 8 + 7
+  constexpr int PSTEPS = W8 ? 8 : 4;                        // k32 steps of a full phase
+  constexpr int RPH = W8 ? 2 : RING;                        // phases that land in the ring (the last bf16 phase lands in the activation blocks)
   __shared__ __align__(1024) unsigned char xw[NS * XR * XBLOCK];
   __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
   __shared__ __align__(1024) unsigned char scw[NORM ? NS * 2048 : 16];
@@ -92,6 +100,14 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     const unsigned b_lo = bias_ptr[(ehead * 64 + ed) >> 1];
     const unsigned b_hi = bias_ptr[(ehead * 64 + 32 + ed) >> 1];
     const float freq0 = fr.v[ed], freq1 = fr.v[ed + 1];
+    float ws_l0 = 1.f, ws_l1 = 1.f, ws_h0 = 1.f, ws_h1 = 1.f;   // W8: the row scales of the lane's four weight rows
+    if constexpr (W8) {
+      const float* sp = a.w_scale + ehead * 64 + ed;        // 4-byte aligned is all the interface asks for
+      ws_l0 = sp[0];
+      ws_l1 = sp[1];
+      ws_h0 = sp[32];
+      ws_h1 = sp[33];
+    }
     float cs0 = 1.f, sn0 = 0.f, cs1 = 1.f, sn1 = 0.f;
     const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
     if (erot) {
@@ -114,6 +130,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     }
     bf16* out = qkv_out_ptr(a, slot, erow, ehead) + ed;
     unsigned red_o = static_cast<unsigned>(REGION + tile * 1024 + lane * 16);
+    if constexpr (W8) asm volatile("" : "+v"(ws_l0), "+v"(ws_l1), "+v"(ws_h0), "+v"(ws_h1));
     // One wavefront runs alone from the last barrier to the stores, so every instruction after that barrier is
     // latency: all of the above is forced to exist here (left to itself the compiler moves it to its first use,
     // behind the barrier).
@@ -132,6 +149,12 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
       acc[3] += t[w][3];
     }
     if (!evalid) return;
+    if constexpr (W8) {
+      acc[0] *= ws_l0;
+      acc[1] *= ws_l1;
+      acc[2] *= ws_h0;
+      acc[3] *= ws_h1;
+    }
     float lo0 = acc[0] + bl0, lo1 = acc[1] + bl1, hi0 = acc[2] + bh0, hi1 = acc[3] + bh1;   // [lo(d), lo(d+1), hi(d), hi(d+1)] of row en
     if (erot) {
       const float r0 = lo0 * cs0 - hi0 * sn0, r2 = hi0 * cs0 + lo0 * sn0;
@@ -165,7 +188,12 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // together read 24 consecutive k32 steps (1536 contiguous bytes of every weight row), wavefront kq steps
   // 24 p + 4 kq .. + 4; in phase 3, 18 steps, wavefront kq steps 72 + 3 kq .. + 3. What a CU requests within a short
   // time is then contiguous in memory. kb(c): byte offset inside a bf16 row of this wavefront's 16-byte chunk c (0..59).
-  auto kb = [&](int c) { return c < 48 ? (c >> 4) * 1536 + kq * 256 + (c & 15) * 16 : 4608 + kq * 192 + (c - 48) * 16; };
+  // (With the fp8 weight the phases are 8 + 7 steps: 48 steps = 3072 bytes of an activation row, wavefront kq the 512
+  // at kq * 512, then 42 steps, wavefront kq the 448 bytes at 3072 + kq * 448.)
+  auto kb = [&](int c) {
+    if constexpr (W8) return c < 32 ? kq * 512 + c * 16 : 3072 + kq * 448 + (c - 32) * 16;
+    else return c < 48 ? (c >> 4) * 1536 + kq * 256 + (c & 15) * 16 : 4608 + kq * 192 + (c - 48) * 16;
+  };
   const int m = lane & 15, g = lane >> 4, m1 = m & 7;
   unsigned char* myx = xw + wave * (XR * XBLOCK);
   unsigned char* myring = ring + wave * (RING * REGION);
@@ -204,9 +232,9 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     }
   }
   // weight: lane -> (row r4 of a 4-row block, position pos): it fetches chunk pos ^ (tile row & 15) of that row
-  unsigned goff[5], goff3[5];                               // phases 0-2 / the three-step phase 3 (chunks 0..11 only)
+  unsigned goff[LPW], goff3[LPW];                           // full phases / the short last phase (bf16: chunks 0..11 only, fp8: 0..13)
 #pragma unroll
-  for (int j = 0; j < 5; ++j) {
+  for (int j = 0; j < LPW; ++j) {
     const int row20 = 4 * j + (lane >> 4);                  // 0..11 tile 0, 12..19 tile 1
     const int tile = row20 >= 12, trow = tile ? row20 - 12 : row20;
     const int quad = trow >> 2, q = trow & 3;
@@ -214,8 +242,13 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     gp = gp < total_pairs ? gp : total_pairs - 1;
     const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + ((q & 2) ? 32u : 0u);
     const int cc = (lane & 15) ^ (trow & 15);
-    goff[j] = wrow * 5760u + kq * 256u + cc * 16u;
-    goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
+    if constexpr (W8) {                                     // a chunk is 16 fp8; a full phase is again 256 bytes per row and wavefront
+      goff[j] = wrow * 2880u + kq * 256u + cc * 16u;
+      goff3[j] = wrow * 2880u + kq * 224u + (cc < 14 ? cc : 13) * 16u;
+    } else {
+      goff[j] = wrow * 5760u + kq * 256u + cc * 16u;
+      goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
+    }
   }
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
@@ -223,11 +256,11 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // as the activation fragments are in registers -- so no weight load ever waits for an MFMA.
   auto phase_region = [&](int p) -> unsigned char* { return p < RING ? myring + p * REGION : myx; };
   auto issue_phase = [&](int p) {
-    const unsigned char* sb = wbase + (p < 3 ? p * 1536 : 4608);
+    const unsigned char* sb = wbase + p * 1536;            // the six wavefronts' pieces of a full phase: 6 x 256 bytes of every row
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {
+    for (int j = 0; j < LPW; ++j) {
       const unsigned dst = lds_addr(phase_region(p) + j * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == 3 ? goff3[j] : goff[j]), "s"(sb) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == NPH - 1 ? goff3[j] : goff[j]), "s"(sb) : "memory", "m0");
     }
   };
 
@@ -256,7 +289,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // would hold the others up at the barrier: so all activation loads go first (the rendezvous puts them at the head
   // of the CU's queue, which returns loads in the order it took them), one phase of weight keeps the memory system
   // busy meanwhile, and the other three phases are requested after the norm.
-  constexpr int EARLY = NORM != 0 ? 1 : RING;
+  constexpr int EARLY = NORM != 0 ? 1 : RPH;
   if constexpr (NORM != 0) {
     if (lane == 0) s_flag[wave] = 0;
     __syncthreads();
@@ -266,7 +299,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   R8_STAMP(1);
 
   // ---- activation fragments into registers (the weight loads issued so far are younger and stay outstanding)
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(EARLY * 5) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(EARLY * LPW) : "memory");
   R8_STAMP(2);
   bf16x8 fb[STEPS];
   auto xfrag = [&](int s) { return *reinterpret_cast<const bf16x8*>(myx + m1 * XBLOCK + (((4 * s + g) ^ (2 * m1)) << 4)); };
@@ -274,7 +307,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) fb[s] = xfrag(s);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    issue_phase(3);
+    if constexpr (NPH > RPH) issue_phase(NPH - 1);
   } else {
     // Columns 8..15 of the MFMA are never stored, so lanes m >= 8 are free to do half of the norm's arithmetic: a
     // lane fetches and scales the fragments of the steps of its own parity (h = bit 3 of the lane), and the lanes
@@ -325,7 +358,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the loads in flight are none of its business
     if (lane == 0) __hip_atomic_store(&s_flag[wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #pragma unroll
-    for (int p = EARLY; p < 4; ++p) issue_phase(p);
+    for (int p = EARLY; p < NPH; ++p) issue_phase(p);
     for (;;) {                                              // every streaming wavefront raises its flag before it gets here or exits
       const unsigned f = lane < NS ? __hip_atomic_load(&s_flag[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : 1u;
       if (__all(f != 0u)) break;
@@ -382,28 +415,49 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
   const int arow0 = m < 12 ? m : m - 12;                    // tile rows past the last real one re-read a real one (their sums are dropped)
   const unsigned a0_o = arow0 * 256, a1_o = (12 + m1) * 256;
+  // W8: the lane's eight fp8 of step st are bytes 32 st + 8 g of the row's 256-byte piece: half g & 1 of chunk
+  // 2 st + g / 2, which sits at position chunk ^ (tile row & 15)
+  auto w8frag = [&](const unsigned char* reg, unsigned row_o, int trow, int st) {
+    typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+    typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+    const u32x2 raw = *reinterpret_cast<const u32x2*>(reg + row_o + (((2 * st + (g >> 1)) ^ trow) << 4) + (g & 1) * 8);
+    u32x4 o;
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    // five loads per phase, all four phases requested by now: phase p has landed when 5 * (3 - p) are outstanding
-    if (p == 0) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-    else if (p == 1) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-    else if (p == 2) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int d = 0; d < 2; ++d) {
+      const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
+      // e4m3 -> fp32 has at most four significant bits: the upper halves are the bf16 values, exactly
+      o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
+      o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
+    }
+    return __builtin_bit_cast(bf16x8, o);
+  };
+#pragma unroll
+  for (int p = 0; p < NPH; ++p) {
+    // LPW loads per phase, every phase requested by now: phase p has landed when LPW * (NPH - 1 - p) are outstanding
+    if (p == NPH - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (p == NPH - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPW) : "memory");
+    else if (p == NPH - 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPW) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPW) : "memory");
     if (NORM == 0 && p == 0) R8_STAMP(3);
-    if (NORM == 0 && p == 3) R8_STAMP(4);
+    if (NORM == 0 && p == NPH - 1) R8_STAMP(4);
     const unsigned char* reg = phase_region(p);
-    constexpr int kMaxSt = 4;
-    bf16x8 fa0[kMaxSt], fa1[kMaxSt];
-    const int nst = p == 3 ? 3 : 4;
+    bf16x8 fa0[PSTEPS], fa1[PSTEPS];
+    const int nst = p == NPH - 1 ? PSTEPS - 1 : PSTEPS;
 #pragma unroll
     for (int st = 0; st < nst; ++st) {                      // all fragment reads of the phase in one go, then its MFMAs
-      fa0[st] = *reinterpret_cast<const bf16x8*>(reg + a0_o + (((4 * st + g) ^ arow0) << 4));
-      fa1[st] = *reinterpret_cast<const bf16x8*>(reg + a1_o + (((4 * st + g) ^ m1) << 4));
+      if constexpr (W8) {
+        fa0[st] = w8frag(reg, a0_o, arow0, st);
+        fa1[st] = w8frag(reg, a1_o, m1, st);
+      } else {
+        fa0[st] = *reinterpret_cast<const bf16x8*>(reg + a0_o + (((4 * st + g) ^ arow0) << 4));
+        fa1[st] = *reinterpret_cast<const bf16x8*>(reg + a1_o + (((4 * st + g) ^ m1) << 4));
+      }
     }
 #pragma unroll
     for (int st = 0; st < nst; ++st) {
-      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[st], fb[4 * p + st], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[st], fb[4 * p + st], acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[st], fb[PSTEPS * p + st], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[st], fb[PSTEPS * p + st], acc1, 0, 0, 0);
     }
   }
 
@@ -414,12 +468,16 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   __syncthreads();
 }
 
-// Host side: pick the instantiation. norm = 0 / 1 (fp32 scale) / 2 (bf16 scale).
-void launch_qkv_decode_r8(int norm, bool emb, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+// Host side: pick the instantiation. norm = 0 / 1 (fp32 scale) / 2 (bf16 scale); w8: fp8 weight with a.w_scale.
+void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
   auto even = [](int64_t v) { return (v & 1) == 0; };
   const int out4 = (reinterpret_cast<uintptr_t>(a.q) % 4 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 4 == 0) &&
                    (reinterpret_cast<uintptr_t>(a.v) % 4 == 0) && even(a.q_rs) && even(a.k_rs) && even(a.v_rs) && even(a.kv_slot_stride);
-#define TLLM_R8(NORM, EMBF) hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF>), grid, dim3(512), 0, st, a, ra, fr, out4)
+#define TLLM_R8(NORM, EMBF)                                                                                               \
+  do {                                                                                                                    \
+    if (w8) hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF, true>), grid, dim3(512), 0, st, a, ra, fr, out4);        \
+    else hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF, false>), grid, dim3(512), 0, st, a, ra, fr, out4);          \
+  } while (0)
   if (emb) {
     if (norm == 1) TLLM_R8(1, true);
     else TLLM_R8(2, true);
