@@ -110,7 +110,7 @@ def host_cpu_info() -> dict:
 
 
 def name_of_stamps(fused: bool) -> str:
-    return "qkv_decode_r8_kernel<2,false>" if fused else "qkv_decode_r8_kernel<0,false>"
+    return "qkv_decode_r8_kernel<2,false,false>" if fused else "qkv_decode_r8_kernel<0,false,false>"
 
 
 def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg, _lib) -> int:
@@ -404,13 +404,13 @@ def main() -> int:
         dominant = lambda i: T.qkv_rope_forward(t, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn,
                                                 positions=positions, mode="decode", out=(q, k, v))
         qkv_bytes = bytes_of["qkv"](B)
-        kernel_name = "qkv_decode_r8_kernel<0,false> (QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
+        kernel_name = "qkv_decode_r8_kernel<0,false,false> (QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
     else:
         dominant = lambda i: T.qkv_rope_forward(x, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD, yarn=yarn,
                                                 positions=positions, mode="decode", out=(q, k, v),
                                                 norm_scale=scales[i % N_LAYERS], norm_eps=1e-5)
         qkv_bytes = bytes_of["norm_qkv"](B)
-        kernel_name = "qkv_decode_r8_kernel<2,false> (RMSNorm + QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
+        kernel_name = "qkv_decode_r8_kernel<2,false,false> (RMSNorm + QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
     qkv_graph = graph_of(dominant, n_launch)
     qkv_graph.replay()
     qkv_s = min(time_graph(qkv_graph) for _ in range(5)) / n_launch
