@@ -161,8 +161,12 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
   // ---- every load of this wavefront, oldest first: activations, then the weight
 #pragma unroll
   for (int n = 0; n < XR; ++n) {
-    const unsigned dst = lds_addr(myx + n * XBLOCK);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+    // Rows past the last one are not fetched: their LDS blocks keep whatever they held, and what the MFMA makes of
+    // that stays in output columns nobody stores. Fewer loads ahead of a wait only make it less strict than written.
+    if (n < nvalid) {
+      const unsigned dst = lds_addr(myx + n * XBLOCK);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+    }
   }
 #pragma unroll
   for (int p = 0; p < RPH; ++p) issue_phase(p);

@@ -24,7 +24,6 @@ constexpr int RING = 2;           // resident phases per wavefront
 constexpr int XPH = 8 * 1024;     // activations of one phase: 32 rows x four k32 steps
 constexpr int WPH = 5 * 1024;     // weight of one phase: 20 rows x four k32 steps
 constexpr int REGION = XPH + WPH;
-constexpr int LPP = 13;           // load instructions per phase
 }  // namespace r32
 
 __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int out4) {
@@ -121,6 +120,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
 
   // ========================================================================= streaming wavefront of K slice `kq`
   const int kq = wave;
+  const int xblocks = (nvalid + 3) >> 2;                    // four-row activation blocks that hold a real row
   const int m = lane & 15, g = lane >> 4, m1 = m & 7;
   unsigned char* myring = ring + wave * (RING * REGION);
 
@@ -158,8 +158,13 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     const unsigned char* wb = wbase + (p < 3 ? p * 1536 : 4608);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const unsigned dst = lds_addr(reg + j * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(p == 3 ? xoff3[j] : xoff[j]), "s"(xb) : "memory", "m0");
+      // Four-row blocks past the last row are not fetched: their LDS keeps whatever it held, and what the MFMA makes
+      // of that stays in output columns nobody stores (a column depends on its own activation row only)
+      // (the waits below count the loads of the phase after the one they wait for, so they depend on xblocks).
+      if (j < xblocks) {
+        const unsigned dst = lds_addr(reg + j * 1024);
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(p == 3 ? xoff3[j] : xoff[j]), "s"(xb) : "memory", "m0");
+      }
     }
 #pragma unroll
     for (int j = 0; j < 5; ++j) {
@@ -182,8 +187,21 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     // phase p has landed when only the loads of the phase after it (if requested) are outstanding
-    if (p < 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPP) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (p < 3) {
+      // s_waitcnt takes an immediate: one case per number of activation blocks a phase fetches (xblocks + 5 loads)
+      switch (xblocks) {
+        case 1: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+        case 5: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
+        case 7: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(13)" ::: "memory"); break;
+      }
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     const unsigned char* reg = myring + (p % RING) * REGION;
     const int nst = p == 3 ? 3 : 4;
     bf16x8 fa0[4], fa1[4], fb0[4], fb1[4];

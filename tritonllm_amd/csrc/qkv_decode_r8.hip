@@ -267,8 +267,13 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // ---- every load of this wavefront, oldest first: activations, norm scale, then the weight
 #pragma unroll
   for (int n = 0; n < XR; ++n) {
-    const unsigned dst = lds_addr(myx + n * XBLOCK);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+    // Rows past the last one are not fetched: their LDS blocks keep whatever they held, and what the MFMA makes of
+    // that stays in output columns nobody stores (a column depends on its own activation row only). Fewer loads ahead
+    // of a wait only make it less strict than written: the counts below are relative to the youngest loads.
+    if (n < nvalid) {
+      const unsigned dst = lds_addr(myx + n * XBLOCK);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+    }
   }
   constexpr int NSC = NORM == 1 ? 2 : (NORM == 2 ? 1 : 0);   // scale loads: 480 fp32 = 120 chunks, 480 bf16 = 60 chunks
   if constexpr (NORM != 0) {
