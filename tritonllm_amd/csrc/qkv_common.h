@@ -55,7 +55,7 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
 // The hidden-2880 decode kernel for up to 8 rows per workgroup, bf16 weight (qkv_decode_r8.hip).
 void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 // ... and for 9..32 rows per workgroup, activations already normalised (qkv_decode_r32.hip).
-void launch_qkv_decode_r32(dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
+void launch_qkv_decode_r32(bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 
 void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, hipStream_t st);
 

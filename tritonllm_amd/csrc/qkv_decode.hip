@@ -624,12 +624,12 @@ static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, 
   TLLM_REQUIRE(static_cast<int64_t>(heads) * 64 * 2880 < (1ll << 31), TLLM_E_SHAPE, "%s: weight too large", what);
   // the activations are addressed with 32-bit byte offsets in the two kernels that load straight into LDS
   const bool fits32 = (a.emb_ids ? a.emb_vocab : rows) * 5760 < (1ll << 32);
-  const bool r32 = rows > 8 && !w8 && norm == 0 && !a.emb_ids && fits32;   // 9..32 rows per workgroup, normalised activations
+  const bool r32 = rows > 8 && norm == 0 && !a.emb_ids && fits32;          // 9..32 rows per workgroup, normalised activations
   const int xr = rows <= 8 ? 8 : ((rows <= 16 && !r32) ? 16 : 32);
   const int64_t chunks = (rows + xr - 1) / xr;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
   const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
-  if (r32) launch_qkv_decode_r32(grid, st, a, ra, fr);
+  if (r32) launch_qkv_decode_r32(w8, grid, st, a, ra, fr);
   else if (xr == 8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, w8, grid, st, a, ra, fr);
   else if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
   else launch_cu(xr, norm, w8, grid, st, a, ra, fr);

@@ -11,6 +11,9 @@
 // a ring of two 13 KB regions per wavefront; a phase is multiplied (two tiles x two column blocks of 16 rows) as soon
 // as it has landed and its region is then refilled with the phase after next. Four epilogue wavefronts, one per
 // (tile, column block).
+// W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (triton_kernels.py:261-268, 927-965): a phase of
+// weight is 20 rows x 128 bytes (three loads of eight rows), fragments are widened to bf16 (exact) between the LDS
+// read and the MFMA, the row scale multiplies the finished sum.
 #include "qkv_common.h"
 
 namespace tllm {
@@ -26,8 +29,10 @@ constexpr int WPH = 5 * 1024;     // weight of one phase: 20 rows x four k32 ste
 constexpr int REGION = XPH + WPH;
 }  // namespace r32
 
+template <bool W8>
 __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int out4) {
   using namespace r32;
+  constexpr int LW = W8 ? 3 : 5;                            // weight load instructions per phase
   __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -55,6 +60,14 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     const unsigned b_lo = bias_ptr[(ehead * 64 + ed) >> 1];
     const unsigned b_hi = bias_ptr[(ehead * 64 + 32 + ed) >> 1];
     const float freq0 = fr.v[ed], freq1 = fr.v[ed + 1];
+    float ws_l0 = 1.f, ws_l1 = 1.f, ws_h0 = 1.f, ws_h1 = 1.f;   // W8: the row scales of the lane's four weight rows
+    if constexpr (W8) {
+      const float* sp = a.w_scale + ehead * 64 + ed;
+      ws_l0 = sp[0];
+      ws_l1 = sp[1];
+      ws_h0 = sp[32];
+      ws_h1 = sp[33];
+    }
     float cs0 = 1.f, sn0 = 0.f, cs1 = 1.f, sn1 = 0.f;
     const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
     if (erot) {
@@ -79,6 +92,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     unsigned red_o = static_cast<unsigned>((2 * tile + cb) * 1024 + lane * 16);
     // everything that does not need the sums exists before the barrier (see qkv_decode_r8.hip)
     asm volatile("" : "+v"(cs0), "+v"(sn0), "+v"(cs1), "+v"(sn1), "+v"(bl0), "+v"(bl1), "+v"(bh0), "+v"(bh1), "+v"(out), "+v"(red_o));
+    if constexpr (W8) asm volatile("" : "+v"(ws_l0), "+v"(ws_l1), "+v"(ws_h0), "+v"(ws_h1));
     __syncthreads();                                        // partial tiles are in LDS
     f32x4 t[NS];
 #pragma unroll
@@ -92,6 +106,12 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
       acc[3] += t[w][3];
     }
     if (!evalid) return;
+    if constexpr (W8) {
+      acc[0] *= ws_l0;
+      acc[1] *= ws_l1;
+      acc[2] *= ws_h0;
+      acc[3] *= ws_h1;
+    }
     float lo0 = acc[0] + bl0, lo1 = acc[1] + bl1, hi0 = acc[2] + bh0, hi1 = acc[3] + bh1;   // [lo(d), lo(d+1), hi(d), hi(d+1)] of row en
     if (erot) {
       const float r0 = lo0 * cs0 - hi0 * sn0, r2 = hi0 * cs0 + lo0 * sn0;
@@ -126,7 +146,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
 
   // lane -> (row r4 of a 4-row block, position pos): it fetches chunk pos ^ (row & 15) of that row, so that the 16 rows
   // a fragment read touches lie in 16 different bank groups. Phase 3 has three steps: chunks 0..11 only.
-  unsigned xoff[8], xoff3[8], goff[5], goff3[5];
+  unsigned xoff[8], xoff3[8], goff[LW], goff3[LW];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int r = 4 * j + (lane >> 4);
@@ -136,16 +156,25 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     xoff3[j] = static_cast<unsigned>(src * 5760 + kq * 192 + (cc < 12 ? cc : 11) * 16);
   }
 #pragma unroll
-  for (int j = 0; j < 5; ++j) {
-    const int row20 = 4 * j + (lane >> 4);                  // 0..11 tile 0, 12..19 tile 1
+  // (W8: a weight row of a phase is 128 bytes = 8 chunks of 16 fp8 and a load covers eight rows: lane -> row
+  // 8 j + lane / 8, position lane % 8, chunk position ^ (row & 7); rows 20..23 of the third load repeat row 19, unread)
+  for (int j = 0; j < LW; ++j) {
+    int row20 = W8 ? 8 * j + (lane >> 3) : 4 * j + (lane >> 4);   // 0..11 tile 0, 12..19 tile 1
+    row20 = row20 < 20 ? row20 : 19;
     const int tile = row20 >= 12, trow = tile ? row20 - 12 : row20;
     const int quad = trow >> 2, q = trow & 3;
     int gp = pair0 + (tile ? 6 : 0) + 2 * quad + (q & 1);
     gp = gp < total_pairs ? gp : total_pairs - 1;
     const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + ((q & 2) ? 32u : 0u);
-    const int cc = (lane & 15) ^ (trow & 15);
-    goff[j] = wrow * 5760u + kq * 256u + cc * 16u;
-    goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
+    if constexpr (W8) {
+      const int cc = (lane & 7) ^ (row20 & 7);
+      goff[j] = wrow * 2880u + kq * 128u + cc * 16u;
+      goff3[j] = wrow * 2880u + kq * 96u + (cc < 6 ? cc : 5) * 16u;
+    } else {
+      const int cc = (lane & 15) ^ (trow & 15);
+      goff[j] = wrow * 5760u + kq * 256u + cc * 16u;
+      goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
+    }
   }
   const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
@@ -155,7 +184,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     // phase p < 3: the six wavefronts together take 24 consecutive k32 steps (1536 contiguous bytes of every row),
     // wavefront kq steps 24 p + 4 kq .. + 4; phase 3: 18 steps, wavefront kq steps 72 + 3 kq .. + 3
     const unsigned char* xb = xbase + (p < 3 ? p * 1536 : 4608);
-    const unsigned char* wb = wbase + (p < 3 ? p * 1536 : 4608);
+    const unsigned char* wb = wbase + (p < 3 ? p * 1536 : 4608) / (W8 ? 2 : 1);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       // Four-row blocks past the last row are not fetched: their LDS keeps whatever it held, and what the MFMA makes
@@ -167,7 +196,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
       }
     }
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {
+    for (int j = 0; j < LW; ++j) {
       const unsigned dst = lds_addr(reg + XPH + j * 1024);
       asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == 3 ? goff3[j] : goff[j]), "s"(wb) : "memory", "m0");
     }
@@ -182,21 +211,40 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     for (int c = 0; c < 2; ++c) acc[t][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int arow0 = m < 12 ? m : m - 12;                    // tile rows past the last real one re-read a real one (their sums are dropped)
-  const unsigned a0_o = XPH + arow0 * 256, a1_o = XPH + (12 + m1) * 256;
+  const unsigned a0_o = XPH + arow0 * (W8 ? 128 : 256), a1_o = XPH + (12 + m1) * (W8 ? 128 : 256);
+  // W8: the lane's eight fp8 of step st are bytes 32 st + 8 g of the 128-byte row: half g & 1 of chunk 2 st + g / 2,
+  // which sits at position chunk ^ (row & 7)
+  auto w8frag = [&](const unsigned char* reg, unsigned row_o, int row, int st) {
+    typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+    typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+    const u32x2 raw = *reinterpret_cast<const u32x2*>(reg + row_o + (((2 * st + (g >> 1)) ^ (row & 7)) << 4) + (g & 1) * 8);
+    u32x4 o;
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
+      // e4m3 -> fp32 has at most four significant bits: the upper halves are the bf16 values, exactly
+      o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
+      o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
+    }
+    return __builtin_bit_cast(bf16x8, o);
+  };
   const unsigned b0_o = m * 256, b1_o = (16 + m) * 256;
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     // phase p has landed when only the loads of the phase after it (if requested) are outstanding
     if (p < 3) {
-      // s_waitcnt takes an immediate: one case per number of activation blocks a phase fetches (xblocks + 5 loads)
-      switch (xblocks) {
-        case 1: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-        case 2: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
-        case 3: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-        case 4: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
-        case 5: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-        case 6: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
-        case 7: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      // s_waitcnt takes an immediate: one case per number of loads of a phase (xblocks activation blocks + LW of weight)
+      switch (xblocks + LW) {
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+        case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+        case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
+        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
         default: asm volatile("s_waitcnt vmcnt(13)" ::: "memory"); break;
       }
     } else {
@@ -209,8 +257,13 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
     for (int st = 0; st < nst; ++st) {
       fb0[st] = *reinterpret_cast<const bf16x8*>(reg + b0_o + (((4 * st + g) ^ m) << 4));
       fb1[st] = *reinterpret_cast<const bf16x8*>(reg + b1_o + (((4 * st + g) ^ m) << 4));
-      fa0[st] = *reinterpret_cast<const bf16x8*>(reg + a0_o + (((4 * st + g) ^ arow0) << 4));
-      fa1[st] = *reinterpret_cast<const bf16x8*>(reg + a1_o + (((4 * st + g) ^ m1) << 4));
+      if constexpr (W8) {
+        fa0[st] = w8frag(reg, a0_o, arow0, st);
+        fa1[st] = w8frag(reg, a1_o, 12 + m1, st);
+      } else {
+        fa0[st] = *reinterpret_cast<const bf16x8*>(reg + a0_o + (((4 * st + g) ^ arow0) << 4));
+        fa1[st] = *reinterpret_cast<const bf16x8*>(reg + a1_o + (((4 * st + g) ^ m1) << 4));
+      }
     }
     if (p + RING < 4) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the region's fragments are in registers: it may be refilled
@@ -234,11 +287,13 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
   __syncthreads();
 }
 
-void launch_qkv_decode_r32(dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+// w8: fp8 weight with a.w_scale
+void launch_qkv_decode_r32(bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
   auto even = [](int64_t v) { return (v & 1) == 0; };
   const int out4 = (reinterpret_cast<uintptr_t>(a.q) % 4 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 4 == 0) &&
                    (reinterpret_cast<uintptr_t>(a.v) % 4 == 0) && even(a.q_rs) && even(a.k_rs) && even(a.v_rs) && even(a.kv_slot_stride);
-  hipLaunchKernelGGL(qkv_decode_r32_kernel, grid, dim3(640), 0, st, a, ra, fr, out4);
+  if (w8) hipLaunchKernelGGL(qkv_decode_r32_kernel<true>, grid, dim3(640), 0, st, a, ra, fr, out4);
+  else hipLaunchKernelGGL(qkv_decode_r32_kernel<false>, grid, dim3(640), 0, st, a, ra, fr, out4);
 }
 
 }  // namespace tllm
