@@ -227,7 +227,7 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         names = ["wavefront started", "first loads issued", "activations landed",
                  "other wavefronts' sums seen" if fused else "weight phase 0 landed",
                  "activations scaled" if fused else "weight phase 3 landed",
-                 "partial tiles written", "epilogue: past the last barrier", "epilogue: before the stores"]
+                 "partial tiles written", "epilogue: past the last barrier", "epilogue: partial tiles summed"]
         table = {}
         for i, name in enumerate(names):
             v = arr[:, :, 6:, i] if i >= 6 else (arr[:, :, :6, i] if i > 0 else arr[..., i])

@@ -122,6 +122,22 @@ __device__ __forceinline__ void rope_cos_sin(const RopeArgs& r, const YarnFreqs&
   }
 }
 
+// Eight fp8 (OCP e4m3) values in two dwords -> eight bf16, exactly: e4m3 -> fp32 has at most four significant bits, so
+// the upper halves of the fp32 values are the bf16 values.
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
+  typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+  const unsigned raw[2] = {lo, hi};
+  u32x4 o;
+#pragma unroll
+  for (int d = 0; d < 2; ++d) {
+    const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
+    o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
+    o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
+  }
+  return __builtin_bit_cast(bf16x8, o);
+}
+
 // Host: validate a TllmRope and flatten it into kernel arguments.
 int make_rope_args(const TllmRope* rope, int head_dim, RopeArgs* out, YarnFreqs* freqs);
 

@@ -187,18 +187,8 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
   // 2 st + g / 2, which sits at position chunk ^ row
   auto w8frag = [&](const unsigned char* reg, int st) {
     typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
-    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
-    typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
     const u32x2 raw = *reinterpret_cast<const u32x2*>(reg + a_o + (((2 * st + (g >> 1)) ^ arow) << 4) + (g & 1) * 8);
-    u32x4 o;
-#pragma unroll
-    for (int d = 0; d < 2; ++d) {
-      const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
-      // e4m3 -> fp32 has at most four significant bits: the upper halves are the bf16 values, exactly
-      o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
-      o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
-    }
-    return __builtin_bit_cast(bf16x8, o);
+    return fp8x8_to_bf16x8(raw[0], raw[1]);
   };
 #pragma unroll
   for (int p = 0; p < NPH; ++p) {

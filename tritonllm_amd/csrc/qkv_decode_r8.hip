@@ -35,7 +35,7 @@
 // wavefront's 480 bytes of a row arrive in two phases of 8 + 7 k32 steps (256 + 224 bytes, so a row piece is as long
 // as in the bf16 form and the LDS layout is the same), fragments are widened to bf16 (exact) between the LDS read and
 // the MFMA, the row scale multiplies the finished sum.
-#include "qkv_common.h"
+#include "qkv_decode_stream.h"
 
 namespace tllm {
 
@@ -85,56 +85,10 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     // the streaming wavefronts' rendezvous between their activation and weight loads (it also publishes their
     // cleared flags): met here at once, before this wavefront has anything to wait for
     if constexpr (NORM != 0) __syncthreads();
-    const int en = lane & 15, eg = lane >> 4;               // activation row, quad of the tile
-    const int epair = pair0 + (tile ? 6 : 0) + 2 * eg;      // even; its neighbour epair + 1 shares head and quad
-    const bool evalid = eg < (tile ? 2 : 3) && epair < total_pairs && en < nvalid;
-    const int egp = evalid ? epair : 0;
-    const int ehead = egp >> 5, ed = egp & 31;
-    const int64_t erow = row0 + (evalid ? en : 0);
-    const bool erot = a.has_rope && ehead < a.n_q_heads + a.n_kv_heads;
-    const int64_t* pos_ptr = ra.positions ? ra.positions + erow : reinterpret_cast<const int64_t*>(a.W);
-    const int64_t* off_ptr = ra.offset ? ra.offset : reinterpret_cast<const int64_t*>(a.W);
-    const unsigned* bias_ptr = reinterpret_cast<const unsigned*>(a.bias ? a.bias : a.W);   // two bf16 per load; ed is even
-    const int64_t pos_ld = *pos_ptr;
-    const int64_t off_ld = *off_ptr;
-    const unsigned b_lo = bias_ptr[(ehead * 64 + ed) >> 1];
-    const unsigned b_hi = bias_ptr[(ehead * 64 + 32 + ed) >> 1];
-    const float freq0 = fr.v[ed], freq1 = fr.v[ed + 1];
-    float ws_l0 = 1.f, ws_l1 = 1.f, ws_h0 = 1.f, ws_h1 = 1.f;   // W8: the row scales of the lane's four weight rows
-    if constexpr (W8) {
-      const float* sp = a.w_scale + ehead * 64 + ed;        // 4-byte aligned is all the interface asks for
-      ws_l0 = sp[0];
-      ws_l1 = sp[1];
-      ws_h0 = sp[32];
-      ws_h1 = sp[33];
-    }
-    float cs0 = 1.f, sn0 = 0.f, cs1 = 1.f, sn1 = 0.f;
-    const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
-    if (erot) {
-      int64_t pos = ra.positions ? pos_ld : (erow % ra.tokens_per_batch) + (ra.offset ? off_ld : 0);
-      pos = rope_wrap(pos, ra.max_ctx);
-      if (ra.use_yarn) {
-        yarn_cos_sin(pos, freq0, ra.concentration, &cs0, &sn0);
-        yarn_cos_sin(pos, freq1, ra.concentration, &cs1, &sn1);
-      } else {
-        rope_cos_sin(ra, fr, pos, ed, &cs0, &sn0);
-        rope_cos_sin(ra, fr, pos, ed + 1, &cs1, &sn1);
-      }
-    }
-    float bl0 = 0.f, bl1 = 0.f, bh0 = 0.f, bh1 = 0.f;
-    if (a.bias) {
-      bl0 = __uint_as_float(b_lo << 16);
-      bl1 = __uint_as_float(b_lo & 0xffff0000u);
-      bh0 = __uint_as_float(b_hi << 16);
-      bh1 = __uint_as_float(b_hi & 0xffff0000u);
-    }
-    bf16* out = qkv_out_ptr(a, slot, erow, ehead) + ed;
+    StreamEpilogueLane<W8> ep;
+    ep.prepare(a, ra, fr, pair0, tile, lane >> 4, lane & 15, row0, nvalid);   // quad of the tile, activation row
     unsigned red_o = static_cast<unsigned>(REGION + tile * 1024 + lane * 16);
-    if constexpr (W8) asm volatile("" : "+v"(ws_l0), "+v"(ws_l1), "+v"(ws_h0), "+v"(ws_h1));
-    // One wavefront runs alone from the last barrier to the stores, so every instruction after that barrier is
-    // latency: all of the above is forced to exist here (left to itself the compiler moves it to its first use,
-    // behind the barrier).
-    asm volatile("" : "+v"(cs0), "+v"(sn0), "+v"(cs1), "+v"(sn1), "+v"(bl0), "+v"(bl1), "+v"(bh0), "+v"(bh1), "+v"(out), "+v"(red_o));
+    asm volatile("" : "+v"(red_o));
     __syncthreads();                                        // partial tiles are in LDS
     R8_STAMP(6);
     f32x4 t[NS];
@@ -148,37 +102,8 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
       acc[2] += t[w][2];
       acc[3] += t[w][3];
     }
-    if (!evalid) return;
-    if constexpr (W8) {
-      acc[0] *= ws_l0;
-      acc[1] *= ws_l1;
-      acc[2] *= ws_h0;
-      acc[3] *= ws_h1;
-    }
-    float lo0 = acc[0] + bl0, lo1 = acc[1] + bl1, hi0 = acc[2] + bh0, hi1 = acc[3] + bh1;   // [lo(d), lo(d+1), hi(d), hi(d+1)] of row en
-    if (erot) {
-      const float r0 = lo0 * cs0 - hi0 * sn0, r2 = hi0 * cs0 + lo0 * sn0;
-      const float r1 = lo1 * cs1 - hi1 * sn1, r3 = hi1 * cs1 + lo1 * sn1;
-      lo0 = r0;
-      lo1 = r1;
-      hi0 = r2;
-      hi1 = r3;
-    }
-    bf16x2 plo, phi;
-    plo[0] = static_cast<bf16>(lo0);
-    plo[1] = static_cast<bf16>(lo1);
-    phi[0] = static_cast<bf16>(hi0);
-    phi[1] = static_cast<bf16>(hi1);
     R8_STAMP(7);
-    if (out4) {
-      *reinterpret_cast<bf16x2*>(out) = plo;
-      *reinterpret_cast<bf16x2*>(out + 32) = phi;
-    } else {
-      out[0] = plo[0];
-      out[1] = plo[1];
-      out[32] = phi[0];
-      out[33] = phi[1];
-    }
+    ep.finish(acc, out4);
     return;
   }
 
@@ -424,18 +349,8 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // 2 st + g / 2, which sits at position chunk ^ (tile row & 15)
   auto w8frag = [&](const unsigned char* reg, unsigned row_o, int trow, int st) {
     typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
-    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
-    typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
     const u32x2 raw = *reinterpret_cast<const u32x2*>(reg + row_o + (((2 * st + (g >> 1)) ^ trow) << 4) + (g & 1) * 8);
-    u32x4 o;
-#pragma unroll
-    for (int d = 0; d < 2; ++d) {
-      const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
-      // e4m3 -> fp32 has at most four significant bits: the upper halves are the bf16 values, exactly
-      o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
-      o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
-    }
-    return __builtin_bit_cast(bf16x8, o);
+    return fp8x8_to_bf16x8(raw[0], raw[1]);
   };
 #pragma unroll
   for (int p = 0; p < NPH; ++p) {
@@ -475,9 +390,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
 
 // Host side: pick the instantiation. norm = 0 / 1 (fp32 scale) / 2 (bf16 scale); w8: fp8 weight with a.w_scale.
 void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
-  auto even = [](int64_t v) { return (v & 1) == 0; };
-  const int out4 = (reinterpret_cast<uintptr_t>(a.q) % 4 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 4 == 0) &&
-                   (reinterpret_cast<uintptr_t>(a.v) % 4 == 0) && even(a.q_rs) && even(a.k_rs) && even(a.v_rs) && even(a.kv_slot_stride);
+  const int out4 = qkv_outputs_allow_4_byte_stores(a);
 #define TLLM_R8(NORM, EMBF)                                                                                               \
   do {                                                                                                                    \
     if (w8) hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF, true>), grid, dim3(512), 0, st, a, ra, fr, out4);        \
