@@ -7,39 +7,40 @@
 // the end of this comment). Eight wavefronts form a 4 x 2 grid (two per SIMD); each owns 32 x 160 of the tile as
 // 1 x 5 v_mfma_f32_32x32x16_bf16 blocks (80 fp32 accumulators per lane) and reads 6 operand
 // fragments from LDS per 5 MFMAs. K is walked in slices of 64 (one 128-byte line per row) through
-// two LDS stages filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers,
-// no ds_write). Such a load puts the 64 lanes' 16-byte chunks at consecutive LDS addresses, so rows
+// LDS stage rings filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers,
+// no ds_write): two stages of 16 KB for the tile's activations, three of 40 KB for its weight. Such a load puts
+// the 64 lanes' 16-byte chunks at consecutive LDS addresses, so rows
 // cannot be padded; instead the chunk order inside each row is XOR-swizzled with the row index --
 // applied by choosing which *global* chunk a lane fetches -- and the fragment reads undo it, which
 // keeps the 128-bit fragment reads of 16 consecutive rows conflict-free.
 // With one tile per CU nothing but the kernel's own schedule overlaps anything:
-//   * the one barrier per slice sits before the slice's last k16 step; the stage just finished is handed to
-//     the slice after next, whose loads go out one per MFMA behind that step and the next (never all in a row:
-//     a CU's load queue is bounded and a wavefront that overflows it stalls, MFMAs included);
+//   * the one barrier per slice sits before the slice's last k16 step; the stages just finished are handed on
+//     (activations: to the slice after next; weight: to the slice three on), the loads going out one per MFMA behind
+//     that step and the next (never all in a row: a CU's load queue is bounded and a wavefront that overflows it
+//     stalls, MFMAs included);
 //   * the fragment reads of the next k16 step are pinned between the MFMAs of the current one
 //     (sched_group_barrier): hoisted to the top of the iteration, as the compiler does by itself, the
 //     wavefronts read a slice's fragments in one burst with no MFMA running.
-// (An L2 warm-up -- every workgroup touching, three slices ahead, its share of the lines its XCD's tiles would need --
-// paid with one wavefront per SIMD; with two it measures as noise or a small loss and is gone.)
-// Where the time goes at T = 2048 (66 us; builds with parts of the loop compiled out): the MFMAs, barriers,
-// prologue and epilogue alone take 43 us (30 us of MFMAs at the 1.9 GHz this load clocks at), adding the
-// fragment reads 55 us, the global->LDS loads alone (no MFMA, no fragment read) 56 us, everything 66 us. The
-// loads are the wall: with two stages the loads of slice i+2 cannot start before slice i has been read by
-// everyone and must have landed before slice i+1 has been, so every slice pays its 56 KB through the CU's
-// 64 B/clk address unit (~900 cycles) plus an L2 round trip inside one slice's 1280 cycles of MFMAs, and a third
-// stage of this tile does not fit (3 x 56 KB > 160 KB). Measured without gain: the 2 x 2 grid of 64 x 160
-// wavefronts this kernel started with (70 us: one wavefront per SIMD, nothing to cover a stalled load issue),
-// pairs of 64 x 160 wavefronts taking alternate k16 steps (fewer fragment reads, 68 us), four extra wavefronts that
-// only load (71-75 us), K slices of 32 in a four-stage ring (77 us), a four-deep feed with two more slices in flight
-// into registers and written to LDS by ds_write (70.6 us -- so the two-stage window above is not the whole story),
-// other spreads of the loads over the steps and other prefetch distances (+-1 us).
-// The feed itself: 256 tiles x 2.58 MB = 660 MB through the L2s in those 44 us (~15 TB/s, 7.1 M requests of 128 B);
-// doubling the requests (every wavefront touching its own lines ahead of time) cost 13 %, so only fewer bytes per
-// flop -- a larger tile, which T = 2048 on 256 CUs does not allow -- would lift the wall.
+// Where the time goes at T = 2048 (builds with parts of the loop compiled out, two 56 KB stages): the MFMAs,
+// barriers, prologue and epilogue alone take 43 us (30 us of MFMAs at the 1.9 GHz this load clocks at), adding the
+// fragment reads 55 us, the global->LDS loads alone (no MFMA, no fragment read) 56 us, everything 64-66 us. Two things
+// bound it. The feed: what a CU receives is its bytes in flight over the latency of a slice (every slice contains
+// lines nobody in the XCD has touched yet, and a CU returns loads in order, so a slice completes at miss latency,
+// 1.2-2 us); two symmetric stages keep one slice (56 KB) in flight, 46 GB/s per CU. The third weight stage (which
+// fits once the cos/sin table no longer sits next to the stages) keeps two weight slices in flight; a probe of the
+// feed with dummy MFMAs went from 59 to 46 us with it -- the kernel itself only from 64-70 to 63-68.5 us, because
+// behind the feed sits the LDS: 8 wavefronts x 6 fragment reads x 4 steps x 8 clocks + 448 clocks of stage writes per
+// slice are 1984 clocks against 1280 of MFMAs. Measured without gain: the 2 x 2 grid of 64 x 160
+// wavefronts this kernel started with (70 us, 75 us with the three-stage ring: one wavefront per SIMD, nothing to cover
+// a stalled load issue), pairs of 64 x 160 wavefronts taking alternate k16 steps (fewer fragment reads, 68 us), four
+// extra wavefronts that only load (71-75 us), K slices of 32 in a four-stage ring (77 us), a four-deep feed with two
+// more slices in flight into registers and written to LDS by ds_write (70.6 us), an L2 warm-up by a ninth wavefront
+// (its loads sit in the same in-order queue), other spreads of the loads over the steps (+-1 us).
 // From T = 4096 up there are enough tokens for 256 x 320 tiles (BM = 256: eight wavefronts of 64 x 160, 36 % fewer
-// bytes per flop through the L2s): 238 -> 213 us at T = 8192 (1131 TFLOP/s). Its 160 accumulators leave room for
-// single-buffered weight fragments only, the cos/sin table is built after the K loop inside the idle stage ring
-// (no LDS for it next to 2 x 72 KB of stages) and the epilogue runs in two passes of 128 rows.
+// bytes per flop through the L2s): 238 -> 202-205 us at T = 8192. Its 160 accumulators leave room for
+// single-buffered weight fragments only, its stages (2 x 32 KB + 2 x 40 KB) for no third weight stage, and the
+// epilogue runs in two passes of 128 rows. Neither tile has LDS left for the cos/sin table next to the stages: it is
+// built after the K loop inside the idle ring.
 //
 // The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
 // a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
@@ -62,12 +63,16 @@ namespace {
 constexpr int HPT = 5;             // heads per tile
 constexpr int BN = HPT * 64;       // 320 columns per tile
 constexpr int BK = 64;             // K slice: one 128-byte line per row
-constexpr int NS = 2;              // LDS stages
+constexpr int XS = 2;              // LDS stages of the activations
 constexpr int KS = BK / 16;        // k16 MFMA steps per slice
 constexpr int CHUNKS = BK / 8;     // 16-byte chunks per LDS row
 constexpr int LROW = BK * 2;       // LDS row, bytes (unpadded: rows are swizzled instead)
 constexpr int RPB = 1024 / LROW;   // rows per 1 KiB block (one load instruction)
-constexpr int stage_bytes(int bm) { return (bm + BN) * LROW; }   // one LDS stage of a bm-token tile
+constexpr int W_STAGE = BN * LROW;                               // one LDS stage of the weight: 320 rows of one K slice
+constexpr int x_stage(int bm) { return bm * LROW; }              // ... of a bm-token tile's activations
+// A 128-token tile has room for a third weight stage (3 x 40 KB + 2 x 16 KB), a 256-token tile has not (2 x 40 + 2 x 32).
+constexpr int w_stages(int bm) { return bm == 128 ? 3 : 2; }
+constexpr int ring_bytes(int bm) { return w_stages(bm) * W_STAGE + XS * x_stage(bm); }
 constexpr int OROW = BN + 4;       // epilogue staging row, elements (648 B: an odd number of 8-byte units)
 constexpr int CSROW = 34;                  // float2 per row of the cos/sin table: 32 frequencies + padding, so that
                                            // lanes reading the same frequency of 32 different rows spread over the banks
@@ -75,15 +80,14 @@ constexpr int EROWS = 128;                 // rows the epilogue finishes per pas
 constexpr int CS_BYTES = EROWS * CSROW * 8;   // cos/sin of (row, frequency) as float2
 constexpr int IMG_BYTES = (EROWS * OROW * 2 + 1023) / 1024 * 1024;   // bf16 image of a pass's rows
 constexpr int BIAS_BYTES = BN * 4;         // the tile's bias as fp32, head-local column order
-// A 128-token tile keeps the cos/sin table in its own region next to the two stages; a 256-token tile has no room for
-// that (2 x 72 KB of stages), keeps only the rows' positions and builds the table inside the idle stage ring, per pass.
-constexpr int prefill_smem(int bm) {
-  return bm == 128 ? NS * stage_bytes(128) + CS_BYTES + BIAS_BYTES : NS * stage_bytes(bm) + BIAS_BYTES + bm * 8;
-}
-static_assert(IMG_BYTES <= NS * stage_bytes(128) && IMG_BYTES + CS_BYTES <= NS * stage_bytes(256), "the epilogue reuses the stage ring");
+// The stages leave no room for the cos/sin table: it is built inside the idle stage ring after the K loop -- by a
+// 128-token tile from values computed while the first slices were in flight and kept in registers, by a 256-token tile
+// (no registers to spare) per pass from the rows' positions parked in LDS.
+constexpr int prefill_smem(int bm) { return ring_bytes(bm) + BIAS_BYTES + bm * 8; }
+static_assert(IMG_BYTES + CS_BYTES <= ring_bytes(128) && IMG_BYTES + CS_BYTES <= ring_bytes(256), "the epilogue reuses the stage ring");
 static_assert(prefill_smem(128) <= 160 * 1024 && prefill_smem(256) <= 160 * 1024, "LDS per workgroup");
-static_assert(KS % 2 == 0 && stage_bytes(128) % 8192 == 0 && stage_bytes(256) % 8192 == 0 && CHUNKS == 8 && NS == 2,
-              "the schedule and the swizzle below are written for BK = 64, two stages");
+static_assert(KS % 2 == 0 && W_STAGE % 8192 == 0 && x_stage(128) % 8192 == 0 && CHUNKS == 8 && XS == 2,
+              "the schedule and the swizzle below are written for BK = 64");
 }  // namespace
 
 // Chunk swizzle of LDS row r: the 16-byte chunk c of the row is stored at chunk position c ^ swz(r).
@@ -110,12 +114,14 @@ __device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
 // the tokens: 36 % fewer bytes per flop through the L2s, which is what bounds the 128-token tile.
 template <int BM, int WROWS>
 __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
-  constexpr int STAGE = stage_bytes(BM);
-  constexpr int BLOCKS = STAGE / 1024;      // 1 KiB blocks per stage
+  constexpr int WS = w_stages(BM);          // weight stages
+  constexpr int XSTAGE = x_stage(BM);
   constexpr int NW = WROWS * 2;             // wavefronts
   constexpr int NT = NW * 64;               // threads
   constexpr int MB = BM / (32 * WROWS);     // 32-token blocks per wavefront
-  constexpr int LPW = BLOCKS / NW;          // load instructions per wavefront per stage
+  constexpr int LPX = XSTAGE / 1024 / NW;   // load instructions (1 KiB blocks) per wavefront per slice: activations ...
+  constexpr int LPWW = W_STAGE / 1024 / NW; // ... weight
+  constexpr int LPW = LPX + LPWW;           // ... together
   constexpr int NMF = MB * 5;               // MFMAs per k16 step
   constexpr int NRD = MB + 5;               // fragment reads per k16 step
   constexpr int NL_LAST = LPW < NMF ? LPW : NMF;   // loads handed out behind a slice's last step ...
@@ -152,35 +158,41 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   const int kvec = a.hidden >> 3;
   const int n_iter = a.hidden / BK;
 
-  // ---- loader setup. Load instruction j of wavefront w fills LDS block w*LPW + j (RPB rows of LROW bytes);
-  // lane L lands at row RPB*blk + L/CHUNKS, chunk position L%CHUNKS, so it fetches global chunk (L%CHUNKS) ^ swz(row).
+  // ---- loader setup. A slice's activations (BM rows) and weight (320 rows) land in separate stage rings; within its
+  // operand, load instruction j of wavefront w fills 1 KiB block w * n + j (RPB rows of LROW bytes); lane L lands at
+  // row RPB * blk + L / CHUNKS, chunk position L % CHUNKS, so it fetches global chunk (L % CHUNKS) ^ swz(row).
+  // A wavefront's loads of a period are numbered activations first (j < LPX), then weight.
   // The tiles that share an XCD's L2 walk K in lockstep and four or eight of them want the same lines;
   // each starts its round of blocks at a different one so that at any moment they pull on different
   // rows (different L2 channels) instead of queueing on the same line.
-  const int rot = (blockIdx.x >> 3) % LPW;
+  const int rotx = (blockIdx.x >> 3) % LPX, rotw = (blockIdx.x >> 3) % LPWW;
   // A load's source is a scalar base (the tile's first activation row, or the weight) plus a 32-bit byte offset per
   // lane: half the registers of a pointer per load, and the loads can use the scalar-base addressing form.
   const unsigned char* const x_base = reinterpret_cast<const unsigned char*>(a.x) + row0 * a.hidden * 2;
   const unsigned char* const w_base = reinterpret_cast<const unsigned char*>(a.W);
+  unsigned char* const wring = smem;                         // WS stages of W_STAGE bytes
+  unsigned char* const xring = smem + WS * W_STAGE;          // XS stages of XSTAGE bytes
   unsigned soff[LPW];
-  int blk_off[LPW];                                          // LDS byte offset of load j's block inside the wavefront's share
-  bool src_is_x[LPW];                                        // scalar: a 1 KiB block lies entirely in one operand
+  int blk_off[LPW];                                          // LDS byte offset of load j's block inside its operand's stage
 #pragma unroll
   for (int j = 0; j < LPW; ++j) {
-    const int bj = (j + rot) % LPW;
-    blk_off[j] = bj * 1024;
-    const int r = (wave * LPW + bj) * RPB + lane / CHUNKS;  // LDS row: 0..BM-1 activations, then 320 weight rows
-    const int c = (lane % CHUNKS) ^ swz(r);
-    src_is_x[j] = (wave * LPW + bj) * RPB < BM;
-    if (src_is_x[j]) {
+    if (j < LPX) {
+      const int bj = wave * LPX + (j + rotx) % LPX;
+      blk_off[j] = bj * 1024;
+      const int r = bj * RPB + lane / CHUNKS;                // activation row of the tile
+      const int c = (lane % CHUNKS) ^ swz(r);
       int64_t lr = r;
-      if (row0 + lr >= a.rows) lr = a.rows - 1 - row0;      // clamp: valid memory, result rows are never stored
+      if (row0 + lr >= a.rows) lr = a.rows - 1 - row0;       // clamp: valid memory, result rows are never stored
       soff[j] = static_cast<unsigned>((lr * kvec + c) * 16);
     } else {
+      const int bj = wave * LPWW + (j - LPX + rotw) % LPWW;
+      blk_off[j] = bj * 1024;
+      const int r = bj * RPB + lane / CHUNKS;                // weight row of the tile (LDS order)
+      const int c = (lane % CHUNKS) ^ swz(r);
       int hl, dim;
-      w_tile_row(r - BM, &hl, &dim);
+      w_tile_row(r, &hl, &dim);
       int h = head0 + hl;
-      if (h >= total_heads) h = total_heads - 1;        // clamp for a ragged last tile
+      if (h >= total_heads) h = total_heads - 1;             // clamp for a ragged last tile
       soff[j] = static_cast<unsigned>(((static_cast<int64_t>(h) * 64 + dim) * kvec + c) * 16);
     }
   }
@@ -194,7 +206,7 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
 
   // fragment addressing: byte offset of (row, chunk c) inside a stage is row*LROW + ((c ^ swz(row)) << 4)
-  const int fa_row = 32 * MB * wm + l32, fb_row = BM + 160 * wn + l32;
+  const int fa_row = 32 * MB * wm + l32, fb_row = 160 * wn + l32;   // rows inside the activation / the weight stage
   // The k16 step kk wants chunks 2 kk + lh of the row; with the row's swizzle that is position (2 kk + lh) ^ swz(row),
   // and because a row starts on a 128-byte boundary the step enters as an XOR of bits 5-6 of the byte offset: one
   // register per 32-row block instead of one per block and step.
@@ -203,25 +215,29 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   for (int mb = 0; mb < MB; ++mb) fa_o[mb] = (fa_row + 32 * mb) * LROW + ((lh ^ swz(fa_row + 32 * mb)) << 4);
 #pragma unroll
   for (int nb = 0; nb < 5; ++nb) fb_o[nb] = (fb_row + 32 * nb) * LROW + ((lh ^ swz(fb_row + 32 * nb)) << 4);
-  auto load_frags = [&](const unsigned char* st, int kk, bf16x8 (&fa)[MB], bf16x8 (&fb)[5]) {
+  auto load_frags = [&](const unsigned char* stx, const unsigned char* stw, int kk, bf16x8 (&fa)[MB], bf16x8 (&fb)[5]) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(st + (fa_o[mb] ^ (kk << 5)));
+    for (int mb = 0; mb < MB; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(stx + (fa_o[mb] ^ (kk << 5)));
 #pragma unroll
-    for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(st + (fb_o[nb] ^ (kk << 5)));
+    for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(stw + (fb_o[nb] ^ (kk << 5)));
   };
-  auto issue_load = [&](int it, int j) {                // one load instruction of slice `it`
-    unsigned char* dst = smem + (it % NS) * STAGE + wave * (LPW * 1024);
-    const int itc = it < n_iter ? it : n_iter - 1;
+  // Period `per` = the loads that go out when slice `per` has been consumed: the activations of slice per + 2 into the
+  // activation stage that slice just vacated, the weight of slice per + WS into the weight stage it vacated.
+  auto issue_load = [&](int per, int j) {                // one load instruction of period `per`
+    const bool is_x = j < LPX;                            // known at compile time wherever j is
+    const int sl = per + (is_x ? XS : WS);
+    const int slc = sl < n_iter ? sl : n_iter - 1;        // look-ahead past the end re-reads the last slice (never used)
+    unsigned char* dst = is_x ? xring + (sl % XS) * XSTAGE : wring + (sl % WS) * W_STAGE;
     // Spelled out rather than through __builtin_amdgcn_global_load_lds: this is the scalar-base form (64-bit base in
     // SGPRs, 32-bit lane offset, LDS block address in M0), where the builtin builds a 64-bit address per lane; 14 / 13
     // fewer registers in the two tile heights and 2-3 % faster. The lanes' 16 bytes land at M0 + 16 * lane.
     const unsigned lds_off = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst + blk_off[j]));
-    const unsigned char* sb = (src_is_x[j] ? x_base : w_base) + static_cast<int64_t>(itc) * (BK * 2);
+    const unsigned char* sb = (is_x ? x_base : w_base) + static_cast<int64_t>(slc) * (BK * 2);
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
   };
-  auto issue_loads = [&](int it) {                      // all of slice `it` -> stage it % NS
+  auto issue_period = [&](int per) {
 #pragma unroll
-    for (int j = 0; j < LPW; ++j) issue_load(it, j);
+    for (int j = 0; j < LPW; ++j) issue_load(per, j);
   };
   // One k16 step: NMF MFMAs on the fragments in buffer `cur`. Behind the MFMAs go the LDS reads of the next step's
   // fragments (into buffer cur ^ 1) and, for m < n, one global->LDS load instruction (j0 + m) of slice `lit`.
@@ -233,11 +249,11 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   //     included, until the queue has drained that far; a slice's loads in a row do exactly that. Handed out one
   //     per MFMA (32 cycles) they never find the queue full.
   bf16x8 fa[2][MB], fb[2][5];
-  auto read_frag = [&](int cur, const unsigned char* nst, int nkk, int i) {   // fragment i of the next step: activations first
-    if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nst + (fa_o[i < MB ? i : 0] ^ (nkk << 5)));
-    else fb[cur ^ 1][i - MB] = *reinterpret_cast<const bf16x8*>(nst + (fb_o[i - MB] ^ (nkk << 5)));
+  auto read_frag = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int i) {   // fragment i of the next step: activations first
+    if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nstx + (fa_o[i < MB ? i : 0] ^ (nkk << 5)));
+    else fb[cur ^ 1][i - MB] = *reinterpret_cast<const bf16x8*>(nstw + (fb_o[i - MB] ^ (nkk << 5)));
   };
-  auto step = [&](int cur, const unsigned char* nst, int nkk, int lit, int j0, int n) {
+  auto step = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int lit, int j0, int n) {
     if constexpr (MB == 2) {
       // 64 x 160 per wavefront: the two MFMAs that share a weight fragment are issued back to back and the fragment is
       // reloaded for the next step right behind them (weight fragments single-buffered: 20 registers instead of 40, which
@@ -247,8 +263,8 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       for (int nb = 0; nb < 5; ++nb) {
         acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][nb], fa[cur][0], acc[0][nb], 0, 0, 0);
         acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][nb], fa[cur][1], acc[1][nb], 0, 0, 0);
-        fb[0][nb] = *reinterpret_cast<const bf16x8*>(nst + (fb_o[nb] ^ (nkk << 5)));
-        if (nb < 2) fa[cur ^ 1][nb] = *reinterpret_cast<const bf16x8*>(nst + (fa_o[nb] ^ (nkk << 5)));
+        fb[0][nb] = *reinterpret_cast<const bf16x8*>(nstw + (fb_o[nb] ^ (nkk << 5)));
+        if (nb < 2) fa[cur ^ 1][nb] = *reinterpret_cast<const bf16x8*>(nstx + (fa_o[nb] ^ (nkk << 5)));
         if (2 * nb < n) issue_load(lit, j0 + 2 * nb);
         if (2 * nb + 1 < n) issue_load(lit, j0 + 2 * nb + 1);
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
@@ -267,7 +283,7 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       constexpr int EXTRA = NRD > NMF ? NRD - NMF : 0;
       const int r0 = m == 0 ? 0 : m + EXTRA, nr = m == 0 ? 1 + EXTRA : (m + EXTRA < NRD ? 1 : 0);
 #pragma unroll
-      for (int i = 0; i < nr; ++i) read_frag(cur, nst, nkk, r0 + i);
+      for (int i = 0; i < nr; ++i) read_frag(cur, nstx, nstw, nkk, r0 + i);
       if (m < n) issue_load(lit, j0 + m);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // one MFMA
       if (nr == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // its LDS reads
@@ -276,16 +292,17 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
     }
   };
 
-  // prologue: slices 0..NS-2 in flight, slice 0 landed
+  // prologue: slice 0 requested first (period -XS asks for activations 0, period -WS for weight 0)
 #pragma unroll
-  for (int i = 0; i < NS - 1; ++i) issue_loads(i);
-  // cos/sin of (row, frequency) for the epilogue, computed from the YaRN parameters. A 128-token tile builds the table
-  // here, into its own LDS region, while the first slices are in flight (the positions are global loads: all of
-  // them are issued before any is used). A 256-token tile only parks the rows' positions in LDS now and builds the
-  // table after the K loop, inside the idle stage ring, 128 rows at a time.
-  constexpr bool CS_EARLY = BM == EROWS;
-  constexpr int CS_OFF = CS_EARLY ? NS * STAGE : IMG_BYTES;
-  constexpr int BIAS_OFF = CS_EARLY ? NS * STAGE + CS_BYTES : NS * STAGE;
+  for (int j = 0; j < LPW; ++j) issue_load(j < LPX ? -XS : -WS, j);
+  // cos/sin of (row, frequency) for the epilogue, computed from the YaRN parameters. There is no LDS for the table
+  // next to the stages; it is built inside the idle stage ring after the K loop. A 128-token tile computes the values
+  // here, while the first slices are in flight (the positions are global loads: all of them are issued before any is
+  // used), and keeps them in registers until then; a 256-token tile (no registers to spare) only parks the rows'
+  // positions in LDS now and computes the table after the loop, 128 rows at a time.
+  constexpr bool CS_REGS = BM == EROWS;
+  constexpr int CS_OFF = IMG_BYTES;
+  constexpr int BIAS_OFF = ring_bytes(BM);
   float2* cs_tab = reinterpret_cast<float2*>(smem + CS_OFF);
   // the tile's 320 bias values, widened once (fetched per group inside the epilogue they were twenty dependent
   // global loads per lane, each waited for)
@@ -297,25 +314,30 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
     bias_s[tid] = a.bias ? static_cast<float>(a.bias[h * 64 + (tid & 63)]) : 0.f;
   }
   constexpr int RPP = NT / 32;                         // table rows per round of the whole workgroup
-  auto fill_cs_rows = [&](auto&& pos_of) {             // the table of EROWS rows; pos_of(row) -> raw position
+  constexpr int CSN = EROWS / RPP;                     // table entries per thread: rows tid / 32 + RPP * j, frequency tid % 32
+  float2 csr[CS_REGS ? CSN : 1];
+  auto compute_cs = [&](auto&& pos_of, auto&& sink) {  // pos_of(row) -> raw position; sink(j, cos, sin)
     const int f = tid & 31;
-    int64_t pos[EROWS / RPP];
+    int64_t pos[CSN];
 #pragma unroll
-    for (int j = 0; j < EROWS / RPP; ++j) pos[j] = pos_of((tid >> 5) + RPP * j);
+    for (int j = 0; j < CSN; ++j) pos[j] = pos_of((tid >> 5) + RPP * j);
 #pragma unroll
-    for (int j = 0; j < EROWS / RPP; ++j) {
+    for (int j = 0; j < CSN; ++j) {
       float c, sn;
       rope_cos_sin(ra, fr, rope_wrap(pos[j], ra.max_ctx), f, &c, &sn);
-      cs_tab[((tid >> 5) + RPP * j) * CSROW + f] = make_float2(c, sn);
+      sink(j, c, sn);
     }
   };
+  auto store_cs = [&](int j, float c, float sn) { cs_tab[((tid >> 5) + RPP * j) * CSROW + (tid & 31)] = make_float2(c, sn); };
   if (a.has_rope) {
-    if constexpr (CS_EARLY) {
-      fill_cs_rows([&](int r) {
-        int64_t grow = row0 + r;
-        if (grow >= a.rows) grow = a.rows - 1;
-        return rope_position_raw(ra, grow);
-      });
+    if constexpr (CS_REGS) {
+      compute_cs(
+          [&](int r) {
+            int64_t grow = row0 + r;
+            if (grow >= a.rows) grow = a.rows - 1;
+            return rope_position_raw(ra, grow);
+          },
+          [&](int j, float c, float sn) { csr[j] = make_float2(c, sn); });
     } else {
       for (int r = tid; r < BM; r += NT) {
         int64_t grow = row0 + r;
@@ -324,33 +346,45 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       }
     }
   }
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPW) : "memory");
+  // The rest of the look-ahead, oldest first: (three weight stages: weight 1,) then period -1 = activations 1 and the
+  // weight of slice WS - 1. Requested only now: the compiler waits for its own loads above (positions, bias) by
+  // count, which would have made it wait for these as well.
+  if constexpr (WS == 3) {
+#pragma unroll
+    for (int j = LPX; j < LPW; ++j) issue_load(-2, j);
+  }
+  issue_period(-1);
+  // slice 0 has landed when only those are outstanding
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");
   __syncthreads();
-  load_frags(smem, 0, fa[0], fb[0]);
+  load_frags(xring, wring, 0, fa[0], fb[0]);
 
-  // Steady state: slices it+1 .. it+NS-1 are in flight or landed while slice it is multiplied. The one
-  // barrier per slice sits before the slice's last k16 step; from there on the stage of slice `it` is free
-  // (all reads of it have been issued) and is handed to slice it+NS, whose loads go out behind the MFMAs of
-  // this last step and, what does not fit there, of the next slice's first step -- a whole slice of MFMAs
-  // before they are needed.
-  issue_loads(NS - 1);
+  // Steady state. While slice `it` is multiplied, outstanding or landed, oldest first: (three weight stages: the
+  // weight of slice it + 1,) the activations of slice it + 1, the weight of slice it + WS - 1. The one barrier per
+  // slice sits before the slice's last k16 step; from there on the stages of slice `it` are free (all reads of them
+  // have been issued) and period `it` goes out behind the MFMAs of this last step and, what does not fit there, of the
+  // next slice's first step: the activations of slice it + 2 -- a whole slice of MFMAs before they are needed -- and
+  // the weight of slice it + WS -- with the third stage, two slices.
   for (int it = 0; it < n_iter; ++it) {
-    const unsigned char* st = smem + (it % NS) * STAGE;
-    const unsigned char* nx = smem + ((it + 1) % NS) * STAGE;
+    const unsigned char* stx = xring + (it % XS) * XSTAGE;
+    const unsigned char* stw = wring + (it % WS) * W_STAGE;
+    const unsigned char* nxx = xring + ((it + 1) % XS) * XSTAGE;
+    const unsigned char* nxw = wring + ((it + 1) % WS) * W_STAGE;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) {
       if (kk + 1 < KS) {
         if (kk == 0 && it > 0) {
-          step(kk & 1, st, kk + 1, it + NS - 1, NL_LAST, NL_FIRST);
+          step(kk & 1, stx, stw, kk + 1, it - 1, NL_LAST, NL_FIRST);
         } else {
-          step(kk & 1, st, kk + 1, 0, 0, 0);
+          step(kk & 1, stx, stw, kk + 1, 0, 0, 0);
         }
       } else {
-        // Slice it+1 has landed (this wavefront's share), then the barrier: everyone's
-        // share has, and everyone has issued its last reads of slice it. Spelled out, because __syncthreads()
-        // carries a fence that drains every load in flight, the look-ahead ones included.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * LPW) : "memory");
-        step(kk & 1, nx, 0, it + NS, 0, NL_LAST);
+        // Slice it + 1 has landed (this wavefront's share: everything but the newest weight slice of a three-stage
+        // ring), then the barrier: everyone's share has, and everyone has issued its last reads of slice it.
+        // Spelled out, because __syncthreads() carries a fence that drains every load in flight, the look-ahead ones
+        // included.
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((WS - 2) * LPWW) : "memory");
+        step(kk & 1, nxx, nxw, 0, it, 0, NL_LAST);
       }
     }
   }
@@ -374,11 +408,18 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
   // dims, their partners: same register index); the mixed block holds the wavefront's 16 low dims of
   // the middle head in rows 0-15 and their partners in rows 16-31 (register v and v + 8).
   // A pass finishes EROWS rows: the wavefronts that hold them write the image, then everyone copies it out.
+  if constexpr (CS_REGS) {
+    if (a.has_rope) {
+#pragma unroll
+      for (int j = 0; j < CSN; ++j) store_cs(j, csr[j].x, csr[j].y);
+    }
+    __syncthreads();
+  }
 #pragma unroll
   for (int pass = 0; pass < BM / EROWS; ++pass) {
-  if constexpr (!CS_EARLY) {
+  if constexpr (!CS_REGS) {
     if (pass > 0) __syncthreads();                        // the previous pass's image and table have been read
-    if (a.has_rope) fill_cs_rows([&](int r) { return pos_s[EROWS * pass + r]; });
+    if (a.has_rope) compute_cs([&](int r) { return pos_s[EROWS * pass + r]; }, store_cs);
     __syncthreads();
   }
   const bool my_pass = (32 * MB * wm) / EROWS == pass;     // uniform per wavefront
