@@ -170,7 +170,8 @@ int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int sc
  * tllm_norm_qkv_rope_decode_bf16 computes them from x_out. ids: int32 or int64 [rows]; an id outside [0, vocab)
  * gives a zero row in x_out (and q / k / v computed from it) and sets *oob_flag (may be NULL), as tllm_embedding_bf16 does.
  * w_scale: NULL for a bf16 W, else W holds fp8 bytes as in tllm_qkv_rope_decode_w8_bf16. norm_scale must not be
- * NULL; hidden 2880, head_dim 64, rows <= 16 (larger batches: gather, then the QKV entry point). */
+ * NULL; hidden 2880, head_dim 64, rows <= 16 (larger batches: gather, then the QKV entry point), table smaller than
+ * 4 GiB (the kernel addresses its rows with 32-bit byte offsets; TLLM_E_SHAPE otherwise). */
 int tllm_embed_norm_qkv_rope_decode_bf16(const void* ids, int ids_is_i64, const void* table, int64_t vocab, void* x_out,
                                          int32_t* oob_flag, const void* norm_scale, int scale_is_bf16, float eps,
                                          const void* W, const float* w_scale, const void* b, void* q, void* k, void* v,

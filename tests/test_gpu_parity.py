@@ -351,6 +351,20 @@ def test_embed_norm_qkv_fp8_weight_and_bad_ids(gpu, yarn):
     assert x.data_ptr() == xo.data_ptr() and torch.equal(xo.cpu(), table[ids])
 
 
+def test_embed_qkv_refuses_a_table_beyond_32_bit_offsets(gpu):
+    """The fused gather addresses table rows with 32-bit byte offsets: a table of 4 GiB or more is refused before
+    anything is launched (the pointers below are never dereferenced)."""
+    from tritonllm_amd import _lib
+    L = _lib.lib()
+    t = torch.zeros(8 * 5120, dtype=torch.bfloat16, device=gpu)
+    ids = torch.zeros(8, dtype=torch.int32, device=gpu)
+    scale = torch.ones(2880, dtype=torch.float32, device=gpu)
+    p = t.data_ptr()
+    rc = L.tllm_embed_norm_qkv_rope_decode_bf16(ids.data_ptr(), 0, p, 745655, p, None, scale.data_ptr(), 0, 1e-5, p, None, None, p, p, p,
+                                                4096, 512, 512, 0, 8, 2880, 64, 8, 64, None, None)
+    assert rc == -2 and b"too large for the fused gather" in L.tllm_last_error()
+
+
 @pytest.mark.parametrize("id_dtype", [torch.int32, torch.int64])
 def test_embed_qkv_bad_ids_same_policy_either_side_of_16_rows(gpu, yarn, id_dtype):
     """One launch (<= 16 rows) and gather + QKV (> 16 rows) behind the same call treat an id outside the table alike: a

@@ -583,55 +583,51 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 
 using namespace tllm;
 
-static void launch_cu_embed(int xr, int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
-#define TLLM_CUE(XR, NORM)                                                                                          \
+// The kernel above serves what the two streaming kernels do not: the fused norm (and gather) at 9..16 rows, and the
+// fused-norm entry point called with more than 16 rows.
+static void launch_cu_embed(int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+#define TLLM_CUE(NORM)                                                                                              \
   do {                                                                                                              \
-    if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, 3, NORM, true, true>), grid, dim3(960), 0, st, a, ra, fr);  \
-    else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, 3, NORM, false, true>), grid, dim3(960), 0, st, a, ra, fr);    \
+    if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<16, 3, NORM, true, true>), grid, dim3(960), 0, st, a, ra, fr);  \
+    else hipLaunchKernelGGL((qkv_decode_cu_kernel<16, 3, NORM, false, true>), grid, dim3(960), 0, st, a, ra, fr);    \
   } while (0)
-  if (xr == 8) {
-    if (norm == 1) TLLM_CUE(8, 1);
-    else TLLM_CUE(8, 2);
-  } else {
-    if (norm == 1) TLLM_CUE(16, 1);
-    else TLLM_CUE(16, 2);
-  }
+  if (norm == 1) TLLM_CUE(1);
+  else TLLM_CUE(2);
 #undef TLLM_CUE
 }
 
 static void launch_cu(int xr, int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
-#define TLLM_CU1(XR, CH, NORM)                                                                                  \
+#define TLLM_CU(XR, CH, NORM)                                                                                   \
   do {                                                                                                          \
     if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, true>), grid, dim3(960), 0, st, a, ra, fr);  \
     else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, false>), grid, dim3(960), 0, st, a, ra, fr);    \
   } while (0)
-#define TLLM_CU(XR, CH)                \
-  do {                                 \
-    if (norm == 0) TLLM_CU1(XR, CH, 0); \
-    else if (norm == 1) TLLM_CU1(XR, CH, 1); \
-    else TLLM_CU1(XR, CH, 2);          \
-  } while (0)
-  if (xr == 8) TLLM_CU(8, 3);
-  else if (xr == 16) TLLM_CU(16, 3);
-  else TLLM_CU(32, 2);
+  if (xr == 16) {
+    if (norm == 1) TLLM_CU(16, 3, 1);
+    else TLLM_CU(16, 3, 2);
+  } else {
+    if (norm == 1) TLLM_CU(32, 2, 1);
+    else TLLM_CU(32, 2, 2);
+  }
 #undef TLLM_CU
-#undef TLLM_CU1
 }
 
 // Shared tail of the hidden-2880 decode entry points: row-count -> kernel variant and grid.
 static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, int norm, bool w8, int64_t rows,
                               int heads, hipStream_t st) {
   TLLM_REQUIRE(static_cast<int64_t>(heads) * 64 * 2880 < (1ll << 31), TLLM_E_SHAPE, "%s: weight too large", what);
-  // the activations are addressed with 32-bit byte offsets in the two kernels that load straight into LDS
-  const bool fits32 = (a.emb_ids ? a.emb_vocab : rows) * 5760 < (1ll << 32);
-  const bool r32 = rows > 8 && norm == 0 && !a.emb_ids && fits32;          // 9..32 rows per workgroup, normalised activations
+  const bool emb = a.emb_ids != nullptr;
+  // the fused gather addresses table rows with 32-bit byte offsets
+  TLLM_REQUIRE(!emb || a.emb_vocab * 5760 < (1ll << 32), TLLM_E_SHAPE, "%s: embedding table of %lld rows too large for the fused gather", what,
+               (long long)a.emb_vocab);
+  const bool r32 = rows > 8 && norm == 0 && !emb;                          // 9..32 rows per workgroup, normalised activations
   const int xr = rows <= 8 ? 8 : ((rows <= 16 && !r32) ? 16 : 32);
   const int64_t chunks = (rows + xr - 1) / xr;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
   const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
   if (r32) launch_qkv_decode_r32(w8, grid, st, a, ra, fr);
-  else if (xr == 8 && fits32) launch_qkv_decode_r8(norm, a.emb_ids != nullptr, w8, grid, st, a, ra, fr);
-  else if (a.emb_ids) launch_cu_embed(xr, norm, w8, grid, st, a, ra, fr);
+  else if (xr == 8) launch_qkv_decode_r8(norm, emb, w8, grid, st, a, ra, fr);
+  else if (emb) launch_cu_embed(norm, w8, grid, st, a, ra, fr);
   else launch_cu(xr, norm, w8, grid, st, a, ra, fr);
   return check_launch(what);
 }

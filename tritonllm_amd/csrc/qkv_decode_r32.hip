@@ -77,7 +77,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int r = 4 * j + (lane >> 4);
-    const int64_t src = row0 + (r < nvalid ? r : nvalid - 1);
+    const int src = r < nvalid ? r : nvalid - 1;            // row inside the workgroup's 32 (the base below points at row0)
     const int cc = (lane & 15) ^ (r & 15);
     xoff[j] = static_cast<unsigned>(src * 5760 + kq * 256 + cc * 16);
     xoff3[j] = static_cast<unsigned>(src * 5760 + kq * 192 + (cc < 12 ? cc : 11) * 16);
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
       goff3[j] = wrow * 5760u + kq * 192u + (cc < 12 ? cc : 11) * 16u;
     }
   }
-  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x);
+  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x) + row0 * 5760;
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
   auto issue_phase = [&](int p) {                           // thirteen loads: the activations of the phase, then its weight

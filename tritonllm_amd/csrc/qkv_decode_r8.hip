@@ -126,12 +126,13 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // activations: row n of the slice -> 1 KB block n; lane i fetches chunk i ^ 2n (60 real chunks, the rest re-read
   // chunk 59), the swizzle that spreads the eight rows of a fragment read over the banks
   unsigned xoff[XR];
-  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(EMB ? a.emb_table : a.x);
+  // 32-bit lane offsets from a scalar base: the workgroup's first row, or (EMB) the table, whose size the host checks
+  const unsigned char* xbase = EMB ? reinterpret_cast<const unsigned char*>(a.emb_table) : reinterpret_cast<const unsigned char*>(a.x) + row0 * 5760;
   bool xok_m1 = true;                                       // EMB: is the id of the row this lane's fragments belong to inside the table?
   {
     int64_t src_row[XR];
 #pragma unroll
-    for (int n = 0; n < XR; ++n) src_row[n] = row0 + (n < nvalid ? n : nvalid - 1);
+    for (int n = 0; n < XR; ++n) src_row[n] = (EMB ? row0 : 0) + (n < nvalid ? n : nvalid - 1);   // EMB: index into the ids; else row inside the workgroup
     if constexpr (EMB) {
       int64_t id[XR];
 #pragma unroll
