@@ -382,7 +382,8 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
     assert ids.ndim == 1 and ids.dtype in (torch.int32, torch.int64)
     assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
     rows, (vocab, hidden) = ids.shape[0], table.shape
-    fused = 0 < rows <= EMBED_FUSED_MAX_ROWS and hidden == 2880 and head_dim == 64
+    # (the one-launch kernel addresses table rows with 32-bit byte offsets: tables of 4 GiB and more take the two launches)
+    fused = 0 < rows <= EMBED_FUSED_MAX_ROWS and hidden == 2880 and head_dim == 64 and vocab * hidden * 2 < 2 ** 32
     if x_out is None:
         x_out = torch.empty(rows, hidden, dtype=_BF16, device=table.device)
     assert x_out.shape == (rows, hidden) and x_out.dtype == _BF16 and x_out.is_contiguous()
