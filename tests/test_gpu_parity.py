@@ -255,9 +255,15 @@ def _check_qkv(gpu, yarn, rows, mode, seed, prefill_positions=False, max_pos=819
     close(v, vr)
 
 
-@pytest.mark.parametrize("rows", [1, 8, 15, 16, 17, 32, 50])
+@pytest.mark.parametrize("rows", [1, 8, 15, 16, 17, 32, 50, 100, 192])
 def test_qkv_rope_decode_parity(gpu, yarn, rows):
     _check_qkv(gpu, yarn, rows, "decode", seed=rows)
+
+
+@pytest.mark.parametrize("rows", [64, 65, 192, 193])
+def test_qkv_rope_auto_mode_either_side_of_the_row_threshold(gpu, yarn, rows):
+    """``mode="auto"``: the weight-streaming kernel up to 192 rows at the gpt-oss shape, the MFMA GEMM above."""
+    _check_qkv(gpu, yarn, rows, "auto", seed=40 + rows)
 
 
 @pytest.mark.parametrize("rows", [1, 100, 128, 200, 2048])

@@ -35,6 +35,13 @@ _BF16 = torch.bfloat16
 
 # rows at or below this use the weight-streaming decode kernel, above it the MFMA GEMM
 DECODE_MAX_ROWS = 64
+# At the gpt-oss shape the streaming kernel takes 32 rows per pass over the weight, ~7.5 us a pass (96 rows 23 us, 128
+# rows 30 us), where the GEMM's one round of tiles costs 48-56 us however few rows there are: they meet near 224 rows.
+DECODE_MAX_ROWS_2880 = 192
+
+
+def _decode_max_rows(hidden: int, head_dim: int) -> int:
+    return DECODE_MAX_ROWS_2880 if hidden == 2880 and head_dim == 64 else DECODE_MAX_ROWS
 
 
 def _stream() -> int:
@@ -353,7 +360,7 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
         desc = _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch if tokens_per_batch else max(rows, 1),
                           max_context_length, keep, rows)
     if mode == "auto":
-        mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
+        mode = "decode" if rows <= _decode_max_rows(x.shape[-1], head_dim) else "prefill"
     assert mode in ("decode", "prefill")
     _launch_qkv(mode, x, weight, bias, q, k, v, q.stride(0), k.stride(0), v.stride(0), 0, num_q_heads, num_kv_heads, head_dim, desc,
                 norm=None if norm_scale is None else (norm_scale, norm_eps),
@@ -504,7 +511,7 @@ def linear_qkv_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     assert total_out % hd == 0
     out = torch.empty((*x.shape[:-1], total_out), dtype=x.dtype, device=x.device)
     o2 = out.view(rows, total_out)
-    mode = "decode" if rows <= DECODE_MAX_ROWS else "prefill"
+    mode = "decode" if rows <= _decode_max_rows(hidden, hd) else "prefill"
     # all columns as "q heads" of one dense output row
     _launch_qkv(mode, x2, weight, bias, o2, None, None, total_out, 0, 0, 0, total_out // hd, 0, hd, None)
     return out
