@@ -45,10 +45,32 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
   if (wave >= NS) {
     // ======================================================================= epilogue wavefront of (tile, column block)
     const int tile = (wave - NS) & 1, cb = (wave - NS) >> 1;
+    // L2 warm-up for the later phases. The activations were written by the kernel before this one, so no XCD's L2
+    // holds them yet; the streaming wavefronts of all CUs ask for a phase at about the same time and wait for it at
+    // memory latency. The first epilogue wavefront of each of the 32 workgroups of an XCD (consecutive workgroup ids go
+    // to consecutive XCDs) touches 1/32 of the rows' bytes now -- a handful of loads per CU -- so that by the time
+    // phases 2 and 3 are requested their lines sit in the XCD's L2.
+    f32x4 warm[6];
+    if (wave == NS) {
+      const unsigned total = static_cast<unsigned>(nvalid) * 5760u;          // bytes of this workgroup's rows (contiguous)
+      const unsigned share = ((total + 31u) / 32u + 1023u) & ~1023u;         // per workgroup of the XCD, whole 1 KB loads
+      const unsigned first = ((blockIdx.x >> 3) & 31u) * share;
+      const unsigned char* xr = reinterpret_cast<const unsigned char*>(a.x) + row0 * 5760;
+#pragma unroll
+      for (int j = 0; j < 6; ++j) {
+        unsigned o = first + j * 1024u + lane * 16u;
+        o = o < total - 16u ? o : total - 16u;
+        warm[j] = *reinterpret_cast<const f32x4*>(xr + o);
+      }
+    }
     StreamEpilogueLane<W8> ep;
     ep.prepare(a, ra, fr, pair0, tile, lane >> 4, 16 * cb + (lane & 15), row0, nvalid);   // quad of the tile, activation row
     unsigned red_o = static_cast<unsigned>((2 * tile + cb) * 1024 + lane * 16);
     asm volatile("" : "+v"(red_o));
+    if (wave == NS) {
+#pragma unroll
+      for (int j = 0; j < 6; ++j) asm volatile("" ::"v"(warm[j]));          // the values themselves are not needed
+    }
     __syncthreads();                                        // partial tiles are in LDS
     f32x4 t[NS];
 #pragma unroll
