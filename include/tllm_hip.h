@@ -154,15 +154,22 @@ int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const void* b,
  * hidden state, the kernel normalises it (fp32, one RNE to bf16 -- the operand the two
  * separate calls would pass between them) while the weight streams in.
  * replaces the pair AttentionBlock.forward issues per decode step, model.py:476 + 489-503.
- * Exists for hidden == 2880, head_dim == 64 (TLLM_E_SHAPE otherwise). Worth it up to 16
- * rows; beyond that the kernel's 32-row variant is short of registers and the two
- * separate calls are the faster form (the result is the same either way). */
+ * Exists for hidden == 2880, head_dim == 64 (TLLM_E_SHAPE otherwise). Up to 16 rows per
+ * workgroup the norm runs inside the weight-streaming kernels; with more rows the call is
+ * the two launches it replaces (RMSNorm into a caller-invisible buffer is not possible
+ * without allocating, so more than 16 rows return TLLM_E_SHAPE: issue the two calls). */
 int tllm_norm_qkv_rope_decode_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps,
                                    const void* W, const void* b, void* q, void* k, void* v,
                                    int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,
                                    int64_t kv_slot_stride,
                                    int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
                                    const TllmRope* rope, void* stream);
+
+/* Diagnostic of the fused-norm decode kernels: inside them the wavefronts of a workgroup wait for one another's
+ * partial sums with a bounded poll. *expired becomes 1 if any such wait ever ran out on the current device since the
+ * library was loaded (the launch then finished with wrong sums instead of hanging), else 0. Synchronises the device.
+ * No counterpart in the reference. */
+int tllm_qkv_decode_wait_expired(int32_t* expired);
 
 /* The first layer of a decode step in one launch: token-embedding gather (torch.nn.Embedding, model.py:906-908, 920)
  * feeding the first block's RMSNorm + QKV + bias + rotary (model.py:476, 489-503). x_out[r, :] = table[ids[r], :]
@@ -237,8 +244,13 @@ int tllm_unembedding_argmax_bf16(const void* x, const void* W, const float* w_sc
  * tllm_unembedding_argmax_noalloc_max_rows() = 16; more rows return TLLM_E_SHAPE. The call allocates nothing and
  * gives the same token_ids as tllm_unembedding_argmax_bf16. All calls on one GPU share the array: calls that may run
  * concurrently on one GPU (different streams without ordering between them) race on it and must be serialised by the
- * caller. Nothing in the array needs clearing between calls. */
+ * caller. Nothing in the array needs clearing between calls.
+ * The array's device address is looked up once per GPU, by a runtime query that is not allowed while a stream is
+ * capturing: tllm_unembedding_argmax_noalloc_init() does it for the current device and is to be called (once per
+ * device, outside any capture) by callers that capture. Without it the first eager call on a device does the look-up,
+ * and a first call on a capturing stream returns TLLM_E_ARG instead of disturbing the capture. */
 int64_t tllm_unembedding_argmax_noalloc_max_rows(void);
+int tllm_unembedding_argmax_noalloc_init(void);
 int tllm_unembedding_argmax_noalloc_bf16(const void* x, const void* W, const float* w_scale, int32_t* token_ids,
                                          int64_t rows, int64_t hidden, int64_t vocab, void* stream);
 

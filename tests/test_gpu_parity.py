@@ -225,12 +225,12 @@ def test_yarn_table_whole_context(gpu, scaling_factor):
 def test_rope_positions_must_cover_every_row(gpu, yarn):
     """The kernels read positions[row] for every row; a shorter tensor is refused on the host."""
     q, k = _qk(4, 1, seed=14)
-    with pytest.raises(AssertionError):
+    with pytest.raises(ValueError, match="3 entries for 4 rows"):
         T.rope_forward(q.to(gpu), k.to(gpu), None, None, O.MAX_CTX, None, yarn=yarn, positions=torch.zeros(3, dtype=torch.int64, device=gpu))
     d = O.make_inputs(8, seed=15)
-    with pytest.raises(AssertionError):
+    with pytest.raises(ValueError, match="7 entries for 8 rows"):
         T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"][:7].to(gpu))
-    with pytest.raises((AssertionError, RuntimeError)):
+    with pytest.raises((ValueError, RuntimeError)):
         T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"])   # CPU positions
 
 
@@ -403,19 +403,22 @@ def test_embed_qkv_bad_ids_same_policy_either_side_of_16_rows(gpu, yarn, id_dtyp
         assert flag.item() == 0
 
 
-@pytest.mark.parametrize("rows", [17, 32, 50])
-def test_norm_qkv_fused_entry_point_beyond_16_rows(gpu, yarn, rows, monkeypatch):
-    """The host picks two launches beyond 16 rows (faster there); the C entry point itself must still be right."""
+@pytest.mark.parametrize("rows", [17, 50])
+def test_norm_qkv_fused_entry_point_refuses_more_than_16_rows(gpu, yarn, rows, monkeypatch):
+    """Beyond 16 rows the norm is a launch of its own: the host composes the two, the C entry point says so."""
     from tritonllm_amd import ops
-    monkeypatch.setattr(ops, "_norm_fusable", lambda kind, r, hidden, hd: kind == "decode" and hidden == 2880 and hd == 64)
     d = O.make_inputs(rows, seed=400 + rows)
-    q, k, v = T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu),
-                                 mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    args = (d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64)
+    kw = dict(yarn=yarn, positions=d["positions"].to(gpu), mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    q, k, v = T.qkv_rope_forward(*args, **kw)                     # two launches
     t_ref = O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16()
     qr, kr, vr = O.qkv_rope_ref(t_ref, d["w"], d["b"], d["positions"])
     close(q, qr)
     close(k, kr)
     close(v, vr)
+    monkeypatch.setattr(ops, "_norm_fusable", lambda kind, r, hidden, hd: kind == "decode" and hidden == 2880 and hd == 64)
+    with pytest.raises(RuntimeError, match="up to 16 rows"):
+        T.qkv_rope_forward(*args, **kw)
 
 
 @pytest.mark.parametrize("rows", [1, 8, 13, 16, 32, 40])
@@ -483,6 +486,22 @@ def test_streaming_decode_kernels_every_row_count(gpu, yarn, rows):
         T.out_residual_decode_forward(nan_ox, weight, ob, torch.zeros(full, 1, 2880, dtype=torch.bfloat16, device=gpu), weight_scale=wscale)
         out = T.out_residual_decode_forward(oxbuf[:rows].view(rows, 1, 4096), weight, ob, o["r"].view(rows, 1, 2880).to(gpu), weight_scale=wscale)
         close(out.view(rows, 2880), O.out_residual_ref(o["x"], wref, o["b"], o["r"]))
+
+
+def test_fused_norm_wait_for_the_other_wavefronts_never_expires(gpu, yarn):
+    """Inside the fused-norm decode kernels a wavefront waits for the others' partial sums with a bounded poll; a wait
+    that runs out is recorded in a device word. After the row-count cases above (and a few more here) it must be 0."""
+    import ctypes
+    from tritonllm_amd import _lib
+    for rows in (1, 5, 8, 11, 16):
+        d = O.make_inputs(rows, seed=1200 + rows)
+        for _ in range(20):
+            T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, yarn=yarn, positions=d["positions"].to(gpu),
+                               mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    expired = ctypes.c_int32(-1)
+    assert _lib.lib().tllm_qkv_decode_wait_expired(ctypes.byref(expired)) == 0, _lib.lib().tllm_last_error()
+    assert expired.value == 0
+    assert _lib.lib().tllm_qkv_decode_wait_expired(None) == -1
 
 
 def test_qkv_fp8_weight_cache_form_module_and_refusals(gpu, yarn, monkeypatch):

@@ -91,3 +91,41 @@ def test_noalloc_argmax_full_vocabulary_and_limits(gpu):
     assert rc == -2 and b"at most 16 rows" in L.tllm_last_error()
     assert L.tllm_unembedding_argmax_noalloc_bf16(x.data_ptr(), w.data_ptr(), None, None, rows, hidden, vocab, stream) == -1
     assert L.tllm_unembedding_argmax_noalloc_bf16(None, None, None, None, 0, hidden, vocab, stream) == 0
+
+
+def test_noalloc_argmax_replays_in_a_captured_graph(gpu):
+    """The use the entry point is for: after the per-device set-up call, the launch is captured in a HIP graph and
+    replayed with new activations; every replay must give the token ids of the workspace form on the same input."""
+    L = _lib.lib()
+    assert L.tllm_unembedding_argmax_noalloc_init() == 0, L.tllm_last_error()
+    rows, vocab, hidden = 8, 6001, O.HIDDEN
+    g = torch.Generator().manual_seed(11)
+    w = (0.02 * torch.randn(vocab, hidden, generator=g)).bfloat16().to(gpu)
+    xs = [torch.randn(rows, hidden, generator=g).bfloat16().to(gpu) for _ in range(3)]
+    x = xs[0].clone()
+    ids = torch.full((rows,), -1, dtype=torch.int32, device=gpu)
+    nbytes = L.tllm_unembedding_argmax_workspace_bytes(rows)
+    work = torch.empty(nbytes, dtype=torch.uint8, device=gpu)
+    ids_ws = torch.full((rows,), -1, dtype=torch.int32, device=gpu)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = L.tllm_unembedding_argmax_noalloc_bf16(x.data_ptr(), w.data_ptr(), None, ids.data_ptr(), rows, hidden, vocab,
+                                                        torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, L.tllm_last_error()
+    torch.cuda.current_stream().wait_stream(side)
+    for xi in xs[1:] + xs[:1]:
+        x.copy_(xi)
+        ids.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        rc = L.tllm_unembedding_argmax_bf16(xi.data_ptr(), w.data_ptr(), None, work.data_ptr(), nbytes, ids_ws.data_ptr(), rows, hidden, vocab,
+                                            torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, L.tllm_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(ids, ids_ws), (ids.tolist(), ids_ws.tolist())
+        want = O.linear_ref(xi.cpu(), w.cpu(), None)
+        got = want.gather(1, ids.cpu().long()[:, None])[:, 0]
+        assert (want.max(dim=1).values - got <= 1e-3).all()

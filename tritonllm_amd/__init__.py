@@ -21,6 +21,7 @@ from .ops import (
     swiglu,
     unembedding_decode_argmax_forward,
     unembedding_decode_argmax_noalloc,
+    unembedding_decode_argmax_noalloc_init,
     unembedding_decode_forward,
     unembedding_decode_fp8_argmax_forward,
     unembedding_decode_fp8_forward,
@@ -32,6 +33,6 @@ from .yarn import YarnParams, gpt_oss_yarn
 __all__ = [
     "Checkpoint", "OUT", "QKV", "Embedding", "RMSNorm", "RotaryEmbedding", "YarnParams", "gpt_oss_yarn", "scratch_pool",
     "attention", "attention_decode", "embed_qkv_rope_forward", "embedding_forward", "embedding_rmsnorm_forward", "linear_qkv_forward", "mxfp4_dequant", "out_residual_decode_forward", "qkv_decode_forward", "qkv_rope_cache_decode_forward",
-    "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu", "UnEmbedding", "unembedding_decode_forward", "unembedding_decode_argmax_forward", "unembedding_decode_argmax_noalloc",
+    "qkv_rope_forward", "quantize_fp8_rows", "rmsnorm_forward", "rope_forward", "swiglu", "UnEmbedding", "unembedding_decode_forward", "unembedding_decode_argmax_forward", "unembedding_decode_argmax_noalloc", "unembedding_decode_argmax_noalloc_init",
     "unembedding_decode_fp8_forward", "unembedding_decode_fp8_argmax_forward", "unembedding_forward",
 ]

@@ -47,12 +47,14 @@ SIGNATURES = {
     "tllm_qkv_rope_decode_bf16": (_i32, _QKV_SIG),
     "tllm_qkv_rope_prefill_bf16": (_i32, _QKV_SIG),
     "tllm_norm_qkv_rope_decode_bf16": (_i32, [_vp, _vp, _i32, _f32] + _QKV_SIG[1:]),
+    "tllm_qkv_decode_wait_expired": (_i32, [_vp]),
     "tllm_embed_norm_qkv_rope_decode_bf16": (_i32, [_vp, _i32, _vp, _i64, _vp, _vp, _vp, _i32, _f32, _vp, _vp] + _QKV_SIG[2:]),
     "tllm_out_residual_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "tllm_unembedding_decode_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "tllm_unembedding_argmax_workspace_bytes": (_i64, [_i64]),
     "tllm_unembedding_argmax_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "tllm_unembedding_argmax_noalloc_max_rows": (_i64, []),
+    "tllm_unembedding_argmax_noalloc_init": (_i32, []),
     "tllm_unembedding_argmax_noalloc_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "tllm_attention_decode_splits": (_i32, [_i64, _i32, _i64, _i32]),
     "tllm_attention_decode_heads_per_workgroup": (_i32, [_i64, _i32, _i64, _i32]),

@@ -160,7 +160,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnPrefillArgs a)
         g = dma_src + static_cast<int64_t>(key) * a.kv_ts + dma_col[j];
       }
       const unsigned m0v = lds0 + stage * PSTAGE + j * 1024;
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
     }
   };
   // wait until all but the `behind` youngest blocks' loads of this wavefront have landed, then meet the others

@@ -154,7 +154,7 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
       const unsigned dst = lds_addr(phase_region(p) + j * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff[j]), "s"(sb) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff[j]), "s"(sb) : "memory", "m0");
     }
   };
 
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(576) void out_decode_r8_kernel(OutArgs a, int vec8)
     // that stays in output columns nobody stores. Fewer loads ahead of a wait only make it less strict than written.
     if (n < nvalid) {
       const unsigned dst = lds_addr(myx + n * XBLOCK);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
     }
   }
 #pragma unroll

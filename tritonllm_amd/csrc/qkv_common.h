@@ -50,13 +50,14 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
                  int64_t k_rs, int64_t v_rs, int64_t kv_slot_stride, int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads,
                  int head_dim, const TllmRope* rope, QkvArgs* a, RopeArgs* ra, YarnFreqs* fr);
 
-// Any hidden size, any even head_dim: one workgroup per (head, row); each wavefront takes
-// rotation pairs (d, d + hd/2) in turn and reduces the two dot products by shuffle.
-// The hidden-2880 decode kernel for up to 8 rows per workgroup, bf16 weight (qkv_decode_r8.hip).
+// The hidden-2880 decode kernel for up to 8 rows per workgroup: bf16 or fp8 weight, optional fused RMSNorm and token
+// gather (qkv_decode_r8.hip).
 void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
-// ... and for 9..32 rows per workgroup, activations already normalised (qkv_decode_r32.hip).
+// ... and for 9..32 rows per workgroup, bf16 or fp8 weight, activations already normalised (qkv_decode_r32.hip).
 void launch_qkv_decode_r32(bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 
+// Any hidden size, any even head_dim: one workgroup per (head, row); each wavefront takes
+// rotation pairs (d, d + hd/2) in turn and reduces the two dot products by shuffle.
 void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, hipStream_t st);
 
 }  // namespace tllm

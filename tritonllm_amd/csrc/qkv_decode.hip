@@ -583,8 +583,7 @@ __global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs 
 
 using namespace tllm;
 
-// The kernel above serves what the two streaming kernels do not: the fused norm (and gather) at 9..16 rows, and the
-// fused-norm entry point called with more than 16 rows.
+// The kernel above serves what the two streaming kernels do not: the fused norm (and gather) at 9..16 rows.
 static void launch_cu_embed(int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
 #define TLLM_CUE(NORM)                                                                                              \
   do {                                                                                                              \
@@ -602,13 +601,9 @@ static void launch_cu(int xr, int norm, bool w8, dim3 grid, hipStream_t st, cons
     if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, true>), grid, dim3(960), 0, st, a, ra, fr);  \
     else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, false>), grid, dim3(960), 0, st, a, ra, fr);    \
   } while (0)
-  if (xr == 16) {
-    if (norm == 1) TLLM_CU(16, 3, 1);
-    else TLLM_CU(16, 3, 2);
-  } else {
-    if (norm == 1) TLLM_CU(32, 2, 1);
-    else TLLM_CU(32, 2, 2);
-  }
+  (void)xr;                                                               // 16: the only height left
+  if (norm == 1) TLLM_CU(16, 3, 1);
+  else TLLM_CU(16, 3, 2);
 #undef TLLM_CU
 }
 
@@ -670,6 +665,11 @@ static int decode_2880_entry(const char* what, const void* x, const void* norm_s
   TLLM_REQUIRE(aligned16(x) && aligned16(W) && aligned16(norm_scale), TLLM_E_ALIGN, "%s: x, W and norm_scale must be 16-byte aligned", what);
   TLLM_REQUIRE(!w8 || (w_scale != nullptr && reinterpret_cast<uintptr_t>(w_scale) % 4 == 0), TLLM_E_ARG,
                "%s: w_scale must be a 4-byte aligned device pointer", what);
+  // 32 rows of raw activations do not fit next to the weight ring, and a row's factor is needed before its first
+  // product: above 16 rows the norm is a launch of its own, which this library cannot insert (it owns no buffer).
+  TLLM_REQUIRE(norm_scale == nullptr || rows <= 16, TLLM_E_SHAPE,
+               "%s: the fused RMSNorm exists for up to 16 rows (got %lld): call tllm_rmsnorm_bf16, then the projection without norm_scale",
+               what, (long long)rows);
   a.bias = (const bf16*)b;
   a.norm_scale = norm_scale;
   a.norm_eps = eps;

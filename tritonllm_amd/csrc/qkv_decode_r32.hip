@@ -141,13 +141,13 @@ __global__ __launch_bounds__(640) void qkv_decode_r32_kernel(QkvArgs a, RopeArgs
       // (the waits below count the loads of the phase after the one they wait for, so they depend on xblocks).
       if (j < xblocks) {
         const unsigned dst = lds_addr(reg + j * 1024);
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(p == 3 ? xoff3[j] : xoff[j]), "s"(xb) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(p == 3 ? xoff3[j] : xoff[j]), "s"(xb) : "memory", "m0");
       }
     }
 #pragma unroll
     for (int j = 0; j < LW; ++j) {
       const unsigned dst = lds_addr(reg + XPH + j * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == 3 ? goff3[j] : goff[j]), "s"(wb) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == 3 ? goff3[j] : goff[j]), "s"(wb) : "memory", "m0");
     }
   };
   issue_phase(0);

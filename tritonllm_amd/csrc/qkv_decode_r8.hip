@@ -50,6 +50,10 @@ constexpr int REGION = 20 * 256;  // one phase: 20 weight rows x four k32 steps
 constexpr int XBLOCK = 1024;      // one activation row of a slice: 60 chunks of 16 bytes (+ 4 spare)
 }  // namespace r8
 
+// Set (and never cleared) by a wavefront whose bounded wait for the other wavefronts' norm sums ran out.
+__device__ int g_qkv_decode_wait_expired = 0;
+constexpr int kFlagPollLimit = 1 << 18;
+
 #ifdef TLLM_R8_STAMPS
 __device__ unsigned long long g_r8_stamps[256 * 8 * 8];
 #define R8_STAMP(i) do { if (lane == 0 && blockIdx.y == 0 && blockIdx.x < 256) g_r8_stamps[(blockIdx.x * 8 + wave) * 8 + (i)] = wall_clock64(); } while (0)
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
       const unsigned dst = lds_addr(phase_region(p) + j * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == NPH - 1 ? goff3[j] : goff[j]), "s"(sb) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(p == NPH - 1 ? goff3[j] : goff[j]), "s"(sb) : "memory", "m0");
     }
   };
 
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     // of a wait only make it less strict than written: the counts below are relative to the youngest loads.
     if (n < nvalid) {
       const unsigned dst = lds_addr(myx + n * XBLOCK);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[n]), "s"(xbase) : "memory", "m0");
     }
   }
   constexpr int NSC = NORM == 1 ? 2 : (NORM == 2 ? 1 : 0);   // scale loads: 480 fp32 = 120 chunks, 480 bf16 = 60 chunks
@@ -211,7 +215,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
       c = c < cmax ? c : cmax;
       const unsigned off = NORM == 1 ? 2u * kb(c >> 1) + (c & 1) * 16u : static_cast<unsigned>(kb(c));
       const unsigned dst = lds_addr(scw + wave * 2048 + t * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(sbase) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(sbase) : "memory", "m0");
     }
   }
   // A CU takes only so many loads at a time; a wavefront that issues one more simply stalls until the queue has
@@ -290,9 +294,17 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     if (lane == 0) __hip_atomic_store(&s_flag[wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #pragma unroll
     for (int p = EARLY; p < NPH; ++p) issue_phase(p);
-    for (;;) {                                              // every streaming wavefront raises its flag before it gets here or exits
+    // Every streaming wavefront raises its flag before it gets here and none returns early, so the flags are up
+    // after a few polls. The wait is bounded all the same: a wavefront that has polled kFlagPollLimit times (tens of
+    // milliseconds) records that in g_qkv_decode_wait_expired and carries on to the kernel's barriers and exit with
+    // whatever sums it has -- a wrong result the host can see instead of a workgroup that never ends.
+    for (int polls = 0;; ++polls) {
       const unsigned f = lane < NS ? __hip_atomic_load(&s_flag[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : 1u;
       if (__all(f != 0u)) break;
+      if (polls >= kFlagPollLimit) {
+        if (lane == 0) g_qkv_decode_wait_expired = 1;
+        break;
+      }
       __builtin_amdgcn_s_sleep(2);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -407,6 +419,15 @@ void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st
 }
 
 }  // namespace tllm
+
+extern "C" int tllm_qkv_decode_wait_expired(int32_t* expired) {
+  TLLM_REQUIRE(expired != nullptr, TLLM_E_ARG, "qkv_decode_wait_expired: expired is NULL");
+  int v = 0;
+  const hipError_t e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(tllm::g_qkv_decode_wait_expired), sizeof(v));
+  TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_decode_wait_expired: %s", hipGetErrorString(e));
+  *expired = v;
+  return TLLM_OK;
+}
 
 #ifdef TLLM_R8_STAMPS
 extern "C" int tllm_debug_r8_stamps(void* host, size_t bytes) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tllm::g_r8_stamps), bytes); }

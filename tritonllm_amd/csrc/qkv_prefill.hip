@@ -233,7 +233,7 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
     // fewer registers in the two tile heights and 2-3 % faster. The lanes' 16 bytes land at M0 + 16 * lane.
     const unsigned lds_off = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst + blk_off[j]));
     const unsigned char* sb = (is_x ? x_base : w_base) + static_cast<int64_t>(slc) * (BK * 2);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
   };
   auto issue_period = [&](int per) {
 #pragma unroll

@@ -1,26 +1,32 @@
 // Half-split (NeoX-style) rotary embedding applied in place to q and k, and the
 // YaRN cos/sin table builder.
 //
-// A workgroup owns kTok consecutive tokens. The cos/sin of a (token, frequency) pair is
-// needed by every head of that token, so the first kTok*n_freq lanes compute them once
+// A workgroup owns TOK consecutive tokens. The cos/sin of a (token, frequency) pair is
+// needed by every head of that token, so the first TOK*n_freq lanes compute them once
 // (in registers, from the YaRN parameters, or by reading the caller's table) into LDS;
 // after one barrier all 256 lanes stream the heads: each work item is the pair of
 // 128-bit vectors (dims d..d+7, dims d+hd/2..d+hd/2+7) of one head, rotated in fp32 and
 // stored back with one round-to-nearest-even per output.
+// Prompts take four tokens per workgroup (the cos/sin work is shared by more items). A decode
+// batch is a handful of tokens: there a workgroup takes one token (the reference makes the same
+// switch below 60 tokens, triton_kernels.py:94-107) and gridDim.y workgroups share its heads, so
+// that every lane has one item and the launch is one load-rotate-store deep.
 #include "common.h"
 
 namespace tllm {
 
 constexpr int kRopeTok = 4;
+constexpr int kRopeSmallRows = 64;   // up to here: one token per workgroup
 
+template <int TOK>
 __global__ __launch_bounds__(256) void rope_kernel(bf16x8* q, bf16x8* k, int64_t rows, int n_q_heads, int n_kv_heads, int head_dim,
                                                    RopeArgs ra, YarnFreqs fr) {
-  __shared__ float s_cos[kRopeTok * TLLM_MAX_ROPE_FREQS];
-  __shared__ float s_sin[kRopeTok * TLLM_MAX_ROPE_FREQS];
+  __shared__ float s_cos[TOK * TLLM_MAX_ROPE_FREQS];
+  __shared__ float s_sin[TOK * TLLM_MAX_ROPE_FREQS];
   const int tid = threadIdx.x;
   const int n_freq = head_dim >> 1;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRopeTok;
-  const int ntok = static_cast<int>(rows - row0 < kRopeTok ? rows - row0 : kRopeTok);
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * TOK;
+  const int ntok = static_cast<int>(rows - row0 < TOK ? rows - row0 : TOK);
 
   for (int e = tid; e < ntok * n_freq; e += 256) {
     const int t = e / n_freq, i = e - t * n_freq;
@@ -35,7 +41,8 @@ __global__ __launch_bounds__(256) void rope_kernel(bf16x8* q, bf16x8* k, int64_t
   const int vph = n_freq >> 3;                       // 128-bit vectors per half head
   const int heads = n_q_heads + n_kv_heads;
   const int items_per_tok = heads * vph;
-  for (int it = tid; it < ntok * items_per_tok; it += 256) {
+  // the workgroups of one token group (gridDim.y of them) deal the items round-robin in runs of 256
+  for (int it = blockIdx.y * 256 + tid; it < ntok * items_per_tok; it += 256 * gridDim.y) {
     const int t = it / items_per_tok;
     const int r = it - t * items_per_tok;
     const int h = r / vph, j = r - h * vph;
@@ -91,10 +98,18 @@ extern "C" int tllm_rope_bf16(void* q, void* k, int64_t rows, int n_q_heads, int
   if (rows == 0 || n_q_heads + n_kv_heads == 0) return TLLM_OK;
   TLLM_REQUIRE(q != nullptr || n_q_heads == 0, TLLM_E_ARG, "rope: q is NULL");
   TLLM_REQUIRE(aligned16(q) && aligned16(k), TLLM_E_ALIGN, "rope: q/k must be 16-byte aligned");
+  if (rows <= kRopeSmallRows) {
+    const int items = (n_q_heads + n_kv_heads) * (head_dim >> 4);     // per token
+    int parts = (items + 255) / 256;
+    parts = parts < 1 ? 1 : (parts > 64 ? 64 : parts);
+    hipLaunchKernelGGL(rope_kernel<1>, dim3((unsigned)rows, (unsigned)parts), dim3(256), 0, static_cast<hipStream_t>(stream), (bf16x8*)q,
+                       (bf16x8*)k, rows, n_q_heads, n_kv_heads, head_dim, ra, fr);
+    return check_launch("rope");
+  }
   const int64_t blocks = (rows + kRopeTok - 1) / kRopeTok;
   TLLM_REQUIRE(blocks < (1ll << 31), TLLM_E_SHAPE, "rope: rows %lld too large", (long long)rows);
-  hipLaunchKernelGGL(rope_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), (bf16x8*)q, (bf16x8*)k, rows,
-                     n_q_heads, n_kv_heads, head_dim, ra, fr);
+  hipLaunchKernelGGL(rope_kernel<kRopeTok>, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), (bf16x8*)q, (bf16x8*)k,
+                     rows, n_q_heads, n_kv_heads, head_dim, ra, fr);
   return check_launch("rope");
 }
 

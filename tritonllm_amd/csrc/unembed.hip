@@ -384,14 +384,23 @@ namespace {
 std::mutex g_scratch_mutex;
 void* g_scratch_ptr[kMaxDevices] = {};
 
-// Device address of `scratch` on the current device (looked up on the first call per device).
-int noalloc_scratch(const char* who, void** out) {
+// Device address of `scratch` on the current device, looked up on the first call per device. The look-up is a runtime
+// query (it may load the code object), which a capturing stream does not allow: `capturing_stream`, when not null, is
+// the stream the caller is about to launch on, and an unresolved address under capture is refused instead of queried.
+int noalloc_scratch(const char* who, void** out, hipStream_t capturing_stream, bool check_capture) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   TLLM_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, TLLM_E_LAUNCH, "%s: hipGetDevice: %s (device %d)", who,
                hipGetErrorString(e), dev);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (g_scratch_ptr[dev] == nullptr) {
+    if (check_capture) {
+      hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+      e = hipStreamIsCapturing(capturing_stream, &cs);
+      TLLM_REQUIRE(e == hipSuccess && cs == hipStreamCaptureStatusNone, TLLM_E_ARG,
+                   "%s: first use on device %d inside a stream capture: call tllm_unembedding_argmax_noalloc_init() on this device "
+                   "before capturing", who, dev);
+    }
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     TLLM_REQUIRE(e == hipSuccess && p != nullptr, TLLM_E_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", who, hipGetErrorString(e));
@@ -401,6 +410,11 @@ int noalloc_scratch(const char* who, void** out) {
   return TLLM_OK;
 }
 }  // namespace
+
+extern "C" int tllm_unembedding_argmax_noalloc_init(void) {
+  void* ws = nullptr;
+  return noalloc_scratch("unembedding_argmax_noalloc_init", &ws, nullptr, false);
+}
 
 extern "C" int64_t tllm_unembedding_argmax_noalloc_max_rows(void) { return kNoAllocMaxRows; }
 
@@ -417,7 +431,7 @@ extern "C" int tllm_unembedding_argmax_noalloc_bf16(const void* x, const void* W
   TLLM_REQUIRE(need <= kNoAllocScratchBytes, TLLM_E_SHAPE, "unembedding_argmax_noalloc: %lld bytes of candidates exceed the scratch",
                (long long)need);
   void* ws = nullptr;
-  rc = noalloc_scratch("unembedding_argmax_noalloc", &ws);
+  rc = noalloc_scratch("unembedding_argmax_noalloc", &ws, static_cast<hipStream_t>(stream), true);
   if (rc != TLLM_OK) return rc;
   return unembed_argmax_run("unembedding_argmax_noalloc", x, W, w_scale, ws, need, token_ids, rows, hidden, vocab, stream);
 }

@@ -101,12 +101,17 @@ def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, kee
         r.cos_table = cos.data_ptr()
         r.sin_table = sin.data_ptr()
         r.table_row_stride = cos.stride(0)
+    # The kernels read positions[row] for every row and offset[0] from device memory: these checks are what keeps
+    # those reads in bounds, so they raise (an `assert` disappears under `python -O`).
     if positions is not None:
-        assert positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous()
-        assert positions.numel() == rows, f"positions holds {positions.numel()} entries for {rows} rows"
+        if not (positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous()):
+            raise ValueError("positions must be a contiguous int64 tensor on the GPU")
+        if positions.numel() != rows:
+            raise ValueError(f"positions holds {positions.numel()} entries for {rows} rows")
         r.positions = positions.data_ptr()
     if offset is not None:
-        assert offset.is_cuda and offset.dtype == torch.int64 and offset.numel() == 1
+        if not (offset.is_cuda and offset.dtype == torch.int64 and offset.numel() == 1):
+            raise ValueError("offset must be an int64 tensor of one element on the GPU")
         r.offset = offset.data_ptr()
     r.tokens_per_batch = int(tokens_per_batch)
     r.max_ctx = int(max_ctx)
@@ -606,14 +611,25 @@ def unembedding_decode_argmax_noalloc(hidden: torch.Tensor, weight: torch.Tensor
     """``unembedding_decode_argmax_forward`` for callers that must not allocate: the caller passes ``token_ids``
     (int32 ``[B]``), the candidates go through a device array the library owns, and nothing is taken from the scratch
     pool or from PyTorch's allocator. At most ``tllm_unembedding_argmax_noalloc_max_rows()`` (16) batch rows. Calls on
-    one GPU share that array: do not overlap them on different streams. No counterpart in the reference."""
+    one GPU share that array: do not overlap them on different streams. A caller that captures this call in a graph
+    runs ``unembedding_decode_argmax_noalloc_init()`` on the device first (the library looks the array's address up
+    once per device, which a capturing stream does not allow). No counterpart in the reference."""
     x2, weight, ws, batch, hidden_size, vocab_size = _unembed_prep(hidden, weight, weight_scale)
     _on_gpu(token_ids)
-    assert token_ids.dtype == torch.int32 and token_ids.shape == (batch,) and token_ids.is_contiguous()
+    # the kernel writes token_ids[0 .. batch): checked with exceptions, which `python -O` keeps
+    if token_ids.dtype != torch.int32 or tuple(token_ids.shape) != (batch,) or not token_ids.is_contiguous():
+        raise ValueError(f"token_ids must be a contiguous int32 tensor of shape ({batch},), got {token_ids.dtype} {tuple(token_ids.shape)}")
     rc = lib().tllm_unembedding_argmax_noalloc_bf16(x2.data_ptr(), weight.data_ptr(), ws.data_ptr() if ws is not None else None,
                                                     token_ids.data_ptr(), batch, hidden_size, vocab_size, _stream())
     check(rc, "unembedding_decode_argmax_noalloc")
     return token_ids
+
+
+def unembedding_decode_argmax_noalloc_init(device=None) -> None:
+    """Look up the library-owned candidate array of ``unembedding_decode_argmax_noalloc`` on ``device`` (default: the
+    current one). Call once per device, outside any stream capture, before capturing that op in a graph."""
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        check(lib().tllm_unembedding_argmax_noalloc_init(), "unembedding_decode_argmax_noalloc_init")
 
 
 def unembedding_forward(hidden: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
