@@ -2,58 +2,37 @@
 //
 //   D[T, 5120] = X[T, 2880] . W[5120, 2880]^T      (both operands K-contiguous)
 //
-// Tiling for 256 CUs: a workgroup computes a 128-token x 320-column tile (five whole heads),
-// so T = 2048 is exactly 16 x 16 = 256 tiles -- one per CU, no tail wave (longer inputs take 256-token tiles, see
-// the end of this comment). Eight wavefronts form a 4 x 2 grid (two per SIMD); each owns 32 x 160 of the tile as
-// 1 x 5 v_mfma_f32_32x32x16_bf16 blocks (80 fp32 accumulators per lane) and reads 6 operand
-// fragments from LDS per 5 MFMAs. K is walked in slices of 64 (one 128-byte line per row) through
-// LDS stage rings filled by direct global->LDS loads (global_load_lds_dwordx4: no staging registers,
-// no ds_write): two stages of 16 KB for the tile's activations, three of 40 KB for its weight. Such a load puts
-// the 64 lanes' 16-byte chunks at consecutive LDS addresses, so rows
-// cannot be padded; instead the chunk order inside each row is XOR-swizzled with the row index --
-// applied by choosing which *global* chunk a lane fetches -- and the fragment reads undo it, which
-// keeps the 128-bit fragment reads of 16 consecutive rows conflict-free.
-// With one tile per CU nothing but the kernel's own schedule overlaps anything:
-//   * the one barrier per slice sits before the slice's last k16 step; the stages just finished are handed on
-//     (activations: to the slice after next; weight: to the slice three on), the loads going out one per MFMA behind
-//     that step and the next (never all in a row: a CU's load queue is bounded and a wavefront that overflows it
-//     stalls, MFMAs included);
-//   * the fragment reads of the next k16 step are pinned between the MFMAs of the current one
-//     (sched_group_barrier): hoisted to the top of the iteration, as the compiler does by itself, the
-//     wavefronts read a slice's fragments in one burst with no MFMA running.
-// Where the time goes at T = 2048 (builds with parts of the loop compiled out, two 56 KB stages): the MFMAs,
-// barriers, prologue and epilogue alone take 43 us (30 us of MFMAs at the 1.9 GHz this load clocks at), adding the
-// fragment reads 55 us, the global->LDS loads alone (no MFMA, no fragment read) 56 us, everything 64-66 us. Two things
-// bound it. The feed: what a CU receives is its bytes in flight over the latency of a slice (every slice contains
-// lines nobody in the XCD has touched yet, and a CU returns loads in order, so a slice completes at miss latency,
-// 1.2-2 us); two symmetric stages keep one slice (56 KB) in flight, 46 GB/s per CU. The third weight stage (which
-// fits once the cos/sin table no longer sits next to the stages) keeps two weight slices in flight; a probe of the
-// feed with dummy MFMAs went from 59 to 46 us with it -- the kernel itself only from 64-70 to 63-68.5 us, because
-// behind the feed sits the LDS: 8 wavefronts x 6 fragment reads x 4 steps x 8 clocks + 448 clocks of stage writes per
-// slice are 1984 clocks against 1280 of MFMAs. Measured without gain: the 2 x 2 grid of 64 x 160
-// wavefronts this kernel started with (70 us, 75 us with the three-stage ring: one wavefront per SIMD, nothing to cover
-// a stalled load issue), pairs of 64 x 160 wavefronts taking alternate k16 steps (fewer fragment reads, 68 us), four
-// extra wavefronts that only load (71-75 us), K slices of 32 in a four-stage ring (77 us), a four-deep feed with two
-// more slices in flight into registers and written to LDS by ds_write (70.6 us), an L2 warm-up by a ninth wavefront
-// (its loads sit in the same in-order queue), other spreads of the loads over the steps (+-1 us).
-// From T = 4096 up there are enough tokens for 256 x 320 tiles (BM = 256: eight wavefronts of 64 x 160, 36 % fewer
-// bytes per flop through the L2s): 238 -> 202-205 us at T = 8192. Its 160 accumulators leave room for
-// single-buffered weight fragments only, its stages (2 x 32 KB + 2 x 40 KB) for no third weight stage, and the
-// epilogue runs in two passes of 128 rows. Neither tile has LDS left for the cos/sin table next to the stages: it is
-// built after the K loop inside the idle ring.
+// A workgroup of eight wavefronts computes a tile of 128 tokens x 320 columns (five whole heads), so T = 2048 is
+// exactly 16 x 16 = 256 tiles -- one per CU, no tail wave; from T = 4096 up a tile is 256 tokens x 320 columns (36 %
+// fewer operand bytes per flop through the L2s). Tiles are handed to the XCDs in compact 8 x 4 super-blocks (each XCD
+// has its own L2). K is walked in slices of 64 (one 128-byte line per row) through LDS stage rings filled by direct
+// global->LDS loads (global_load_lds_dwordx4: no staging registers, no ds_write). Such a load puts the 64 lanes'
+// 16-byte chunks at consecutive LDS addresses, so rows cannot be padded; instead the chunk order inside each row is
+// XOR-swizzled with the row index -- applied by choosing which *global* chunk a lane fetches -- and the fragment reads
+// undo it. One hand-spelled s_waitcnt + s_barrier per slice; the loads that refill a freed stage are handed out one
+// behind an MFMA at a time (a CU's load queue is bounded: a wavefront that overflows it stalls, MFMAs included), and
+// the LDS reads of the next step's fragments are pinned between the MFMAs of the current one (sched_group_barrier).
 //
-// The rotary pair (d, d+32) has to sit in one lane. The weights go on the MFMA's M side, so in
-// a 32x32 block a lane owns one token and sixteen output columns (four runs of four); for a
-// whole head the pair is the same register of two neighbouring blocks. 160 columns per
-// wavefront are 2.5 heads; the tile's middle head is therefore split by *dims*: wavefront
-// column 0 takes dims [0,16) u [32,48), column 1 takes [16,32) u [48,64), packed into one
-// "mixed" block whose pair partner is sixteen rows down, i.e. register v + 8 of the same lane.
-// The W rows are permuted accordingly when they are copied into LDS, which costs nothing.
+// The 128-token tile (qkv_prefill_quads_kernel): wavefronts as 2 (tokens) x 4 (columns), 64 x 80 each, on
+// v_mfma_f32_16x16x32_bf16 -- 144 operand rows read from LDS per K step and wavefront, against 192 for a 32 x 160
+// wavefront. Three weight stages (40 KB) + two activation stages (16 KB): two weight slices and one activation slice
+// are in flight while a slice is multiplied. Weight rows sit on the MFMA's M side: a lane owns one token of a
+// 16-token block and four consecutive weight rows of a 16-row block, and the weight rows are dealt to LDS rows so that
+// those four are [lo(p), lo(p+1), hi(p), hi(p+1)] of two adjacent rotation pairs (d, d + 32) -- the rotation never
+// leaves the lane, and every 16-row block is laid out alike, so 80 columns (1.25 heads) need no special case.
+// What the LDS wants from the fragment reads: a 128-bit read is served 16 lanes at a time, lanes 0-7 together with
+// 32-39, 8-15 with 40-47 and so on; see the comment at the fragment addressing.
 //
-// Epilogue: cos/sin of the tile's 128 positions x 32 frequencies are computed once per
-// workgroup from the YaRN parameters into their own LDS region while the first slices are in
-// flight; after the loop every lane adds the bias to its fp32 accumulators, rotates q/k pairs,
-// rounds once to bf16 into an LDS image of the tile, and the image leaves as coalesced 128-bit
+// The 256-token tile (qkv_prefill_kernel256): wavefronts as 4 x 2, 64 x 160 each, on v_mfma_f32_32x32x16_bf16 (160
+// accumulators per lane leave room for single-buffered weight fragments only); two stages of each operand. 160 columns
+// are 2.5 heads: the tile's middle head is split by *dims* between the two wavefront columns (column 0 takes dims
+// [0,16) u [32,48), column 1 [16,32) u [48,64)), packed into one "mixed" 32-row block whose pair partner is sixteen
+// rows down, i.e. register v + 8 of the same lane.
+//
+// Epilogue of both: cos/sin of the tile's positions x 32 frequencies come from the YaRN parameters (in the 128-token
+// tile computed while the first slices are in flight and kept in registers; there is no LDS for the table next to
+// the stages, it is built inside the idle ring after the K loop); every lane adds the bias to its fp32 accumulators,
+// rotates q/k pairs, rounds once to bf16 into an LDS image of the tile, and the image leaves as coalesced 128-bit
 // stores straight into the separate q / k / v outputs (no split / contiguous copies afterwards).
 #include "qkv_common.h"
 
@@ -64,7 +43,6 @@ constexpr int HPT = 5;             // heads per tile
 constexpr int BN = HPT * 64;       // 320 columns per tile
 constexpr int BK = 64;             // K slice: one 128-byte line per row
 constexpr int XS = 2;              // LDS stages of the activations
-constexpr int KS = BK / 16;        // k16 MFMA steps per slice
 constexpr int CHUNKS = BK / 8;     // 16-byte chunks per LDS row
 constexpr int LROW = BK * 2;       // LDS row, bytes (unpadded: rows are swizzled instead)
 constexpr int RPB = 1024 / LROW;   // rows per 1 KiB block (one load instruction)
@@ -75,414 +53,53 @@ constexpr int w_stages(int bm) { return bm == 128 ? 3 : 2; }
 constexpr int ring_bytes(int bm) { return w_stages(bm) * W_STAGE + XS * x_stage(bm); }
 constexpr int OROW = BN + 4;       // epilogue staging row, elements (648 B: an odd number of 8-byte units)
 constexpr int CSROW = 34;                  // float2 per row of the cos/sin table: 32 frequencies + padding, so that
-                                           // lanes reading the same frequency of 32 different rows spread over the banks
+                                           // lanes reading the same frequency of different rows spread over the banks
 constexpr int EROWS = 128;                 // rows the epilogue finishes per pass (one pass for a 128-token tile, two for 256)
 constexpr int CS_BYTES = EROWS * CSROW * 8;   // cos/sin of (row, frequency) as float2
 constexpr int IMG_BYTES = (EROWS * OROW * 2 + 1023) / 1024 * 1024;   // bf16 image of a pass's rows
 constexpr int BIAS_BYTES = BN * 4;         // the tile's bias as fp32, head-local column order
-// The stages leave no room for the cos/sin table: it is built inside the idle stage ring after the K loop -- by a
-// 128-token tile from values computed while the first slices were in flight and kept in registers, by a 256-token tile
-// (no registers to spare) per pass from the rows' positions parked in LDS.
+// Behind the ring: the bias, and (256-token tile) the rows' positions.
 constexpr int prefill_smem(int bm) { return ring_bytes(bm) + BIAS_BYTES + bm * 8; }
 static_assert(IMG_BYTES + CS_BYTES <= ring_bytes(128) && IMG_BYTES + CS_BYTES <= ring_bytes(256), "the epilogue reuses the stage ring");
 static_assert(prefill_smem(128) <= 160 * 1024 && prefill_smem(256) <= 160 * 1024, "LDS per workgroup");
-static_assert(KS % 2 == 0 && W_STAGE % 8192 == 0 && x_stage(128) % 8192 == 0 && CHUNKS == 8 && XS == 2,
-              "the schedule and the swizzle below are written for BK = 64");
+static_assert(W_STAGE % 8192 == 0 && x_stage(128) % 8192 == 0 && CHUNKS == 8 && XS == 2, "the schedules and the swizzle below are written for BK = 64");
 }  // namespace
 
-// Chunk swizzle of LDS row r: the 16-byte chunk c of the row is stored at chunk position c ^ swz(r).
-// Chosen so that the 16 consecutive rows one fragment read touches land in 16 different bank groups.
+// Chunk swizzle of LDS row r: the 16-byte chunk c of the row is stored at chunk position c ^ swz(r). Eight consecutive
+// rows of one chunk land on the eight chunk positions, and rows r, r + 8 on positions that differ in bit 0.
 __device__ __forceinline__ int swz(int r) { return (r ^ (r >> 3)) & 7; }
 
-// LDS row i of the W tile -> (head within tile, dim within head); see the header comment.
-__device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
-  const int w = i >= 160 ? 1 : 0;
-  const int j = i - 160 * w;
-  if (j < 128) {
-    *head_local = 3 * w + (j >> 6);
-    *dim = j & 63;
+// Tile of a workgroup, XCD-aware: consecutive block ids go to different XCDs (8 of them, each with its own L2), so
+// every XCD gets a compact super-block of `swizzle` x (32 / swizzle) tiles (token tiles x column tiles).
+__device__ __forceinline__ void prefill_tile_of_block(int b, int tiles_m, int tiles_n, int swizzle, int* tile_m, int* tile_n) {
+  if (swizzle) {
+    const int per = (tiles_m * tiles_n) >> 3;
+    const int id = (b & 7) * per + (b >> 3);
+    const int sb = id >> 5, in = id & 31;
+    const int sm = swizzle, sn = 32 / swizzle;
+    const int sbm = tiles_m / sm;
+    *tile_m = (sb % sbm) * sm + (in % sm);
+    *tile_n = (sb / sbm) * sn + (in / sm);
   } else {
-    const int jj = j - 128;
-    *head_local = 2;
-    *dim = (jj < 16) ? (16 * w + jj) : (32 + 16 * w + (jj - 16));
+    *tile_m = b % tiles_m;
+    *tile_n = b / tiles_m;
   }
 }
 
-// WROWS wavefront rows x 2 wavefront columns: 4 x 2 (two wavefronts per SIMD, 32 x 160 each) is what is launched;
-// 2 x 2 (one per SIMD, 64 x 160 each) compiles from the same source.
-// BM: tokens per tile. 128 makes T = 2048 one tile per CU; 256 (from T = 4096 up) reads each weight slice for twice
-// the tokens: 36 % fewer bytes per flop through the L2s, which is what bounds the 128-token tile.
-template <int BM, int WROWS>
-__global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
-  constexpr int WS = w_stages(BM);          // weight stages
-  constexpr int XSTAGE = x_stage(BM);
-  constexpr int NW = WROWS * 2;             // wavefronts
-  constexpr int NT = NW * 64;               // threads
-  constexpr int MB = BM / (32 * WROWS);     // 32-token blocks per wavefront
-  constexpr int LPX = XSTAGE / 1024 / NW;   // load instructions (1 KiB blocks) per wavefront per slice: activations ...
-  constexpr int LPWW = W_STAGE / 1024 / NW; // ... weight
-  constexpr int LPW = LPX + LPWW;           // ... together
-  constexpr int NMF = MB * 5;               // MFMAs per k16 step
-  constexpr int NRD = MB + 5;               // fragment reads per k16 step
-  constexpr int NL_LAST = LPW < NMF ? LPW : NMF;   // loads handed out behind a slice's last step ...
-  constexpr int NL_FIRST = LPW - NL_LAST;          // ... and behind the next slice's first step
-  static_assert(NL_FIRST <= NMF, "a slice's loads fit behind two k16 steps");
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar: which operand a load belongs to is then a scalar choice
-  const int wm = wave >> 1, wn = wave & 1;
-  const int l32 = lane & 31, lh = lane >> 5;
-
-  // ---- tile assignment: XCD-aware. Consecutive block ids go to different XCDs (8 of them, each
-  // with its own L2), so give every XCD a compact 8 x 4 super-block of tiles to maximise L2 reuse.
-  int tile_m, tile_n;
-  {
-    const int b = blockIdx.x;
-    if (swizzle) {
-      // `swizzle` = token tiles per super-block (SM); a super-block is SM x (32 / SM) tiles
-      const int per = (tiles_m * tiles_n) >> 3;
-      const int id = (b & 7) * per + (b >> 3);
-      const int sb = id >> 5, in = id & 31;
-      const int sm = swizzle, sn = 32 / swizzle;
-      const int sbm = tiles_m / sm;
-      tile_m = (sb % sbm) * sm + (in % sm);
-      tile_n = (sb / sbm) * sn + (in / sm);
-    } else {
-      tile_m = b % tiles_m;
-      tile_n = b / tiles_m;
-    }
-  }
-  const int64_t row0 = static_cast<int64_t>(tile_m) * BM;
-  const int head0 = tile_n * HPT;
-  const int total_heads = a.n_q_heads + 2 * a.n_kv_heads;
-  const int kvec = a.hidden >> 3;
-  const int n_iter = a.hidden / BK;
-
-  // ---- loader setup. A slice's activations (BM rows) and weight (320 rows) land in separate stage rings; within its
-  // operand, load instruction j of wavefront w fills 1 KiB block w * n + j (RPB rows of LROW bytes); lane L lands at
-  // row RPB * blk + L / CHUNKS, chunk position L % CHUNKS, so it fetches global chunk (L % CHUNKS) ^ swz(row).
-  // A wavefront's loads of a period are numbered activations first (j < LPX), then weight.
-  // The tiles that share an XCD's L2 walk K in lockstep and four or eight of them want the same lines;
-  // each starts its round of blocks at a different one so that at any moment they pull on different
-  // rows (different L2 channels) instead of queueing on the same line.
-  const int rotx = (blockIdx.x >> 3) % LPX, rotw = (blockIdx.x >> 3) % LPWW;
-  // A load's source is a scalar base (the tile's first activation row, or the weight) plus a 32-bit byte offset per
-  // lane: half the registers of a pointer per load, and the loads can use the scalar-base addressing form.
-  const unsigned char* const x_base = reinterpret_cast<const unsigned char*>(a.x) + row0 * a.hidden * 2;
-  const unsigned char* const w_base = reinterpret_cast<const unsigned char*>(a.W);
-  unsigned char* const wring = smem;                         // WS stages of W_STAGE bytes
-  unsigned char* const xring = smem + WS * W_STAGE;          // XS stages of XSTAGE bytes
-  unsigned soff[LPW];
-  int blk_off[LPW];                                          // LDS byte offset of load j's block inside its operand's stage
-#pragma unroll
-  for (int j = 0; j < LPW; ++j) {
-    if (j < LPX) {
-      const int bj = wave * LPX + (j + rotx) % LPX;
-      blk_off[j] = bj * 1024;
-      const int r = bj * RPB + lane / CHUNKS;                // activation row of the tile
-      const int c = (lane % CHUNKS) ^ swz(r);
-      int64_t lr = r;
-      if (row0 + lr >= a.rows) lr = a.rows - 1 - row0;       // clamp: valid memory, result rows are never stored
-      soff[j] = static_cast<unsigned>((lr * kvec + c) * 16);
-    } else {
-      const int bj = wave * LPWW + (j - LPX + rotw) % LPWW;
-      blk_off[j] = bj * 1024;
-      const int r = bj * RPB + lane / CHUNKS;                // weight row of the tile (LDS order)
-      const int c = (lane % CHUNKS) ^ swz(r);
-      int hl, dim;
-      w_tile_row(r, &hl, &dim);
-      int h = head0 + hl;
-      if (h >= total_heads) h = total_heads - 1;             // clamp for a ragged last tile
-      soff[j] = static_cast<unsigned>(((static_cast<int64_t>(h) * 64 + dim) * kvec + c) * 16);
-    }
-  }
-
-  f32x16 acc[MB][5];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < 5; ++nb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
-
-  // fragment addressing: byte offset of (row, chunk c) inside a stage is row*LROW + ((c ^ swz(row)) << 4)
-  const int fa_row = 32 * MB * wm + l32, fb_row = 160 * wn + l32;   // rows inside the activation / the weight stage
-  // The k16 step kk wants chunks 2 kk + lh of the row; with the row's swizzle that is position (2 kk + lh) ^ swz(row),
-  // and because a row starts on a 128-byte boundary the step enters as an XOR of bits 5-6 of the byte offset: one
-  // register per 32-row block instead of one per block and step.
-  int fa_o[MB], fb_o[5];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) fa_o[mb] = (fa_row + 32 * mb) * LROW + ((lh ^ swz(fa_row + 32 * mb)) << 4);
-#pragma unroll
-  for (int nb = 0; nb < 5; ++nb) fb_o[nb] = (fb_row + 32 * nb) * LROW + ((lh ^ swz(fb_row + 32 * nb)) << 4);
-  auto load_frags = [&](const unsigned char* stx, const unsigned char* stw, int kk, bf16x8 (&fa)[MB], bf16x8 (&fb)[5]) {
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) fa[mb] = *reinterpret_cast<const bf16x8*>(stx + (fa_o[mb] ^ (kk << 5)));
-#pragma unroll
-    for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(stw + (fb_o[nb] ^ (kk << 5)));
-  };
-  // Period `per` = the loads that go out when slice `per` has been consumed: the activations of slice per + 2 into the
-  // activation stage that slice just vacated, the weight of slice per + WS into the weight stage it vacated.
-  auto issue_load = [&](int per, int j) {                // one load instruction of period `per`
-    const bool is_x = j < LPX;                            // known at compile time wherever j is
-    const int sl = per + (is_x ? XS : WS);
-    const int slc = sl < n_iter ? sl : n_iter - 1;        // look-ahead past the end re-reads the last slice (never used)
-    unsigned char* dst = is_x ? xring + (sl % XS) * XSTAGE : wring + (sl % WS) * W_STAGE;
-    // Spelled out rather than through __builtin_amdgcn_global_load_lds: this is the scalar-base form (64-bit base in
-    // SGPRs, 32-bit lane offset, LDS block address in M0), where the builtin builds a 64-bit address per lane; 14 / 13
-    // fewer registers in the two tile heights and 2-3 % faster. The lanes' 16 bytes land at M0 + 16 * lane.
-    const unsigned lds_off = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst + blk_off[j]));
-    const unsigned char* sb = (is_x ? x_base : w_base) + static_cast<int64_t>(slc) * (BK * 2);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
-  };
-  auto issue_period = [&](int per) {
-#pragma unroll
-    for (int j = 0; j < LPW; ++j) issue_load(per, j);
-  };
-  // One k16 step: NMF MFMAs on the fragments in buffer `cur`. Behind the MFMAs go the LDS reads of the next step's
-  // fragments (into buffer cur ^ 1) and, for m < n, one global->LDS load instruction (j0 + m) of slice `lit`.
-  // The interleaving is pinned with sched_group_barrier, for two reasons:
-  //   * left alone, the compiler hoists all fragment reads of a slice to the top of the iteration; the wavefronts
-  //     then read them from LDS in one burst with no MFMA running and do their MFMAs afterwards -- the two costs
-  //     add up instead of overlapping;
-  //   * a CU takes only so many loads into its queue and a wavefront that issues one more stalls, MFMAs
-  //     included, until the queue has drained that far; a slice's loads in a row do exactly that. Handed out one
-  //     per MFMA (32 cycles) they never find the queue full.
-  bf16x8 fa[2][MB], fb[2][5];
-  auto read_frag = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int i) {   // fragment i of the next step: activations first
-    if (i < MB) fa[cur ^ 1][i < MB ? i : 0] = *reinterpret_cast<const bf16x8*>(nstx + (fa_o[i < MB ? i : 0] ^ (nkk << 5)));
-    else fb[cur ^ 1][i - MB] = *reinterpret_cast<const bf16x8*>(nstw + (fb_o[i - MB] ^ (nkk << 5)));
-  };
-  auto step = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int lit, int j0, int n) {
-    if constexpr (MB == 2) {
-      // 64 x 160 per wavefront: the two MFMAs that share a weight fragment are issued back to back and the fragment is
-      // reloaded for the next step right behind them (weight fragments single-buffered: 20 registers instead of 40, which
-      // is what keeps this variant's 160 accumulators + fragments inside 256 registers); the activation fragments of the
-      // next step go into their second buffer behind the first two pairs.
-#pragma unroll
-      for (int nb = 0; nb < 5; ++nb) {
-        acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][nb], fa[cur][0], acc[0][nb], 0, 0, 0);
-        acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][nb], fa[cur][1], acc[1][nb], 0, 0, 0);
-        fb[0][nb] = *reinterpret_cast<const bf16x8*>(nstw + (fb_o[nb] ^ (nkk << 5)));
-        if (nb < 2) fa[cur ^ 1][nb] = *reinterpret_cast<const bf16x8*>(nstx + (fa_o[nb] ^ (nkk << 5)));
-        if (2 * nb < n) issue_load(lit, j0 + 2 * nb);
-        if (2 * nb + 1 < n) issue_load(lit, j0 + 2 * nb + 1);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        if (nb < 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (2 * nb + 1 < n) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-        else if (2 * nb < n) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      }
-      return;
-    }
-#pragma unroll
-    for (int m = 0; m < NMF; ++m) {
-      const int mb = m / 5, nb = m % 5;
-      acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][nb], fa[cur][mb], acc[mb][nb], 0, 0, 0);   // weights on M, tokens on N
-      // NRD reads over NMF MFMAs: one each (7 over 10), or two behind the first when there are more reads than MFMAs (6 over 5)
-      constexpr int EXTRA = NRD > NMF ? NRD - NMF : 0;
-      const int r0 = m == 0 ? 0 : m + EXTRA, nr = m == 0 ? 1 + EXTRA : (m + EXTRA < NRD ? 1 : 0);
-#pragma unroll
-      for (int i = 0; i < nr; ++i) read_frag(cur, nstx, nstw, nkk, r0 + i);
-      if (m < n) issue_load(lit, j0 + m);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // one MFMA
-      if (nr == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // its LDS reads
-      if (nr == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      if (m < n) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // one VMEM read
-    }
-  };
-
-  // prologue: slice 0 requested first (period -XS asks for activations 0, period -WS for weight 0)
-#pragma unroll
-  for (int j = 0; j < LPW; ++j) issue_load(j < LPX ? -XS : -WS, j);
-  // cos/sin of (row, frequency) for the epilogue, computed from the YaRN parameters. There is no LDS for the table
-  // next to the stages; it is built inside the idle stage ring after the K loop. A 128-token tile computes the values
-  // here, while the first slices are in flight (the positions are global loads: all of them are issued before any is
-  // used), and keeps them in registers until then; a 256-token tile (no registers to spare) only parks the rows'
-  // positions in LDS now and computes the table after the loop, 128 rows at a time.
-  constexpr bool CS_REGS = BM == EROWS;
-  constexpr int CS_OFF = IMG_BYTES;
-  constexpr int BIAS_OFF = ring_bytes(BM);
-  float2* cs_tab = reinterpret_cast<float2*>(smem + CS_OFF);
-  // the tile's 320 bias values, widened once (fetched per group inside the epilogue they were twenty dependent
-  // global loads per lane, each waited for)
-  float* bias_s = reinterpret_cast<float*>(smem + BIAS_OFF);
-  int64_t* pos_s = reinterpret_cast<int64_t*>(smem + BIAS_OFF + BIAS_BYTES);   // 256-token tile only
-  if (tid < BN) {
-    int h = head0 + (tid >> 6);
-    if (h >= total_heads) h = total_heads - 1;
-    bias_s[tid] = a.bias ? static_cast<float>(a.bias[h * 64 + (tid & 63)]) : 0.f;
-  }
-  constexpr int RPP = NT / 32;                         // table rows per round of the whole workgroup
-  constexpr int CSN = EROWS / RPP;                     // table entries per thread: rows tid / 32 + RPP * j, frequency tid % 32
-  float2 csr[CS_REGS ? CSN : 1];
-  auto compute_cs = [&](auto&& pos_of, auto&& sink) {  // pos_of(row) -> raw position; sink(j, cos, sin)
-    const int f = tid & 31;
-    int64_t pos[CSN];
-#pragma unroll
-    for (int j = 0; j < CSN; ++j) pos[j] = pos_of((tid >> 5) + RPP * j);
-#pragma unroll
-    for (int j = 0; j < CSN; ++j) {
-      float c, sn;
-      rope_cos_sin(ra, fr, rope_wrap(pos[j], ra.max_ctx), f, &c, &sn);
-      sink(j, c, sn);
-    }
-  };
-  auto store_cs = [&](int j, float c, float sn) { cs_tab[((tid >> 5) + RPP * j) * CSROW + (tid & 31)] = make_float2(c, sn); };
-  if (a.has_rope) {
-    if constexpr (CS_REGS) {
-      compute_cs(
-          [&](int r) {
-            int64_t grow = row0 + r;
-            if (grow >= a.rows) grow = a.rows - 1;
-            return rope_position_raw(ra, grow);
-          },
-          [&](int j, float c, float sn) { csr[j] = make_float2(c, sn); });
-    } else {
-      for (int r = tid; r < BM; r += NT) {
-        int64_t grow = row0 + r;
-        if (grow >= a.rows) grow = a.rows - 1;
-        pos_s[r] = rope_position_raw(ra, grow);
-      }
-    }
-  }
-  // The rest of the look-ahead, oldest first: (three weight stages: weight 1,) then period -1 = activations 1 and the
-  // weight of slice WS - 1. Requested only now: the compiler waits for its own loads above (positions, bias) by
-  // count, which would have made it wait for these as well.
-  if constexpr (WS == 3) {
-#pragma unroll
-    for (int j = LPX; j < LPW; ++j) issue_load(-2, j);
-  }
-  issue_period(-1);
-  // slice 0 has landed when only those are outstanding
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");
-  __syncthreads();
-  load_frags(xring, wring, 0, fa[0], fb[0]);
-
-  // Steady state. While slice `it` is multiplied, outstanding or landed, oldest first: (three weight stages: the
-  // weight of slice it + 1,) the activations of slice it + 1, the weight of slice it + WS - 1. The one barrier per
-  // slice sits before the slice's last k16 step; from there on the stages of slice `it` are free (all reads of them
-  // have been issued) and period `it` goes out behind the MFMAs of this last step and, what does not fit there, of the
-  // next slice's first step: the activations of slice it + 2 -- a whole slice of MFMAs before they are needed -- and
-  // the weight of slice it + WS -- with the third stage, two slices.
-  for (int it = 0; it < n_iter; ++it) {
-    const unsigned char* stx = xring + (it % XS) * XSTAGE;
-    const unsigned char* stw = wring + (it % WS) * W_STAGE;
-    const unsigned char* nxx = xring + ((it + 1) % XS) * XSTAGE;
-    const unsigned char* nxw = wring + ((it + 1) % WS) * W_STAGE;
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-      if (kk + 1 < KS) {
-        if (kk == 0 && it > 0) {
-          step(kk & 1, stx, stw, kk + 1, it - 1, NL_LAST, NL_FIRST);
-        } else {
-          step(kk & 1, stx, stw, kk + 1, 0, 0, 0);
-        }
-      } else {
-        // Slice it + 1 has landed (this wavefront's share: everything but the newest weight slice of a three-stage
-        // ring), then the barrier: everyone's share has, and everyone has issued its last reads of slice it.
-        // Spelled out, because __syncthreads() carries a fence that drains every load in flight, the look-ahead ones
-        // included.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((WS - 2) * LPWW) : "memory");
-        step(kk & 1, nxx, nxw, 0, it, 0, NL_LAST);
-      }
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // drain the look-ahead loads before LDS is reused
-  __syncthreads();
-
-  // ---- epilogue -------------------------------------------------------------------------------
-  // The stage ring is idle now and becomes a bf16 image of the output tile (rows padded to 656 B so the
-  // two half-wavefronts of a store hit different banks). Every lane finishes its accumulators (bias,
-  // rotation with the cos/sin table, one RNE) into the image; then the tile leaves as coalesced
-  // 128-bit stores, eight columns of one head per lane.
-  bf16* img = reinterpret_cast<bf16*>(smem);
-  const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
+// The epilogue's last phase, shared by both tile heights: rows [pass_row0, pass_row0 + EROWS) of the tile sit in LDS as
+// a bf16 image (OROW elements per row); a chunk = 8 consecutive dims of one head of one row goes out as one 128-bit store.
+template <int NT>
+__device__ __forceinline__ void prefill_copy_out(const QkvArgs& a, const bf16* img, int tid, int head0, int total_heads, int64_t pass_row0,
+                                                 int64_t slot_off) {
   const bool vec_ok = (reinterpret_cast<uintptr_t>(a.q) % 16 == 0) && (reinterpret_cast<uintptr_t>(a.k) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(a.v) % 16 == 0) && a.q_rs % 8 == 0 && a.k_rs % 8 == 0 && a.v_rs % 8 == 0 &&
                       a.kv_slot_stride % 8 == 0;
-
-  // Accumulator layout (weights on the MFMA's M side): the lane owns token l32 of each 32-token block and,
-  // in each 32-column block, columns 8*(v>>2) + 4*lh + (v&3) -- runs of four consecutive columns, so
-  // bias, cos/sin and the image stores all move in 4-element vectors. A whole head is two blocks (low
-  // dims, their partners: same register index); the mixed block holds the wavefront's 16 low dims of
-  // the middle head in rows 0-15 and their partners in rows 16-31 (register v and v + 8).
-  // A pass finishes EROWS rows: the wavefronts that hold them write the image, then everyone copies it out.
-  if constexpr (CS_REGS) {
-    if (a.has_rope) {
-#pragma unroll
-      for (int j = 0; j < CSN; ++j) store_cs(j, csr[j].x, csr[j].y);
-    }
-    __syncthreads();
-  }
-#pragma unroll
-  for (int pass = 0; pass < BM / EROWS; ++pass) {
-  if constexpr (!CS_REGS) {
-    if (pass > 0) __syncthreads();                        // the previous pass's image and table have been read
-    if (a.has_rope) compute_cs([&](int r) { return pos_s[EROWS * pass + r]; }, store_cs);
-    __syncthreads();
-  }
-  const bool my_pass = (32 * MB * wm) / EROWS == pass;     // uniform per wavefront
-#pragma unroll
-  for (int hp = 0; hp < 3; ++hp) {
-    if (!my_pass) break;
-    const int hl = (hp < 2) ? (3 * wn + hp) : 2;
-    int head = head0 + hl;
-    if (head >= total_heads) head = total_heads - 1;        // ragged last tile: computed, never copied out
-    const bool rotate = a.has_rope && head < a.n_q_heads + a.n_kv_heads;
-    const int ngrp = hp < 2 ? 4 : 2;                         // groups of four (lo, hi) pairs per lane
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      if (g >= ngrp) continue;
-      // first of the four consecutive low dims of this group, and where its partner lives
-      const int d0 = hp < 2 ? (8 * g + 4 * lh) : (16 * wn + 8 * g + 4 * lh);
-      const f32x4 b_lo = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + d0);
-      const f32x4 b_hi = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + 32 + d0);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const int r = 32 * MB * wm + 32 * mb + l32 - EROWS * pass;   // row inside the pass
-        float lo[4], hi[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (hp < 2) {
-            lo[j] = acc[mb][2 * hp][4 * g + j] + b_lo[j];
-            hi[j] = acc[mb][2 * hp + 1][4 * g + j] + b_hi[j];
-          } else {
-            lo[j] = acc[mb][4][4 * g + j] + b_lo[j];
-            hi[j] = acc[mb][4][8 + 4 * g + j] + b_hi[j];
-          }
-        }
-        bf16x4 olo, ohi;
-        if (rotate) {                                      // uniform per wavefront and head
-          const f32x4 c01 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0);       // (cos, sin) of dims d0, d0 + 1
-          const f32x4 c23 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0 + 2);   // ... d0 + 2, d0 + 3
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float c = j < 2 ? c01[2 * j] : c23[2 * j - 4], sn = j < 2 ? c01[2 * j + 1] : c23[2 * j - 3];
-            olo[j] = static_cast<bf16>(lo[j] * c - hi[j] * sn);
-            ohi[j] = static_cast<bf16>(hi[j] * c + lo[j] * sn);
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            olo[j] = static_cast<bf16>(lo[j]);
-            ohi[j] = static_cast<bf16>(hi[j]);
-          }
-        }
-        *reinterpret_cast<bf16x4*>(img + r * OROW + hl * 64 + d0) = olo;
-        *reinterpret_cast<bf16x4*>(img + r * OROW + hl * 64 + 32 + d0) = ohi;
-      }
-    }
-  }
-  __syncthreads();
-
-  // copy-out: chunk = 8 consecutive dims of one head of one row
 #pragma unroll 4
   for (int ch = tid; ch < EROWS * (BN / 8); ch += NT) {
     const int r = ch / (BN / 8), cc = ch - r * (BN / 8);
     const int hl = cc >> 3, d8 = (cc & 7) * 8;
     const int head = head0 + hl;
-    const int64_t grow = row0 + EROWS * pass + r;
+    const int64_t grow = pass_row0 + r;
     if (head >= total_heads || grow >= a.rows) continue;
     bf16* dst;
     if (head < a.n_q_heads)
@@ -507,7 +124,542 @@ __global__ __launch_bounds__(WROWS * 128) void qkv_prefill_kernel(QkvArgs a, Rop
       for (int e = 0; e < 8; ++e) dst[e] = val[e];
     }
   }
-  }   // pass
+}
+
+// ===================================================================================== the 128-token tile
+// LDS row i of the W tile -> (head within tile, dim within head): block b = i / 16 (0..19) holds pairs 8 (b % 4) .. + 8
+// of head b / 4; row i % 16 of the block is pair 8 (b % 4) + 2 (i16 / 4) + (i16 & 1), half (i16 >> 1) & 1.
+__device__ __forceinline__ void w_tile_row_quads(int i, int* head_local, int* dim) {
+  const int b = i >> 4, i16 = i & 15;
+  *head_local = b >> 2;
+  *dim = 8 * (b & 3) + 2 * (i16 >> 2) + (i16 & 1) + 32 * ((i16 >> 1) & 1);
+}
+
+// Unwrapped rotary positions of 16 consecutive rows starting at row g0 (the same in every lane; rows past the last one
+// repeat it), read through the scalar cache: positions and offset were written before this kernel started and nothing
+// writes them while it runs, and a scalar load does not involve the vector-memory counter the look-ahead loads are
+// waited for with. Without a positions tensor the result is offset[0] alone and the caller adds row % tokens_per_batch.
+__device__ __forceinline__ void rope_positions_16_uniform(const RopeArgs& r, const void* any_valid, int64_t g0, int64_t rows, int64_t (&pos_even)[8],
+                                                          int64_t (&pos_odd)[8]) {
+  typedef const int64_t __attribute__((address_space(4))) * const_i64_ptr;
+  // branch-free (an absent tensor reads a valid dummy address), so that the sixteen values stay in scalar registers
+  const_i64_ptr pp = reinterpret_cast<const_i64_ptr>(reinterpret_cast<uintptr_t>(r.positions ? static_cast<const void*>(r.positions) : any_valid));
+  const_i64_ptr po = reinterpret_cast<const_i64_ptr>(reinterpret_cast<uintptr_t>(r.offset ? static_cast<const void*>(r.offset) : any_valid));
+  const int64_t off_ld = po[0];
+  const int64_t off = r.offset ? off_ld : 0;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int64_t gi = g0 + j < rows ? g0 + j : rows - 1;
+    const int64_t ld = pp[r.positions ? gi : 0];
+    // two arrays: a lane picks row 2 i or 2 i + 1 by a select between them (of one array the compiler makes an
+    // indexed access, and the array then lives in scratch memory)
+    if (j & 1) pos_odd[j >> 1] = r.positions ? ld : off;
+    else pos_even[j >> 1] = r.positions ? ld : off;
+  }
+}
+
+__global__ __launch_bounds__(512) void qkv_prefill_quads_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
+  constexpr int BM = 128;
+  constexpr int WS = w_stages(BM);          // weight stages (3)
+  constexpr int XSTAGE = x_stage(BM);
+  constexpr int NW = 8, NT = 512;
+  constexpr int TB = BM / 2 / 16;           // 16-token blocks per wavefront (4)
+  constexpr int RB = 5;                     // 16-row weight blocks per wavefront
+  constexpr int KSTEPS = BK / 32;           // k32 MFMA steps per slice (2)
+  constexpr int LPX = XSTAGE / 1024 / NW;   // load instructions (1 KiB blocks) per wavefront per slice: activations (2) ...
+  constexpr int LPWW = W_STAGE / 1024 / NW; // ... weight (5)
+  constexpr int LPW = LPX + LPWW;
+  constexpr int NMF = TB * RB;              // MFMAs per k32 step (20)
+  constexpr int NRD = TB + RB;              // fragment reads per k32 step (9)
+  static_assert(WS == 3 && KSTEPS == 2 && 2 * LPW <= NMF && 2 * NRD <= NMF, "the schedule below: two steps per slice, reads and loads behind alternate MFMAs");
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar: which operand a load belongs to is then a scalar choice
+  const int wm = wave >> 2, wn = wave & 3;
+  const int m16 = lane & 15, g = lane >> 4;
+
+  int tile_m, tile_n;
+  prefill_tile_of_block(blockIdx.x, tiles_m, tiles_n, swizzle, &tile_m, &tile_n);
+  const int64_t row0 = static_cast<int64_t>(tile_m) * BM;
+  const int head0 = tile_n * HPT;
+  const int total_heads = a.n_q_heads + 2 * a.n_kv_heads;
+  const int kvec = a.hidden >> 3;
+  const int n_iter = a.hidden / BK;
+
+  // ---- loader setup. A slice's activations (128 rows) and weight (320 rows) land in separate stage rings; within its
+  // operand, load instruction j of wavefront w fills 1 KiB block w * n + j (RPB rows of LROW bytes); lane L lands at
+  // row RPB * blk + L / CHUNKS, chunk position L % CHUNKS, so it fetches global chunk (L % CHUNKS) ^ swz(row).
+  // A wavefront's loads of a period are numbered activations first (j < LPX), then weight.
+  // The tiles that share an XCD's L2 walk K in lockstep and four or eight of them want the same lines; each starts
+  // its round of blocks at a different one so that at any moment they pull on different rows (different L2 channels).
+  const int rotx = (blockIdx.x >> 3) % LPX, rotw = (blockIdx.x >> 3) % LPWW;
+  // A load's source is a scalar base (the tile's first activation row, or the weight) plus a 32-bit byte offset per lane.
+  const unsigned char* const x_base = reinterpret_cast<const unsigned char*>(a.x) + row0 * a.hidden * 2;
+  const unsigned char* const w_base = reinterpret_cast<const unsigned char*>(a.W);
+  unsigned char* const wring = smem;                         // WS stages of W_STAGE bytes
+  unsigned char* const xring = smem + WS * W_STAGE;          // XS stages of XSTAGE bytes
+  unsigned soff[LPW];
+  int blk_off[LPW];                                          // LDS byte offset of load j's block inside its operand's stage
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) {
+    if (j < LPX) {
+      const int bj = wave * LPX + (j + rotx) % LPX;
+      blk_off[j] = bj * 1024;
+      const int r = bj * RPB + lane / CHUNKS;                // activation row of the tile
+      const int c = (lane % CHUNKS) ^ swz(r);
+      int64_t lr = r;
+      if (row0 + lr >= a.rows) lr = a.rows - 1 - row0;       // clamp: valid memory, result rows are never stored
+      soff[j] = static_cast<unsigned>((lr * kvec + c) * 16);
+    } else {
+      const int bj = wave * LPWW + (j - LPX + rotw) % LPWW;
+      blk_off[j] = bj * 1024;
+      const int r = bj * RPB + lane / CHUNKS;                // weight row of the tile (LDS order)
+      const int c = (lane % CHUNKS) ^ swz(r);
+      int hl, dim;
+      w_tile_row_quads(r, &hl, &dim);
+      int h = head0 + hl;
+      if (h >= total_heads) h = total_heads - 1;             // clamp for a ragged last tile
+      soff[j] = static_cast<unsigned>(((static_cast<int64_t>(h) * 64 + dim) * kvec + c) * 16);
+    }
+  }
+  // Period `per` = the loads that go out when slice `per` has been consumed: the activations of slice per + 2 into the
+  // activation stage that slice just vacated, the weight of slice per + 3 into the weight stage it vacated.
+  auto issue_load = [&](int per, int j) {
+    const bool is_x = j < LPX;                            // known at compile time wherever j is
+    const int sl = per + (is_x ? XS : WS);
+    const int slc = sl < n_iter ? sl : n_iter - 1;        // look-ahead past the end re-reads the last slice (never used)
+    unsigned char* dst = is_x ? xring + (sl % XS) * XSTAGE : wring + (sl % WS) * W_STAGE;
+    // Spelled out rather than through __builtin_amdgcn_global_load_lds: this is the scalar-base form (64-bit base in
+    // SGPRs, 32-bit lane offset, LDS block address in M0), where the builtin builds a 64-bit address per lane. The
+    // lanes' 16 bytes land at M0 + 16 * lane; the s_nop is the wait state an M0 write needs before an LDS-DMA load reads it.
+    const unsigned lds_off = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst + blk_off[j]));
+    const unsigned char* sb = (is_x ? x_base : w_base) + static_cast<int64_t>(slc) * (BK * 2);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
+  };
+
+  f32x4 acc[RB][TB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) acc[rb][tb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // Fragment addressing. Lane group g = lane / 16 supplies k = 8 g .. 8 g + 7 of a k32 step; which 16-byte chunk of
+  // the step's 64 bytes that is does not matter as long as both operands agree (a dot product does not care about the
+  // order of its terms), and it is chosen for the LDS banks: a 128-bit read is served 16 lanes at a time, lanes
+  // 0-7 together with 32-39, 8-15 with 40-47 and so on, i.e. groups g and g + 2 of eight consecutive rows. Under the
+  // row swizzle those two must read chunks that differ in bit 0: group g reads chunk 4 kk + (g >> 1 | (g & 1) << 1)
+  // (with chunk 4 kk + g half of all LDS cycles of this kernel were bank conflicts). With the row's swizzle that is
+  // position chunk ^ swz(row), and the step enters as an XOR of bit 6 of the byte offset.
+  const int gc = (g >> 1) | ((g & 1) << 1);
+  int fx_o[TB], fw_o[RB];
+#pragma unroll
+  for (int tb = 0; tb < TB; ++tb) {
+    const int r = 64 * wm + 16 * tb + m16;
+    fx_o[tb] = r * LROW + ((gc ^ swz(r)) << 4);
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int r = 80 * wn + 16 * rb + m16;
+    fw_o[rb] = r * LROW + ((gc ^ swz(r)) << 4);
+  }
+  bf16x8 fx[2][TB], fw[2][RB];
+  auto read_frag = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int i) {   // fragment i of the next step
+    if (i < TB) fx[cur ^ 1][i < TB ? i : 0] = *reinterpret_cast<const bf16x8*>(nstx + (fx_o[i < TB ? i : 0] ^ (nkk << 6)));
+    else fw[cur ^ 1][i - TB] = *reinterpret_cast<const bf16x8*>(nstw + (fw_o[i - TB] ^ (nkk << 6)));
+  };
+  // One k32 step: 20 MFMAs on the fragments in buffer `cur` (weights on M, tokens on N). Behind every even MFMA goes one
+  // LDS read of the next step's fragments (into buffer cur ^ 1), behind the first n odd ones one global->LDS load of
+  // period `lit`. The interleaving is pinned with sched_group_barrier: left alone, the compiler hoists all fragment
+  // reads to the top of the iteration, where the wavefronts read them in one burst with no MFMA running; and a slice's
+  // loads in a row overflow the CU's load queue.
+  auto step = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int lit, int n) {
+#pragma unroll
+    for (int m = 0; m < NMF; ++m) {
+      const int rb = m / TB, tb = m % TB;
+      acc[rb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[cur][rb], fx[cur][tb], acc[rb][tb], 0, 0, 0);
+      const bool rd = (m % 2 == 0) && (m / 2 < NRD);
+      const bool ld = (m % 2 == 1) && (m / 2 < n);
+      if (rd) read_frag(cur, nstx, nstw, nkk, m / 2);
+      if (ld) issue_load(lit, m / 2);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);           // one MFMA
+      if (rd) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // its LDS read
+      if (ld) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // its VMEM read
+    }
+  };
+
+  // ---- prologue. Nothing in it may wait for a vector load before the first slice is needed: a wait counts back from
+  // the youngest load, so it would also wait for every look-ahead load issued before it. Hence: the one vector load
+  // of the prologue (a bias value per thread) goes out first and is not looked at until the epilogue; the rows'
+  // positions come through the scalar cache (a wavefront computes the cos/sin of 16 whole rows, so their indices are
+  // uniform); then all look-ahead loads, oldest first: slice 0, weight 1, activations 1, weight 2.
+  constexpr int CS_OFF = IMG_BYTES;
+  constexpr int BIAS_OFF = ring_bytes(BM);
+  float2* cs_tab = reinterpret_cast<float2*>(smem + CS_OFF);
+  float* bias_s = reinterpret_cast<float*>(smem + BIAS_OFF);
+  bf16 bias_raw;
+  {
+    const int c = tid < BN ? tid : BN - 1;
+    int h = head0 + (c >> 6);
+    if (h >= total_heads) h = total_heads - 1;
+    const bf16* bp = a.bias ? a.bias : a.W;                 // absent: a valid dummy address instead of a branch around the load
+    bias_raw = bp[h * 64 + (c & 63)];
+  }
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) issue_load(j < LPX ? -XS : -WS, j);
+#pragma unroll
+  for (int j = LPX; j < LPW; ++j) issue_load(-2, j);
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) issue_load(-1, j);
+  // cos/sin of (row, frequency) for the epilogue, computed while the first slices are in flight and kept in registers.
+  // Wavefront w: rows 16 w .. 16 w + 15 of the tile; lane: frequency lane % 32, rows 16 w + 2 j + lane / 32.
+  constexpr int CSN = 8;
+  static_assert(NW * 2 * CSN == EROWS && EROWS == BM, "eight wavefronts x two rows x eight rounds cover the tile");
+  float2 csr[CSN];
+  if (a.has_rope) {
+    const int f = lane & 31;
+    int64_t pos_even[CSN], pos_odd[CSN];
+    rope_positions_16_uniform(ra, a.W, row0 + 16 * wave, a.rows, pos_even, pos_odd);
+#pragma unroll
+    for (int j = 0; j < CSN; ++j) {
+      int64_t p = lane < 32 ? pos_even[j] : pos_odd[j];
+      if (!ra.positions) {                                  // uniform
+        int64_t grow = row0 + 16 * wave + 2 * j + (lane >> 5);
+        if (grow >= a.rows) grow = a.rows - 1;
+        p += grow < ra.tokens_per_batch ? grow : grow % ra.tokens_per_batch;
+      }
+      float c, sn;
+      rope_cos_sin(ra, fr, rope_wrap(p, ra.max_ctx), f, &c, &sn);
+      csr[j] = make_float2(c, sn);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");   // slice 0 has landed when only those are outstanding
+  __syncthreads();
+#pragma unroll
+  for (int tb = 0; tb < TB; ++tb) fx[0][tb] = *reinterpret_cast<const bf16x8*>(xring + fx_o[tb]);
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) fw[0][rb] = *reinterpret_cast<const bf16x8*>(wring + fw_o[rb]);
+
+  // ---- steady state. While slice `it` is multiplied, outstanding or landed, oldest first: the weight of slice it + 1,
+  // the activations of slice it + 1, the weight of slice it + 2. Step 0 of a slice reads the fragments of its step 1;
+  // then the slice's one barrier (this wavefront's share of slice it + 1 has landed -- everything but the newest weight
+  // slice --, then: everyone's has, and everyone has issued its last reads of slice it; spelled out, because
+  // __syncthreads() carries a fence that drains every load in flight, the look-ahead ones included); step 1 reads the
+  // fragments of the next slice's step 0 and hands the freed stages on.
+  for (int it = 0; it < n_iter; ++it) {
+    const unsigned char* stx = xring + (it % XS) * XSTAGE;
+    const unsigned char* stw = wring + (it % WS) * W_STAGE;
+    const unsigned char* nxx = xring + ((it + 1) % XS) * XSTAGE;
+    const unsigned char* nxw = wring + ((it + 1) % WS) * W_STAGE;
+    step(0, stx, stw, 1, 0, 0);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((WS - 2) * LPWW) : "memory");
+    step(1, nxx, nxw, 0, it, LPW);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // drain the look-ahead loads before LDS is reused
+  __syncthreads();
+
+  // ---- epilogue: the cos/sin table and the bias into the idle ring; bias, rotation, one rounding into a bf16 image of
+  // the tile (rows padded to 648 B); coalesced copy-out. The lane owns token m16 of each of its 16-token blocks and, in
+  // 16-row block b = 5 wn + rb of the tile, [lo(p), lo(p+1), hi(p), hi(p+1)] of head b / 4 with p = 8 (b % 4) + 2 g.
+  bf16* img = reinterpret_cast<bf16*>(smem);
+  const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
+  if (a.has_rope) {
+#pragma unroll
+    for (int j = 0; j < CSN; ++j) cs_tab[(16 * wave + 2 * j + (lane >> 5)) * CSROW + (lane & 31)] = csr[j];
+  }
+  if (tid < BN) bias_s[tid] = a.bias ? static_cast<float>(bias_raw) : 0.f;
+  __syncthreads();
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int b = RB * wn + rb;
+    const int hl = b >> 2;
+    int head = head0 + hl;
+    if (head >= total_heads) head = total_heads - 1;        // ragged last tile: computed, never copied out
+    const bool rotate = a.has_rope && head < a.n_q_heads + a.n_kv_heads;   // uniform per wavefront and block
+    const int p = 8 * (b & 3) + 2 * g;
+    const float2 b_lo = *reinterpret_cast<const float2*>(bias_s + hl * 64 + p);
+    const float2 b_hi = *reinterpret_cast<const float2*>(bias_s + hl * 64 + 32 + p);
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) {
+      const int r = 64 * wm + 16 * tb + m16;
+      float lo0 = acc[rb][tb][0] + b_lo.x, lo1 = acc[rb][tb][1] + b_lo.y;
+      float hi0 = acc[rb][tb][2] + b_hi.x, hi1 = acc[rb][tb][3] + b_hi.y;
+      if (rotate) {
+        const f32x4 cs = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + p);   // cos p, sin p, cos p+1, sin p+1
+        const float r0 = lo0 * cs[0] - hi0 * cs[1], r2 = hi0 * cs[0] + lo0 * cs[1];
+        const float r1 = lo1 * cs[2] - hi1 * cs[3], r3 = hi1 * cs[2] + lo1 * cs[3];
+        lo0 = r0;
+        lo1 = r1;
+        hi0 = r2;
+        hi1 = r3;
+      }
+      bf16x2 olo, ohi;
+      olo[0] = static_cast<bf16>(lo0);
+      olo[1] = static_cast<bf16>(lo1);
+      ohi[0] = static_cast<bf16>(hi0);
+      ohi[1] = static_cast<bf16>(hi1);
+      *reinterpret_cast<bf16x2*>(img + r * OROW + hl * 64 + p) = olo;
+      *reinterpret_cast<bf16x2*>(img + r * OROW + hl * 64 + 32 + p) = ohi;
+    }
+  }
+  __syncthreads();
+  prefill_copy_out<NT>(a, img, tid, head0, total_heads, row0, slot_off);
+}
+
+// ===================================================================================== the 256-token tile
+// LDS row i of the W tile -> (head within tile, dim within head): wavefront column w = i / 160 holds heads 3 w, 3 w + 1
+// whole (rows 0..127 of its 160) and its half of the tile's middle head (rows 128..159: 16 low dims, then their partners).
+__device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
+  const int w = i >= 160 ? 1 : 0;
+  const int j = i - 160 * w;
+  if (j < 128) {
+    *head_local = 3 * w + (j >> 6);
+    *dim = j & 63;
+  } else {
+    const int jj = j - 128;
+    *head_local = 2;
+    *dim = (jj < 16) ? (16 * w + jj) : (32 + 16 * w + (jj - 16));
+  }
+}
+
+__global__ __launch_bounds__(512) void qkv_prefill_kernel256(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
+  constexpr int BM = 256;
+  constexpr int WS = w_stages(BM);          // weight stages (2)
+  constexpr int KS = BK / 16;               // k16 MFMA steps per slice
+  constexpr int XSTAGE = x_stage(BM);
+  constexpr int NW = 8, NT = 512;
+  constexpr int MB = 2;                     // 32-token blocks per wavefront
+  constexpr int LPX = XSTAGE / 1024 / NW;   // load instructions (1 KiB blocks) per wavefront per slice: activations ...
+  constexpr int LPWW = W_STAGE / 1024 / NW; // ... weight
+  constexpr int LPW = LPX + LPWW;           // ... together
+  constexpr int NMF = MB * 5;               // MFMAs per k16 step
+  constexpr int NL_LAST = LPW < NMF ? LPW : NMF;   // loads handed out behind a slice's last step ...
+  constexpr int NL_FIRST = LPW - NL_LAST;          // ... and behind the next slice's first step
+  static_assert(WS == 2 && NL_FIRST <= NMF && KS % 2 == 0, "a slice's loads fit behind two k16 steps");
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  int tile_m, tile_n;
+  prefill_tile_of_block(blockIdx.x, tiles_m, tiles_n, swizzle, &tile_m, &tile_n);
+  const int64_t row0 = static_cast<int64_t>(tile_m) * BM;
+  const int head0 = tile_n * HPT;
+  const int total_heads = a.n_q_heads + 2 * a.n_kv_heads;
+  const int kvec = a.hidden >> 3;
+  const int n_iter = a.hidden / BK;
+
+  // ---- loader setup: as in the 128-token kernel
+  const int rotx = (blockIdx.x >> 3) % LPX, rotw = (blockIdx.x >> 3) % LPWW;
+  const unsigned char* const x_base = reinterpret_cast<const unsigned char*>(a.x) + row0 * a.hidden * 2;
+  const unsigned char* const w_base = reinterpret_cast<const unsigned char*>(a.W);
+  unsigned char* const wring = smem;
+  unsigned char* const xring = smem + WS * W_STAGE;
+  unsigned soff[LPW];
+  int blk_off[LPW];
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) {
+    if (j < LPX) {
+      const int bj = wave * LPX + (j + rotx) % LPX;
+      blk_off[j] = bj * 1024;
+      const int r = bj * RPB + lane / CHUNKS;
+      const int c = (lane % CHUNKS) ^ swz(r);
+      int64_t lr = r;
+      if (row0 + lr >= a.rows) lr = a.rows - 1 - row0;
+      soff[j] = static_cast<unsigned>((lr * kvec + c) * 16);
+    } else {
+      const int bj = wave * LPWW + (j - LPX + rotw) % LPWW;
+      blk_off[j] = bj * 1024;
+      const int r = bj * RPB + lane / CHUNKS;
+      const int c = (lane % CHUNKS) ^ swz(r);
+      int hl, dim;
+      w_tile_row(r, &hl, &dim);
+      int h = head0 + hl;
+      if (h >= total_heads) h = total_heads - 1;
+      soff[j] = static_cast<unsigned>(((static_cast<int64_t>(h) * 64 + dim) * kvec + c) * 16);
+    }
+  }
+
+  f32x16 acc[MB][5];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 5; ++nb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
+
+  // fragment addressing: byte offset of (row, chunk c) inside a stage is row*LROW + ((c ^ swz(row)) << 4). The k16 step
+  // kk wants chunks 2 kk + lh of the row; because a row starts on a 128-byte boundary the step enters as an XOR of bits
+  // 5-6 of the byte offset: one register per 32-row block instead of one per block and step. (Lanes 0-7 and 32-39,
+  // served together, read chunks 2 kk and 2 kk + 1 of eight consecutive rows: conflict-free under the swizzle.)
+  const int fa_row = 32 * MB * wm + l32, fb_row = 160 * wn + l32;
+  int fa_o[MB], fb_o[5];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) fa_o[mb] = (fa_row + 32 * mb) * LROW + ((lh ^ swz(fa_row + 32 * mb)) << 4);
+#pragma unroll
+  for (int nb = 0; nb < 5; ++nb) fb_o[nb] = (fb_row + 32 * nb) * LROW + ((lh ^ swz(fb_row + 32 * nb)) << 4);
+  // Period `per`: the activations of slice per + 2 and the weight of slice per + 2 into the stages slice `per` vacated.
+  auto issue_load = [&](int per, int j) {
+    const bool is_x = j < LPX;
+    const int sl = per + (is_x ? XS : WS);
+    const int slc = sl < n_iter ? sl : n_iter - 1;
+    unsigned char* dst = is_x ? xring + (sl % XS) * XSTAGE : wring + (sl % WS) * W_STAGE;
+    const unsigned lds_off = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst + blk_off[j]));
+    const unsigned char* sb = (is_x ? x_base : w_base) + static_cast<int64_t>(slc) * (BK * 2);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(soff[j]), "s"(sb) : "memory", "m0");
+  };
+  // One k16 step, 64 x 160 per wavefront: the two MFMAs that share a weight fragment are issued back to back and the
+  // fragment is reloaded for the next step right behind them (weight fragments single-buffered: 20 registers instead of
+  // 40, which is what keeps 160 accumulators + fragments inside 256 registers); the activation fragments of the next
+  // step go into their second buffer behind the first two pairs; for m < n one global->LDS load (j0 + m) of period `lit`.
+  bf16x8 fa[2][MB], fb[5];
+  auto step = [&](int cur, const unsigned char* nstx, const unsigned char* nstw, int nkk, int lit, int j0, int n) {
+#pragma unroll
+    for (int nb = 0; nb < 5; ++nb) {
+      acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nb], fa[cur][0], acc[0][nb], 0, 0, 0);   // weights on M, tokens on N
+      acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nb], fa[cur][1], acc[1][nb], 0, 0, 0);
+      fb[nb] = *reinterpret_cast<const bf16x8*>(nstw + (fb_o[nb] ^ (nkk << 5)));
+      if (nb < 2) fa[cur ^ 1][nb] = *reinterpret_cast<const bf16x8*>(nstx + (fa_o[nb] ^ (nkk << 5)));
+      if (2 * nb < n) issue_load(lit, j0 + 2 * nb);
+      if (2 * nb + 1 < n) issue_load(lit, j0 + 2 * nb + 1);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      if (nb < 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (2 * nb + 1 < n) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+      else if (2 * nb < n) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+  };
+
+  // prologue: slice 0 requested first; the rows' positions are parked in LDS for the epilogue (no registers to spare
+  // for cos/sin values), the bias widened once; then slice 1.
+  constexpr int CS_OFF = IMG_BYTES;
+  constexpr int BIAS_OFF = ring_bytes(BM);
+  float2* cs_tab = reinterpret_cast<float2*>(smem + CS_OFF);
+  float* bias_s = reinterpret_cast<float*>(smem + BIAS_OFF);
+  int64_t* pos_s = reinterpret_cast<int64_t*>(smem + BIAS_OFF + BIAS_BYTES);
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) issue_load(-2, j);
+  if (tid < BN) {
+    int h = head0 + (tid >> 6);
+    if (h >= total_heads) h = total_heads - 1;
+    bias_s[tid] = a.bias ? static_cast<float>(a.bias[h * 64 + (tid & 63)]) : 0.f;
+  }
+  if (a.has_rope) {
+    for (int r = tid; r < BM; r += NT) {
+      int64_t grow = row0 + r;
+      if (grow >= a.rows) grow = a.rows - 1;
+      pos_s[r] = rope_position_raw(ra, grow);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) issue_load(-1, j);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPW) : "memory");   // slice 0 has landed when only slice 1 is outstanding
+  __syncthreads();
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) fa[0][mb] = *reinterpret_cast<const bf16x8*>(xring + fa_o[mb]);
+#pragma unroll
+  for (int nb = 0; nb < 5; ++nb) fb[nb] = *reinterpret_cast<const bf16x8*>(wring + fb_o[nb]);
+
+  // Steady state. The one barrier per slice sits before the slice's last k16 step; from there on the stages of slice
+  // `it` are free (all reads of them have been issued) and period `it` goes out behind the MFMAs of this last step
+  // and, what does not fit there, of the next slice's first step.
+  for (int it = 0; it < n_iter; ++it) {
+    const unsigned char* stx = xring + (it % XS) * XSTAGE;
+    const unsigned char* stw = wring + (it % WS) * W_STAGE;
+    const unsigned char* nxx = xring + ((it + 1) % XS) * XSTAGE;
+    const unsigned char* nxw = wring + ((it + 1) % WS) * W_STAGE;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      if (kk + 1 < KS) {
+        if (kk == 0 && it > 0) step(kk & 1, stx, stw, kk + 1, it - 1, NL_LAST, NL_FIRST);
+        else step(kk & 1, stx, stw, kk + 1, 0, 0, 0);
+      } else {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        step(kk & 1, nxx, nxw, 0, it, 0, NL_LAST);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  // ---- epilogue, in two passes of 128 rows: the wavefronts that hold the pass's rows write the image, then everyone
+  // copies it out. Accumulator layout: the lane owns token l32 of each 32-token block and, in each 32-column block,
+  // columns 8*(v>>2) + 4*lh + (v&3) -- runs of four consecutive columns. A whole head is two blocks (low dims, their
+  // partners: same register index); the mixed block holds the wavefront's 16 low dims of the middle head in rows 0-15
+  // and their partners in rows 16-31 (register v and v + 8).
+  bf16* img = reinterpret_cast<bf16*>(smem);
+  const int64_t slot_off = qkv_slot(a, ra) * a.kv_slot_stride;
+#pragma unroll
+  for (int pass = 0; pass < BM / EROWS; ++pass) {
+    if (pass > 0) __syncthreads();                        // the previous pass's image and table have been read
+    if (a.has_rope) {
+      // table rows tid / 32 + 16 j, frequency tid % 32
+      const int f = tid & 31;
+      int64_t pos[EROWS / 16];
+#pragma unroll
+      for (int j = 0; j < EROWS / 16; ++j) pos[j] = pos_s[EROWS * pass + (tid >> 5) + 16 * j];
+#pragma unroll
+      for (int j = 0; j < EROWS / 16; ++j) {
+        float c, sn;
+        rope_cos_sin(ra, fr, rope_wrap(pos[j], ra.max_ctx), f, &c, &sn);
+        cs_tab[((tid >> 5) + 16 * j) * CSROW + f] = make_float2(c, sn);
+      }
+    }
+    __syncthreads();
+    const bool my_pass = (32 * MB * wm) / EROWS == pass;     // uniform per wavefront
+#pragma unroll
+    for (int hp = 0; hp < 3; ++hp) {
+      if (!my_pass) break;
+      const int hl = (hp < 2) ? (3 * wn + hp) : 2;
+      int head = head0 + hl;
+      if (head >= total_heads) head = total_heads - 1;
+      const bool rotate = a.has_rope && head < a.n_q_heads + a.n_kv_heads;
+      const int ngrp = hp < 2 ? 4 : 2;                         // groups of four (lo, hi) pairs per lane
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (g >= ngrp) continue;
+        const int d0 = hp < 2 ? (8 * g + 4 * lh) : (16 * wn + 8 * g + 4 * lh);   // first of the four consecutive low dims
+        const f32x4 b_lo = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + d0);
+        const f32x4 b_hi = *reinterpret_cast<const f32x4*>(bias_s + hl * 64 + 32 + d0);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const int r = 32 * MB * wm + 32 * mb + l32 - EROWS * pass;   // row inside the pass
+          float lo[4], hi[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (hp < 2) {
+              lo[j] = acc[mb][2 * hp][4 * g + j] + b_lo[j];
+              hi[j] = acc[mb][2 * hp + 1][4 * g + j] + b_hi[j];
+            } else {
+              lo[j] = acc[mb][4][4 * g + j] + b_lo[j];
+              hi[j] = acc[mb][4][8 + 4 * g + j] + b_hi[j];
+            }
+          }
+          bf16x4 olo, ohi;
+          if (rotate) {
+            const f32x4 c01 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0);       // (cos, sin) of dims d0, d0 + 1
+            const f32x4 c23 = *reinterpret_cast<const f32x4*>(cs_tab + r * CSROW + d0 + 2);   // ... d0 + 2, d0 + 3
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float c = j < 2 ? c01[2 * j] : c23[2 * j - 4], sn = j < 2 ? c01[2 * j + 1] : c23[2 * j - 3];
+              olo[j] = static_cast<bf16>(lo[j] * c - hi[j] * sn);
+              ohi[j] = static_cast<bf16>(hi[j] * c + lo[j] * sn);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              olo[j] = static_cast<bf16>(lo[j]);
+              ohi[j] = static_cast<bf16>(hi[j]);
+            }
+          }
+          *reinterpret_cast<bf16x4*>(img + r * OROW + hl * 64 + d0) = olo;
+          *reinterpret_cast<bf16x4*>(img + r * OROW + hl * 64 + 32 + d0) = ohi;
+        }
+      }
+    }
+    __syncthreads();
+    prefill_copy_out<NT>(a, img, tid, head0, total_heads, row0 + EROWS * pass, slot_off);
+  }
 }
 
 }  // namespace tllm
@@ -527,27 +679,25 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   a.bias = (const bf16*)b;
   if (rows == 0) return TLLM_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // the kernel addresses a tile's rows and the weight with 32-bit byte offsets
+  // the kernels address a tile's rows and the weight with 32-bit byte offsets
   const bool fast = head_dim == 64 && hidden % BK == 0 && aligned16(x) && aligned16(W) &&
                     static_cast<int64_t>(n_q_heads + 2 * n_kv_heads) * 64 * hidden * 2 < (1ll << 32) && 256 * hidden * 2 < (1ll << 32);
   if (!fast) {
     launch_qkv_generic(a, ra, fr, st);
     return check_launch("qkv_rope_prefill(generic)");
   }
-  constexpr int WROWS = 4;
   static bool attr_set = false;   // raising the dynamic-LDS limit is idempotent; a benign race at worst repeats it
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel<128, WROWS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, prefill_smem(128));
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_quads_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       prefill_smem(128));
     if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel<256, WROWS>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              prefill_smem(256));
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel256), hipFuncAttributeMaxDynamicSharedMemorySize, prefill_smem(256));
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_prefill: cannot raise LDS limit: %s", hipGetErrorString(e));
     attr_set = true;
   }
   const int heads = n_q_heads + 2 * n_kv_heads;
-  // Tile height by a two-number cost model: a round of 128-token tiles over the 256 CUs takes ~65 us, a round of
-  // 256-token tiles ~109 us (3 : 5); whichever needs less in total. T = 2048 is one round of 128s; anything that would
+  // Tile height by a two-number cost model: a round of 128-token tiles over the 256 CUs takes ~62 us, a round of
+  // 256-token tiles ~105 us (3 : 5); whichever needs less in total. T = 2048 is one round of 128s; anything that would
   // need a second round of 128s is one round of 256s instead, T = 8192 two rounds of 256s instead of four of 128s.
   const int64_t tn = (heads + HPT - 1) / HPT;
   const int64_t rounds128 = (((rows + 127) / 128) * tn + 255) / 256, rounds256 = (((rows + 255) / 256) * tn + 255) / 256;
@@ -560,10 +710,9 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   // 4 x 8 71 us, 2 x 16 and no grouping 75 us; from T = 4096 up (256-token tiles) the shape makes no difference.
   const int swizzle = (tiles_m % 8 == 0 && tiles_n % 4 == 0) ? 8 : 0;
   if (BM == 256)
-    hipLaunchKernelGGL((qkv_prefill_kernel<256, WROWS>), dim3((unsigned)tiles), dim3(WROWS * 128), prefill_smem(256), st, a, ra, fr,
-                       (int)tiles_m, tiles_n, swizzle);
+    hipLaunchKernelGGL(qkv_prefill_kernel256, dim3((unsigned)tiles), dim3(512), prefill_smem(256), st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
   else
-    hipLaunchKernelGGL((qkv_prefill_kernel<128, WROWS>), dim3((unsigned)tiles), dim3(WROWS * 128), prefill_smem(128), st, a, ra, fr,
-                       (int)tiles_m, tiles_n, swizzle);
+    hipLaunchKernelGGL(qkv_prefill_quads_kernel, dim3((unsigned)tiles), dim3(512), prefill_smem(128), st, a, ra, fr, (int)tiles_m, tiles_n,
+                       swizzle);
   return check_launch("qkv_rope_prefill");
 }
