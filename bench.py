@@ -452,7 +452,7 @@ def main() -> int:
         bench_kernel("rmsnorm_B8", lambda i: T.rmsnorm_forward(x, scales[i % N_LAYERS], 1e-5, out=t), bytes_of["rmsnorm"](B))
         bench_kernel("embedding_B8", lambda i: T.embedding_forward(ids, table, out=h), bytes_of["embedding"](B))
         bench_kernel("swiglu_M32", lambda i: T.swiglu(swiglu_x, out=s_out), bytes_of["swiglu"](SWIGLU_ROWS))
-        for r in (1, 8, 32):
+        for r in (1, 8, 16, 32):
             xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
             pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
             qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),

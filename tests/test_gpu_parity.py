@@ -444,12 +444,13 @@ def test_qkv_fp8_weight_decode_parity(gpu, yarn, rows, with_norm):
     close(v, vr)
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 13, 31])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 31])
 def test_streaming_decode_kernels_every_row_count(gpu, yarn, rows):
     """The kernels that stream their operands straight into LDS fetch only the rows that exist (the LDS of the others
     keeps what the launch before left there). Every row count of one workgroup, QKV and out-projection, bf16 and fp8
-    weight, with and without the fused norm; each run is preceded by one on NaN activations of the full 8 / 32 rows so
-    that whatever is left behind in LDS would show, and the rows behind the last one in memory are NaN as well."""
+    weight, with and without the fused norm (9 to 16 rows with the norm: the 16-row form of the 8-row kernel); each run
+    is preceded by one of the same kernel on NaN activations of its full 8 / 16 / 32 rows so that whatever is left
+    behind in LDS would show, and the rows behind the last one in memory are NaN as well."""
     full = 8 if rows <= 8 else 32
     d = O.make_inputs(rows, seed=900 + rows)
     w, b = d["w"].to(gpu), d["b"].to(gpu)
@@ -468,9 +469,10 @@ def test_streaming_decode_kernels_every_row_count(gpu, yarn, rows):
             if with_norm and rows > 16 and wscale is None:
                 continue                                    # composed of two launches above 16 rows: covered elsewhere
             kw = dict(weight_scale=wscale) if wscale is not None else {}
-            T.qkv_rope_forward(nan_x, weight, b, 64, 8, 64, yarn=yarn, positions=nan_pos, mode="decode", **kw)
             if with_norm:
                 kw.update(norm_scale=scale, norm_eps=1e-5)
+            nfull = min(full, 16) if with_norm else full
+            T.qkv_rope_forward(nan_x[:nfull], weight, b, 64, 8, 64, yarn=yarn, positions=nan_pos[:nfull], mode="decode", **kw)
             q, k, v = T.qkv_rope_forward(x, weight, b, 64, 8, 64, yarn=yarn, positions=pos, mode="decode", **kw)
             qr, kr, vr = O.qkv_rope_ref(normed if with_norm else d["x"], wref, d["b"], d["positions"])
             close(q, qr)

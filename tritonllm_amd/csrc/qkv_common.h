@@ -50,9 +50,9 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
                  int64_t k_rs, int64_t v_rs, int64_t kv_slot_stride, int64_t rows, int64_t hidden, int n_q_heads, int n_kv_heads,
                  int head_dim, const TllmRope* rope, QkvArgs* a, RopeArgs* ra, YarnFreqs* fr);
 
-// The hidden-2880 decode kernel for up to 8 rows per workgroup: bf16 or fp8 weight, optional fused RMSNorm and token
-// gather (qkv_decode_r8.hip).
-void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
+// The hidden-2880 decode kernel for up to xr = 8 rows per workgroup, or xr = 16 with the fused RMSNorm: bf16 or fp8 weight,
+// optional fused RMSNorm and token gather (qkv_decode_r8.hip).
+void launch_qkv_decode_r8(int xr, int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 // ... and for 9..32 rows per workgroup, bf16 or fp8 weight, activations already normalised (qkv_decode_r32.hip).
 void launch_qkv_decode_r32(bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 

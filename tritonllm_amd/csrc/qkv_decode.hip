@@ -5,10 +5,9 @@
 // the activation rows on the N side -- the MFMA does the K reduction across lanes for free and
 // leaves the VALU to the rotary epilogue -- and keep a rotation pair (row d and row d+32 of a
 // head) inside one workgroup so the rotation needs no second pass. The kernels:
-//   qkv_decode_r8_kernel   hidden == 2880 (gpt-oss), up to 8 rows, bf16 weight: qkv_decode_r8.hip, the fastest.
-//   qkv_decode_r32_kernel  hidden == 2880, 9..32 rows per workgroup, bf16 weight, no fused norm: qkv_decode_r32.hip.
-//   qkv_decode_cu_kernel   hidden == 2880, the other cases (fused norm beyond 8 rows, fp8 weight): one workgroup per CU, coalesced
-//                          loads, LDS-transposed operands; see its comment.
+//   qkv_decode_r8_kernel   hidden == 2880 (gpt-oss), up to 8 rows per workgroup, or up to 16 with the fused RMSNorm; bf16 or
+//                          fp8 weight, optional fused norm and token gather: qkv_decode_r8.hip, the fastest.
+//   qkv_decode_r32_kernel  hidden == 2880, 9..32 rows per workgroup, bf16 or fp8 weight, no fused norm: qkv_decode_r32.hip.
 //   qkv_decode_kernel      head_dim == 64, hidden % 32 == 0: operands loaded straight into MFMA
 //                          layout (simple, ~1.8x slower: every lane is its own cache-line request).
 //   qkv_generic_kernel     anything else: shuffle-reduced dot products.
@@ -198,414 +197,9 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   *reinterpret_cast<bf16x2*>(out + d0 + 32) = phi;
 }
 
-// ------------------------------------------------------------------------------------------------
-// One-workgroup-per-CU variant for hidden == 2880 (the default decode kernel).
-//
-// The 2560 rotation pairs are dealt out ten at a time: 256 workgroups, each needing most of a CU's
-// LDS, so the dispatcher has to place exactly one per CU and every CU streams exactly 1/256 of the
-// weight (20 rows x 5760 B). Fifteen wavefronts split K (six k32-steps each); all loads of the
-// kernel -- the small ones the epilogue needs first, then activations, then weights -- are issued
-// unconditionally (indices clamped, never predicated) before anything is consumed, so the compiler
-// has no join to wait at and ~180 KB per CU is in flight from the first microsecond.
-// Loads are coalesced along K; the MFMA operand layout is produced by a pass through a
-// wavefront-private LDS patch. v_mfma_f32_32x32x16_bf16: M = 32 tile rows (pair slot p at row p, its
-// partner at row p + 16), N = up to XR activation rows. After one barrier the fifteen partial tiles
-// are summed by 16 x XR threads, one (pair, activation row) each, which also add the bias, rotate
-// with cos/sin they computed while the loads were in flight, round once and store.
-// NORM: 0 = x is used as it is; 1 / 2 = x is first RMS-normalised with an fp32 / bf16 scale (fused prologue).
-// W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row, W[n][k] = fp8[n][k] * w_scale[n]
-// (triton_kernels.py:261-268, 927-940, 963-965). Half the bytes to stream; the values are widened to bf16 (exact)
-// on their way into the LDS patch, so the MFMAs and the fp32 accumulation are those of the bf16 kernel, and the
-// row scale multiplies the finished sum.
-// EMB: the activation rows are gathered from an embedding table by token id (the first layer of a decode step:
-// model.py:906-920 feeds the gather straight into the first block's norm + QKV); the workgroup with blockIdx.x == 0
-// also writes the gathered rows out, as the residual stream. An id outside the table gives a zero row (its loads are
-// clamped to a real row and the values discarded) and raises the flag, as the stand-alone gather does.
-template <int XR, int CH, int NORM, bool W8, bool EMB = false>
-__global__ __launch_bounds__(960) void qkv_decode_cu_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
-  static_assert(!EMB || NORM != 0, "the fused gather exists with the fused norm only");
-  constexpr int NW = 15, SPW = 6, NCH = SPW / CH, PAIRS = 10;
-  constexpr int KV = 360;                 // 16-byte vectors per activation row (hidden 2880)
-  constexpr int KVW = W8 ? 180 : 360;     // ... per weight row
-  constexpr int WROW = CH * 64 + 16;      // padded patch row, bytes
-  constexpr int CPR = CH * 4;             // 16-byte chunks per row per patch (bf16)
-  constexpr int CPRW = W8 ? CPR / 2 : CPR;            // ... of the weight as it lies in memory
-  constexpr int WL = (2 * PAIRS * CPRW + 63) / 64;    // weight load instructions per patch
-  constexpr int XL = (XR * CPR + 63) / 64;          // activation load instructions per patch
-  constexpr int PATCH = (32 + XR) * WROW;
-  constexpr int RED = XR * 32;            // floats per wavefront in the reduction buffer
-  static_assert(SPW % CH == 0, "patches must tile the K slice");
-  static_assert(NW * RED * 4 <= NW * PATCH, "reduction buffer aliases the patches");
-  static_assert(16 * XR <= 960, "one epilogue thread per (pair slot, activation row)");
-  __shared__ __align__(16) unsigned char lds[NW * PATCH];
-  __shared__ float s_pin[16];
-  __shared__ float s_part[NORM ? NW * XR : 1], s_rinv[NORM ? XR : 1];
-  static_assert((NCH * XR * CPR + SPW * 32) * 4 <= PATCH, "sum-of-squares and scale scratch alias the wavefront's patch");
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int total_pairs = (a.n_q_heads + 2 * a.n_kv_heads) * 32;
-  const int pair0 = blockIdx.x * PAIRS;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
-  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
-
-  // ---- epilogue role of this thread: pair slot es, activation row en (clamped to real ones for the loads)
-  const int es = tid & 15, en = tid >> 4;
-  const bool evalid = tid < 16 * XR && es < PAIRS && pair0 + es < total_pairs && en < nvalid;
-  const int egp = evalid ? pair0 + es : 0;
-  const int ehead = egp >> 5, ed = egp & 31;
-  const int64_t erow = row0 + (evalid ? en : 0);
-  const bool erot = a.has_rope && ehead < a.n_q_heads + a.n_kv_heads;
-
-  // ---- every global load of the kernel, oldest first
-  const int64_t* pos_ptr = ra.positions ? ra.positions + erow : reinterpret_cast<const int64_t*>(a.W);
-  const int64_t* off_ptr = ra.offset ? ra.offset : reinterpret_cast<const int64_t*>(a.W);
-  const unsigned short* bias_ptr = reinterpret_cast<const unsigned short*>(a.bias ? a.bias : a.W);
-  const int64_t pos_ld = *pos_ptr;
-  const int64_t off_ld = *off_ptr;
-  // The 32-row variant with the fused norm has no register left to hold the two bias values through the kernel
-  // (the compiler would spill them at the very top, behind a full wait for the first loads): it fetches them
-  // after the MFMAs instead, where the two reduction barriers cover the latency.
-  constexpr bool LATE_BIAS = NORM != 0 && XR == 32;
-  unsigned short b_lo = 0, b_hi = 0;
-  if constexpr (!LATE_BIAS) {
-    b_lo = bias_ptr[ehead * 64 + ed];
-    b_hi = bias_ptr[ehead * 64 + 32 + ed];
-  }
-  const float freq = fr.v[ed];
-  float ws_lo = 1.f, ws_hi = 1.f;
-  if constexpr (W8) {
-    ws_lo = a.w_scale[ehead * 64 + ed];
-    ws_hi = a.w_scale[ehead * 64 + 32 + ed];
-  }
-  __builtin_amdgcn_sched_barrier(0);
-
-  const bf16x8* xg = reinterpret_cast<const bf16x8*>(a.x) + row0 * KV + wave * (SPW * 4);
-  const bf16x8* wg = reinterpret_cast<const bf16x8*>(a.W) + wave * (W8 ? SPW * 2 : SPW * 4);   // 16-byte units either way
-  bf16x8 xr[NCH * XL], wr[NCH * WL];
-  // The norm scale of this wavefront's K slice (SPW * 32 values): one load per wavefront, parked in LDS later.
-  f32x4 sc32 = {};
-  bf16x8 sc16 = {};
-  if constexpr (NORM == 1) sc32 = reinterpret_cast<const f32x4*>(a.norm_scale)[wave * (SPW * 8) + (lane < SPW * 8 ? lane : SPW * 8 - 1)];
-  if constexpr (NORM == 2) sc16 = reinterpret_cast<const bf16x8*>(a.norm_scale)[wave * (SPW * 4) + (lane < SPW * 4 ? lane : SPW * 4 - 1)];
-  // EMB: where each of this lane's activation rows starts in the table (one id per load slot, fetched first)
-  const bf16x8* xsrc[XL];
-  bool xok[XL];
-  if constexpr (EMB) {
-    int64_t id[XL];
-#pragma unroll
-    for (int i = 0; i < XL; ++i) {
-      int e = i * 64 + lane;
-      e = e < XR * CPR ? e : XR * CPR - 1;
-      int r = e / CPR;
-      r = r < nvalid ? r : nvalid - 1;
-      id[i] = a.emb_ids_i64 ? reinterpret_cast<const int64_t*>(a.emb_ids)[row0 + r]
-                            : static_cast<int64_t>(reinterpret_cast<const int*>(a.emb_ids)[row0 + r]);
-    }
-#pragma unroll
-    for (int i = 0; i < XL; ++i) {
-      const bool ok = id[i] >= 0 && id[i] < a.emb_vocab;
-      xok[i] = ok;
-      if (!ok && a.emb_oob) *a.emb_oob = 1;
-      const int64_t idc = id[i] < 0 ? 0 : (id[i] < a.emb_vocab ? id[i] : a.emb_vocab - 1);
-      xsrc[i] = reinterpret_cast<const bf16x8*>(a.emb_table) + idc * KV + wave * (SPW * 4);
-    }
-  }
-  auto load_x = [&]() {
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-#pragma unroll
-      for (int i = 0; i < XL; ++i) {          // patch chunk e -> activation row e / CPR, chunk e % CPR
-        int e = i * 64 + lane;
-        e = e < XR * CPR ? e : XR * CPR - 1;
-        int r = e / CPR;
-        const int kc = e - r * CPR;
-        r = r < nvalid ? r : nvalid - 1;
-        if constexpr (EMB) xr[j * XL + i] = xsrc[i][j * CPR + kc];
-        else xr[j * XL + i] = xg[r * KV + j * CPR + kc];
-      }
-    }
-  };
-  // Order of the requests. All 256 workgroups read the same few activation rows, which the L2s can only hand
-  // out at their own pace (32 CUs per L2 asking for the same lines), while the weight stream has the whole
-  // HBM latency ahead of it: without the norm the weight requests go first and the activations follow in
-  // their shadow. With the fused norm the activations are needed first (see below).
-  if constexpr (NORM != 0) load_x();
-  auto load_w = [&](int idx) {               // weight load idx: patch j = idx / WL, chunk slot i = idx % WL
-    const int j = idx / WL, i = idx % WL;
-    int e = i * 64 + lane;                    // patch chunk e -> weight row e / CPRW: the ten low rows, then their partners
-    e = e < 2 * PAIRS * CPRW ? e : 2 * PAIRS * CPRW - 1;
-    const int r = e / CPRW, kc = e - r * CPRW;
-    int gp = pair0 + (r < PAIRS ? r : r - PAIRS);
-    gp = gp < total_pairs ? gp : total_pairs - 1;
-    const unsigned wrow = static_cast<unsigned>(gp >> 5) * 64u + (gp & 31) + (r < PAIRS ? 0u : 32u);
-    wr[idx] = __builtin_nontemporal_load(wg + wrow * static_cast<unsigned>(KVW) + j * CPRW + kc);
-  };
-  // A CU holds a bounded number of loads in flight and a wavefront stalls when it issues one beyond that. With
-  // the fused norm every wavefront must see its activations, and meet the others at a barrier, before any MFMA
-  // can start; a wavefront stuck issuing weight loads would get there only when the stream has almost drained.
-  // So only the first NEARLY weight loads are requested up front (enough to keep the memory pipe busy during
-  // the norm), behind a rendezvous that puts every wavefront's activation loads ahead of them in the queue;
-  // the rest follow right after the norm's barriers.
-  constexpr int NEARLY = NORM == 0 ? NCH * WL : (XR == 32 ? 0 : 2);   // XR == 32 has no registers to spare for any
-  if constexpr (NORM != 0) __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int idx = 0; idx < NEARLY; ++idx) load_w(idx);
-  if constexpr (NORM == 0) load_x();
-  __builtin_amdgcn_sched_barrier(0);
-
-  // ---- cos/sin of this thread's (pair, row) while the weights are in flight.
-  // The store pins the frequency load above the weight stream: with its only use inside the
-  // conditional below, the compiler would sink it there and then have to drain every load to read it.
-  s_pin[es] = freq;
-  float cs = 1.f, sn = 0.f;
-  const int64_t slot = (a.kv_slot_stride != 0 && ra.offset != nullptr) ? off_ld : 0;
-  // Only the first 16 * XR threads have an epilogue role; the test is uniform per wavefront, and the other
-  // wavefronts must skip this: the 64-bit position arithmetic and the sincos are some six hundred vector
-  // instructions, and fifteen wavefronts doing them on four SIMDs would take as long as the whole weight stream.
-  if (a.has_rope && tid < 16 * XR) {
-    int64_t pos = ra.positions ? pos_ld : (erow % ra.tokens_per_batch) + (ra.offset ? off_ld : 0);
-    pos = rope_wrap(pos, ra.max_ctx);
-    if (ra.use_yarn) yarn_cos_sin(pos, freq, ra.concentration, &cs, &sn);
-    else rope_cos_sin(ra, fr, pos, ed, &cs, &sn);
-  }
-
-  __builtin_amdgcn_sched_barrier(0);
-
-  // ---- fused RMSNorm prologue: turn the raw activation chunks held in registers into
-  // bf16(x * rsqrt(mean(x^2) + eps) * scale), the exact operand the two-launch form passes between its kernels.
-  // Sum of squares: per-chunk partials -> the wavefront's LDS patch (idle so far) -> one lane per row adds its
-  // row's chunks -> the fifteen K slices meet in s_part -> s_rinv.
-  if constexpr (NORM != 0) {
-    float* tmp = reinterpret_cast<float*>(lds + wave * PATCH);
-    float* wscale = tmp + NCH * XR * CPR;
-    if constexpr (EMB) {                      // an id outside the table stands for a zero row (the load itself read a real one)
-#pragma unroll
-      for (int c = 0; c < NCH * XL; ++c) {
-        if (!xok[c % XL]) {
-#pragma unroll
-          for (int q = 0; q < 8; ++q) xr[c][q] = static_cast<bf16>(0.f);
-        }
-      }
-    }
-    if constexpr (NORM == 1) {
-      if (lane < SPW * 8) reinterpret_cast<f32x4*>(wscale)[lane] = sc32;
-    } else {
-      if (lane < SPW * 4) {
-        f32x4 lo4, hi4;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          lo4[q] = static_cast<float>(sc16[q]);
-          hi4[q] = static_cast<float>(sc16[4 + q]);
-        }
-        reinterpret_cast<f32x4*>(wscale)[2 * lane] = lo4;
-        reinterpret_cast<f32x4*>(wscale)[2 * lane + 1] = hi4;
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < NCH * XL; ++c) {
-      const int e = (c % XL) * 64 + lane;
-      float ssq = 0.f;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float f = static_cast<float>(xr[c][q]);
-        ssq = fmaf(f, f, ssq);
-      }
-      if (e < XR * CPR) tmp[(c / XL) * (XR * CPR) + e] = ssq;
-    }
-    if constexpr (EMB) {
-      if (blockIdx.x == 0) {                  // one workgroup per row chunk leaves the gathered rows behind
-        bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + row0 * KV + wave * (SPW * 4);
-#pragma unroll
-        for (int c = 0; c < NCH * XL; ++c) {
-          const int e = (c % XL) * 64 + lane;
-          const int r = e / CPR, kc = e - r * CPR;
-          if (e < XR * CPR && r < nvalid) xo[r * KV + (c / XL) * CPR + kc] = xr[c];
-        }
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    if (lane < XR) {
-      float p = 0.f;
-#pragma unroll
-      for (int j = 0; j < NCH; ++j) {
-#pragma unroll
-        for (int c = 0; c < CPR / 4; ++c) {
-          const f32x4 t4 = *reinterpret_cast<const f32x4*>(tmp + j * (XR * CPR) + lane * CPR + 4 * c);
-          p += (t4[0] + t4[1]) + (t4[2] + t4[3]);
-        }
-      }
-      s_part[wave * XR + lane] = p;
-    }
-    __syncthreads();
-    if (tid < XR) {
-      float ss = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) ss += s_part[w * XR + tid];
-      s_rinv[tid] = rsqrtf(ss * (1.0f / 2880.0f) + a.norm_eps);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int idx = NEARLY; idx < NCH * WL; ++idx) load_w(idx);
-    __builtin_amdgcn_sched_barrier(0);
-    // Chunk c's scale values and 1/rms are fetched from LDS while chunk c-1 is being scaled, and each chunk is
-    // fenced off from the next: written plainly, the compiler either serialises every LDS latency or sinks the
-    // arithmetic down to the patch writes and keeps every chunk's scale values alive until then, next to all the
-    // weight loads' destination registers (it then spills those, with a full drain of the load queue each).
-    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
-    constexpr int NC = NCH * XL;
-    f32x4 s_lo, s_hi, n_lo = {}, n_hi = {};
-    float rinv, n_rinv = 0.f;
-    auto fetch = [&](int c, f32x4& lo4, f32x4& hi4, float& ri) {
-      int e = (c % XL) * 64 + lane;
-      e = e < XR * CPR ? e : XR * CPR - 1;
-      const f32x4* sp = reinterpret_cast<const f32x4*>(wscale) + 2 * ((c / XL) * CPR + e % CPR);
-      lo4 = sp[0];
-      hi4 = sp[1];
-      ri = s_rinv[e / CPR];
-    };
-    fetch(0, s_lo, s_hi, rinv);
-#pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      if (c + 1 < NC) fetch(c + 1, n_lo, n_hi, n_rinv);
-      __builtin_amdgcn_sched_barrier(0);
-      u32x4 bits = __builtin_bit_cast(u32x4, xr[c]);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        asm volatile("" : "+v"(bits[q]));       // the fp32 copies of the sum-of-squares pass must not stay alive
-        bf16x2 t;
-        t[0] = static_cast<bf16>(__uint_as_float(bits[q] << 16) * rinv * (q < 2 ? s_lo[2 * q] : s_hi[2 * q - 4]));
-        t[1] = static_cast<bf16>(__uint_as_float(bits[q] & 0xffff0000u) * rinv * (q < 2 ? s_lo[2 * q + 1] : s_hi[2 * q - 3]));
-        bits[q] = __builtin_bit_cast(unsigned, t);
-        asm volatile("" : "+v"(bits[q]));       // ... and the arithmetic must not sink to the patch write below
-      }
-      xr[c] = __builtin_bit_cast(bf16x8, bits);
-      __builtin_amdgcn_sched_barrier(0);
-      s_lo = n_lo;
-      s_hi = n_hi;
-      rinv = n_rinv;
-    }
-  }
-
-  f32x16 acc;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-  const int m = lane & 31, h = lane >> 5;
-  unsigned char* wp = lds + wave * PATCH;            // 32 tile rows (only those of real pairs are written)
-  unsigned char* xp = wp + 32 * WROW;                // XR activation rows
-  const unsigned char* wfrag = wp + m * WROW + h * 16;
-  const unsigned char* xfrag = xp + (m & (XR - 1)) * WROW + h * 16;   // stale LDS in unused rows/columns is never stored
-#pragma unroll
-  for (int j = 0; j < NCH; ++j) {
-#pragma unroll
-    for (int i = 0; i < XL; ++i) {
-      const int e = i * 64 + lane;
-      const int r = e / CPR, kc = e - r * CPR;
-      if (e < XR * CPR && r < nvalid) *reinterpret_cast<bf16x8*>(xp + r * WROW + kc * 16) = xr[j * XL + i];
-    }
-#pragma unroll
-    for (int i = 0; i < WL; ++i) {
-      const int e = i * 64 + lane;
-      const int r = e / CPRW, kc = e - r * CPRW;
-      const int trow = r < PAIRS ? r : r - PAIRS + 16;
-      if constexpr (W8) {
-        // sixteen fp8 -> sixteen bf16 (exact: e4m3 fits), two chunks of the patch row
-        typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
-        typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
-        const i32x4 raw = __builtin_bit_cast(i32x4, wr[j * WL + i]);
-        bf16x8 w0, w1;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[d], false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[d], true);
-          bf16x8& dst = d < 2 ? w0 : w1;
-          dst[4 * (d & 1) + 0] = static_cast<bf16>(p0[0]);
-          dst[4 * (d & 1) + 1] = static_cast<bf16>(p0[1]);
-          dst[4 * (d & 1) + 2] = static_cast<bf16>(p1[0]);
-          dst[4 * (d & 1) + 3] = static_cast<bf16>(p1[1]);
-        }
-        if (e < 2 * PAIRS * CPRW) {
-          *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 32) = w0;
-          *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 32 + 16) = w1;
-        }
-      } else {
-        if (e < 2 * PAIRS * CPRW) *reinterpret_cast<bf16x8*>(wp + trow * WROW + kc * 16) = wr[j * WL + i];
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int t = 0; t < 2 * CH; ++t) {
-      const bf16x8 fa = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
-      const bf16x8 fb = *reinterpret_cast<const bf16x8*>(xfrag + t * 32);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-  }
-  if constexpr (LATE_BIAS) {
-    b_lo = bias_ptr[ehead * 64 + ed];
-    b_hi = bias_ptr[ehead * 64 + 32 + ed];
-  }
-  // ---- fifteen partial tiles -> LDS as [wave][tile row][activation row] (lanes of one store hit distinct banks)
-  __syncthreads();
-  float* red = reinterpret_cast<float*>(lds);
-  if (m < XR) {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) red[wave * RED + (8 * (v >> 2) + 4 * h + (v & 3)) * XR + m] = acc[v];
-  }
-  __syncthreads();
-  if (!evalid) return;
-  float lo = 0.f, hi = 0.f;
-#pragma unroll
-  for (int w = 0; w < NW; ++w) {
-    lo += red[w * RED + es * XR + en];
-    hi += red[w * RED + (16 + es) * XR + en];
-  }
-  if constexpr (W8) {
-    lo *= ws_lo;
-    hi *= ws_hi;
-  }
-  if (a.bias) {
-    lo += __uint_as_float(static_cast<unsigned>(b_lo) << 16);
-    hi += __uint_as_float(static_cast<unsigned>(b_hi) << 16);
-  }
-  if (erot) {
-    const float rl = lo * cs - hi * sn, rh = hi * cs + lo * sn;
-    lo = rl;
-    hi = rh;
-  }
-  bf16* out = qkv_out_ptr(a, slot, erow, ehead);
-  out[ed] = static_cast<bf16>(lo);
-  out[ed + 32] = static_cast<bf16>(hi);
-}
-
 }  // namespace tllm
 
 using namespace tllm;
-
-// The kernel above serves what the two streaming kernels do not: the fused norm (and gather) at 9..16 rows.
-static void launch_cu_embed(int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
-#define TLLM_CUE(NORM)                                                                                              \
-  do {                                                                                                              \
-    if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<16, 3, NORM, true, true>), grid, dim3(960), 0, st, a, ra, fr);  \
-    else hipLaunchKernelGGL((qkv_decode_cu_kernel<16, 3, NORM, false, true>), grid, dim3(960), 0, st, a, ra, fr);    \
-  } while (0)
-  if (norm == 1) TLLM_CUE(1);
-  else TLLM_CUE(2);
-#undef TLLM_CUE
-}
-
-static void launch_cu(int xr, int norm, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
-#define TLLM_CU(XR, CH, NORM)                                                                                   \
-  do {                                                                                                          \
-    if (w8) hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, true>), grid, dim3(960), 0, st, a, ra, fr);  \
-    else hipLaunchKernelGGL((qkv_decode_cu_kernel<XR, CH, NORM, false>), grid, dim3(960), 0, st, a, ra, fr);    \
-  } while (0)
-  (void)xr;                                                               // 16: the only height left
-  if (norm == 1) TLLM_CU(16, 3, 1);
-  else TLLM_CU(16, 3, 2);
-#undef TLLM_CU
-}
 
 // Shared tail of the hidden-2880 decode entry points: row-count -> kernel variant and grid.
 static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr, int norm, bool w8, int64_t rows,
@@ -615,15 +209,14 @@ static int launch_decode_2880(const char* what, QkvArgs& a, const RopeArgs& ra, 
   // the fused gather addresses table rows with 32-bit byte offsets
   TLLM_REQUIRE(!emb || a.emb_vocab * 5760 < (1ll << 32), TLLM_E_SHAPE, "%s: embedding table of %lld rows too large for the fused gather", what,
                (long long)a.emb_vocab);
-  const bool r32 = rows > 8 && norm == 0 && !emb;                          // 9..32 rows per workgroup, normalised activations
-  const int xr = rows <= 8 ? 8 : ((rows <= 16 && !r32) ? 16 : 32);
+  // up to 8 rows: the 8-row streaming kernel; 9..16 rows with the fused norm (and gather): its 16-row form; everything
+  // else (no norm: the callers refuse a fused norm above 16 rows) the 32-row kernel, one pass over the weight per 32 rows
+  const int xr = rows <= 8 ? 8 : ((rows <= 16 && (norm != 0 || emb)) ? 16 : 32);
   const int64_t chunks = (rows + xr - 1) / xr;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many for the decode kernel", what, (long long)rows);
   const dim3 grid((unsigned)((heads * 32 + 9) / 10), (unsigned)chunks);
-  if (r32) launch_qkv_decode_r32(w8, grid, st, a, ra, fr);
-  else if (xr == 8) launch_qkv_decode_r8(norm, emb, w8, grid, st, a, ra, fr);
-  else if (emb) launch_cu_embed(norm, w8, grid, st, a, ra, fr);
-  else launch_cu(xr, norm, w8, grid, st, a, ra, fr);
+  if (xr == 32) launch_qkv_decode_r32(w8, grid, st, a, ra, fr);
+  else launch_qkv_decode_r8(xr, norm, emb, w8, grid, st, a, ra, fr);
   return check_launch(what);
 }
 

@@ -1,5 +1,5 @@
 // Decode-size fused (RMSNorm +) QKV projection + bias + rotary for hidden == 2880 and up to 8 activation rows per
-// workgroup: the weight-streaming kernel of the gpt-oss decode step (B <= 8).
+// workgroup -- the weight-streaming kernel of the gpt-oss decode step (B <= 8) -- and, with the fused norm, up to 16.
 //
 // Work per CU. The 2560 rotation pairs are dealt ten at a time to 256 workgroups, each needing most of a CU's LDS, so
 // exactly one lands on every CU and every CU streams 1/256 of the weight: 20 rows of 5760 bytes. The rows form two
@@ -31,6 +31,10 @@
 // fp32 arithmetic, one rounding to bf16: the operand the separate rmsnorm launch would hand over.
 // EMB: the activation rows are gathered from an embedding table by token id (model.py:906-920 feeding the first
 // block); workgroup 0 also writes the gathered rows out. An id outside the table gives a zero row and raises the flag.
+// XR: 8 or 16 activation rows per workgroup. Sixteen rows (with the fused norm only; without it qkv_decode_r32.hip
+// takes 9..32 rows) fill the MFMA's 16 columns and 96 KB of LDS, which leaves room for one ring region: phase 0 lands
+// there and is requested before the norm; the later phases are requested after the sums are published -- by then the
+// activation fragments are in registers -- and land in the activation blocks.
 // W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (triton_kernels.py:261-268, 927-965). A
 // wavefront's 480 bytes of a row arrive in two phases of 8 + 7 k32 steps (256 + 224 bytes, so a row piece is as long
 // as in the bf16 form and the LDS layout is the same), fragments are widened to bf16 (exact) between the LDS read and
@@ -40,14 +44,13 @@
 namespace tllm {
 
 namespace r8 {
-constexpr int XR = 8;             // activation rows per workgroup
 constexpr int NS = 6;             // streaming wavefronts = K slices
 constexpr int NE = 2;             // epilogue wavefronts = tiles
 constexpr int STEPS = 15;         // k32 steps per slice
 constexpr int PAIRS = 10;         // rotation pairs per workgroup
-constexpr int RING = 3;           // resident phases per wavefront
 constexpr int REGION = 20 * 256;  // one phase: 20 weight rows x four k32 steps
 constexpr int XBLOCK = 1024;      // one activation row of a slice: 60 chunks of 16 bytes (+ 4 spare)
+constexpr int ring_regions(int xr) { return xr == 8 ? 3 : 1; }   // ring regions per wavefront
 }  // namespace r8
 
 // Set (and never cleared) by a wavefront whose bounded wait for the other wavefronts' norm sums ran out.
@@ -61,14 +64,19 @@ __device__ unsigned long long g_r8_stamps[256 * 8 * 8];
 #define R8_STAMP(i) do { } while (0)
 #endif
 
-template <int NORM, bool EMB, bool W8>
+template <int XR, int NORM, bool EMB, bool W8>
 __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int out4) {
   using namespace r8;
   static_assert(!EMB || NORM != 0, "the fused gather exists with the fused norm only");
+  static_assert(XR == 8 || (XR == 16 && NORM != 0), "sixteen rows: with the fused norm only");
+  constexpr int RING = ring_regions(XR);
   constexpr int LPW = 5;                                    // weight load instructions per phase and wavefront
   constexpr int NPH = W8 ? 2 : 4;                           // phases: bf16 4 + 4 + 4 + 3 k32 steps, fp8 8 + 7
   constexpr int PSTEPS = W8 ? 8 : 4;                        // k32 steps of a full phase
-  constexpr int RPH = W8 ? 2 : RING;                        // phases that land in the ring (the last bf16 phase lands in the activation blocks)
+  // phases that land in the ring; the others land in the activation blocks, which are free once the activation
+  // fragments are in registers (8 rows: the last bf16 phase; 16 rows: every phase but the first)
+  constexpr int RPH = XR == 8 ? (W8 ? 2 : RING) : 1;
+  static_assert((NPH - RPH) * REGION <= XR * XBLOCK, "the phases behind the ring fit the activation blocks");
   __shared__ __align__(1024) unsigned char xw[NS * XR * XBLOCK];
   __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
   __shared__ __align__(1024) unsigned char scw[NORM ? NS * 2048 : 16];
@@ -91,7 +99,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     if constexpr (NORM != 0) __syncthreads();
     StreamEpilogueLane<W8> ep;
     ep.prepare(a, ra, fr, pair0, tile, lane >> 4, lane & 15, row0, nvalid);   // quad of the tile, activation row
-    unsigned red_o = static_cast<unsigned>(REGION + tile * 1024 + lane * 16);
+    unsigned red_o = static_cast<unsigned>((RING > 1 ? REGION : 0) + tile * 1024 + lane * 16);
     asm volatile("" : "+v"(red_o));
     __syncthreads();                                        // partial tiles are in LDS
     R8_STAMP(6);
@@ -123,7 +131,8 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     if constexpr (W8) return c < 32 ? kq * 512 + c * 16 : 3072 + kq * 448 + (c - 32) * 16;
     else return c < 48 ? (c >> 4) * 1536 + kq * 256 + (c & 15) * 16 : 4608 + kq * 192 + (c - 48) * 16;
   };
-  const int m = lane & 15, g = lane >> 4, m1 = m & 7;
+  const int m = lane & 15, g = lane >> 4;
+  const int m1 = XR == 8 ? (m & 7) : m;                     // activation row of the lane's MFMA column (8 rows: columns 8..15 repeat 0..7, never stored)
   unsigned char* myx = xw + wave * (XR * XBLOCK);
   unsigned char* myring = ring + wave * (RING * REGION);
 
@@ -133,6 +142,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   // 32-bit lane offsets from a scalar base: the workgroup's first row, or (EMB) the table, whose size the host checks
   const unsigned char* xbase = EMB ? reinterpret_cast<const unsigned char*>(a.emb_table) : reinterpret_cast<const unsigned char*>(a.x) + row0 * 5760;
   bool xok_m1 = true;                                       // EMB: is the id of the row this lane's fragments belong to inside the table?
+  static_assert(2 * (XR - 1) < 64, "the row swizzle stays inside a 1 KB block");
   {
     int64_t src_row[XR];
 #pragma unroll
@@ -140,7 +150,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     if constexpr (EMB) {
       int64_t id[XR];
 #pragma unroll
-      for (int n = 0; n < XR; ++n) {                        // all eight ids first: nothing between these loads that could order them
+      for (int n = 0; n < XR; ++n) {                        // all ids first: nothing between these loads that could order them
         id[n] = a.emb_ids_i64 ? reinterpret_cast<const int64_t*>(a.emb_ids)[src_row[n]]
                               : static_cast<int64_t>(reinterpret_cast<const int*>(a.emb_ids)[src_row[n]]);
       }
@@ -182,9 +192,9 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
   }
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
-  // Phases 0..2 land in the wavefront's three ring regions, phase 3 in its activation blocks, which are free as soon
-  // as the activation fragments are in registers -- so no weight load ever waits for an MFMA.
-  auto phase_region = [&](int p) -> unsigned char* { return p < RING ? myring + p * REGION : myx; };
+  // The first RPH phases land in the wavefront's ring regions, the others in its activation blocks, which are free as
+  // soon as the activation fragments are in registers -- so no weight load ever waits for an MFMA.
+  auto phase_region = [&](int p) -> unsigned char* { return p < RPH ? myring + p * REGION : myx + (p - RPH) * REGION; };
   auto issue_phase = [&](int p) {
     const unsigned char* sb = wbase + p * 1536;            // the six wavefronts' pieces of a full phase: 6 x 256 bytes of every row
 #pragma unroll
@@ -244,81 +254,36 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if constexpr (NPH > RPH) issue_phase(NPH - 1);
   } else {
-    // Columns 8..15 of the MFMA are never stored, so lanes m >= 8 are free to do half of the norm's arithmetic: a
-    // lane fetches and scales the fragments of the steps of its own parity (h = bit 3 of the lane), and the lanes
-    // m < 8 then take the other parity's from their partner 8 lanes up (one DPP move per register).
-    const int h = (lane >> 3) & 1;
-    typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
-    bf16x8 own[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int sj = 2 * j + h;
-      own[j] = xfrag(sj < STEPS ? sj : STEPS - 2);            // (h = 1, j = 7) has no step: re-reads step 13, masked below
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the activation blocks are free from here on
-    if constexpr (EMB) {
-      if (!xok_m1) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-#pragma unroll
-          for (int q = 0; q < 8; ++q) own[j][q] = static_cast<bf16>(0.f);
-        }
-      }
-      if (blockIdx.x == 0 && m1 < nvalid) {                 // the gathered rows, as the residual stream: every lane its own fragments
-        bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + (row0 + m1) * 360;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (2 * j + h < STEPS) xo[kb(4 * (2 * j + h) + g) >> 4] = own[j];
-        }
-      }
-    }
-    float ssq = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float part = 0.f;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float f = static_cast<float>(own[j][q]);
-        part = fmaf(f, f, part);
-      }
-      ssq += (j == 7 && h == 1) ? 0.f : part;
-    }
-    ssq += __shfl_xor(ssq, 8, 64);
-    ssq += __shfl_xor(ssq, 16, 64);
-    ssq += __shfl_xor(ssq, 32, 64);
-    // The six slices' sums meet through LDS, but not at a barrier: a wavefront publishes its eight sums, raises
-    // its flag and goes on to request the rest of its weight (where it may sit for a microsecond until the CU's
-    // queue takes the loads); only then does it wait for the other five flags, which by that time are long up.
-    if (lane < XR) s_part[wave * XR + lane] = ssq;          // lanes 0..7: row m1 == lane
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the loads in flight are none of its business
-    if (lane == 0) __hip_atomic_store(&s_flag[wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-#pragma unroll
-    for (int p = EARLY; p < NPH; ++p) issue_phase(p);
+    // The six slices' sums meet through LDS, but not at a barrier: a wavefront publishes its sums, raises its flag and
+    // goes on to request the rest of its weight (where it may sit for a microsecond until the CU's queue takes the
+    // loads); only then does it wait for the other five flags, which by that time are long up.
     // Every streaming wavefront raises its flag before it gets here and none returns early, so the flags are up
     // after a few polls. The wait is bounded all the same: a wavefront that has polled kFlagPollLimit times (tens of
     // milliseconds) records that in g_qkv_decode_wait_expired and carries on to the kernel's barriers and exit with
     // whatever sums it has -- a wrong result the host can see instead of a workgroup that never ends.
-    for (int polls = 0;; ++polls) {
-      const unsigned f = lane < NS ? __hip_atomic_load(&s_flag[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : 1u;
-      if (__all(f != 0u)) break;
-      if (polls >= kFlagPollLimit) {
-        if (lane == 0) g_qkv_decode_wait_expired = 1;
-        break;
+    auto publish_and_meet = [&](float ssq) {                // ssq: sum of squares of row `lane` of this slice, in lanes 0 .. XR - 1
+      if (lane < XR) s_part[wave * XR + lane] = ssq;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS only: the loads in flight are none of its business
+      if (lane == 0) __hip_atomic_store(&s_flag[wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+      for (int p = EARLY; p < NPH; ++p) issue_phase(p);
+      for (int polls = 0;; ++polls) {
+        const unsigned f = lane < NS ? __hip_atomic_load(&s_flag[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : 1u;
+        if (__all(f != 0u)) break;
+        if (polls >= kFlagPollLimit) {
+          if (lane == 0) g_qkv_decode_wait_expired = 1;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
       }
-      __builtin_amdgcn_s_sleep(2);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-#ifdef TLLM_R8_STAMPS
-    R8_STAMP(3);
-#endif
-    float ss = 0.f;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+      float ss = 0.f;
 #pragma unroll
-    for (int w = 0; w < NS; ++w) ss += s_part[w * XR + m1];
-    const float rinv = rsqrtf(ss * (1.0f / 2880.0f) + a.norm_eps);
+      for (int w = 0; w < NS; ++w) ss += s_part[w * XR + m1];
+      return rsqrtf(ss * (1.0f / 2880.0f) + a.norm_eps);
+    };
     const unsigned char* sc = scw + wave * 2048;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int sj = 2 * j + h < STEPS ? 2 * j + h : STEPS - 2;
+    auto scaled = [&](bf16x8 v, int sj, float rinv) {       // bf16(x * rinv * scale), fp32 arithmetic, one rounding
       f32x4 s_lo, s_hi;
       if constexpr (NORM == 1) {
         s_lo = *reinterpret_cast<const f32x4*>(sc + (4 * sj + g) * 32);
@@ -333,20 +298,101 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
       }
       bf16x8 t;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) t[q] = static_cast<bf16>(static_cast<float>(own[j][q]) * rinv * (q < 4 ? s_lo[q] : s_hi[q - 4]));
-      own[j] = t;
-    }
-    // lanes m < 8 (h = 0): even steps are their own, odd steps come from lane + 8; lanes m >= 8 end up with a mix
-    // that only feeds the unused columns
+      for (int q = 0; q < 8; ++q) t[q] = static_cast<bf16>(static_cast<float>(v[q]) * rinv * (q < 4 ? s_lo[q] : s_hi[q - 4]));
+      return t;
+    };
+    auto sumsq = [](bf16x8 v) {
+      float part = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      fb[2 * j] = own[j];
-      if (2 * j + 1 < STEPS) {
-        const u32x4 mine = __builtin_bit_cast(u32x4, own[j]);
-        u32x4 theirs;
+      for (int q = 0; q < 8; ++q) {
+        const float f = static_cast<float>(v[q]);
+        part = fmaf(f, f, part);
+      }
+      return part;
+    };
+    if constexpr (XR == 16) {
+      // all sixteen MFMA columns are real rows: every lane fetches and scales the fifteen fragments of its own row
 #pragma unroll
-        for (int q = 0; q < 4; ++q) theirs[q] = __builtin_amdgcn_update_dpp(0u, mine[q], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
-        fb[2 * j + 1] = __builtin_bit_cast(bf16x8, theirs);
+      for (int s = 0; s < STEPS; ++s) fb[s] = xfrag(s);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the activation blocks are free from here on
+      if constexpr (EMB) {
+        if (!xok_m1) {
+#pragma unroll
+          for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) fb[s][q] = static_cast<bf16>(0.f);
+          }
+        }
+        if (blockIdx.x == 0 && m1 < nvalid) {               // the gathered rows, as the residual stream: every lane its own fragments
+          bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + (row0 + m1) * 360;
+#pragma unroll
+          for (int s = 0; s < STEPS; ++s) xo[kb(4 * s + g) >> 4] = fb[s];
+        }
+      }
+      float ssq = 0.f;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) ssq += sumsq(fb[s]);
+      ssq += __shfl_xor(ssq, 16, 64);
+      ssq += __shfl_xor(ssq, 32, 64);
+      const float rinv = publish_and_meet(ssq);             // lanes 0..15: row m1 == lane
+#ifdef TLLM_R8_STAMPS
+      R8_STAMP(3);
+#endif
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) fb[s] = scaled(fb[s], s, rinv);
+    } else {
+      // Columns 8..15 of the MFMA are never stored, so lanes m >= 8 are free to do half of the norm's arithmetic: a
+      // lane fetches and scales the fragments of the steps of its own parity (h = bit 3 of the lane), and the lanes
+      // m < 8 then take the other parity's from their partner 8 lanes up (one DPP move per register).
+      const int h = (lane >> 3) & 1;
+      typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+      bf16x8 own[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int sj = 2 * j + h;
+        own[j] = xfrag(sj < STEPS ? sj : STEPS - 2);          // (h = 1, j = 7) has no step: re-reads step 13, masked below
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the activation blocks are free from here on
+      if constexpr (EMB) {
+        if (!xok_m1) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) own[j][q] = static_cast<bf16>(0.f);
+          }
+        }
+        if (blockIdx.x == 0 && m1 < nvalid) {               // the gathered rows, as the residual stream: every lane its own fragments
+          bf16x8* xo = reinterpret_cast<bf16x8*>(a.emb_out) + (row0 + m1) * 360;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            if (2 * j + h < STEPS) xo[kb(4 * (2 * j + h) + g) >> 4] = own[j];
+          }
+        }
+      }
+      float ssq = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ssq += (j == 7 && h == 1) ? 0.f : sumsq(own[j]);
+      ssq += __shfl_xor(ssq, 8, 64);
+      ssq += __shfl_xor(ssq, 16, 64);
+      ssq += __shfl_xor(ssq, 32, 64);
+      const float rinv = publish_and_meet(ssq);             // lanes 0..7: row m1 == lane
+#ifdef TLLM_R8_STAMPS
+      R8_STAMP(3);
+#endif
+#pragma unroll
+      for (int j = 0; j < 8; ++j) own[j] = scaled(own[j], 2 * j + h < STEPS ? 2 * j + h : STEPS - 2, rinv);
+      // lanes m < 8 (h = 0): even steps are their own, odd steps come from lane + 8; lanes m >= 8 end up with a mix
+      // that only feeds the unused columns
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        fb[2 * j] = own[j];
+        if (2 * j + 1 < STEPS) {
+          const u32x4 mine = __builtin_bit_cast(u32x4, own[j]);
+          u32x4 theirs;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) theirs[q] = __builtin_amdgcn_update_dpp(0u, mine[q], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+          fb[2 * j + 1] = __builtin_bit_cast(bf16x8, theirs);
+        }
       }
     }
 #ifdef TLLM_R8_STAMPS
@@ -394,27 +440,35 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
     }
   }
 
-  // ---- partial tiles -> LDS (the wavefront's own region 1, long since consumed), then the epilogue wavefronts take over
-  *reinterpret_cast<f32x4*>(myring + REGION + lane * 16) = acc0;
-  *reinterpret_cast<f32x4*>(myring + REGION + 1024 + lane * 16) = acc1;
+  // ---- partial tiles -> LDS (a ring region of the wavefront's own, long since consumed), then the epilogue wavefronts take over
+  unsigned char* part = myring + (RING > 1 ? REGION : 0);
+  *reinterpret_cast<f32x4*>(part + lane * 16) = acc0;
+  *reinterpret_cast<f32x4*>(part + 1024 + lane * 16) = acc1;
   R8_STAMP(5);
   __syncthreads();
 }
 
-// Host side: pick the instantiation. norm = 0 / 1 (fp32 scale) / 2 (bf16 scale); w8: fp8 weight with a.w_scale.
-void launch_qkv_decode_r8(int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
+// Host side: pick the instantiation. xr = 8 or 16 rows per workgroup (16: fused norm only); norm = 0 / 1 (fp32 scale) / 2
+// (bf16 scale); w8: fp8 weight with a.w_scale.
+void launch_qkv_decode_r8(int xr, int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr) {
   const int out4 = qkv_outputs_allow_4_byte_stores(a);
-#define TLLM_R8(NORM, EMBF)                                                                                               \
-  do {                                                                                                                    \
-    if (w8) hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF, true>), grid, dim3(512), 0, st, a, ra, fr, out4);        \
-    else hipLaunchKernelGGL((qkv_decode_r8_kernel<NORM, EMBF, false>), grid, dim3(512), 0, st, a, ra, fr, out4);          \
+#define TLLM_R8(XRR, NORM, EMBF)                                                                                             \
+  do {                                                                                                                       \
+    if (w8) hipLaunchKernelGGL((qkv_decode_r8_kernel<XRR, NORM, EMBF, true>), grid, dim3(512), 0, st, a, ra, fr, out4);      \
+    else hipLaunchKernelGGL((qkv_decode_r8_kernel<XRR, NORM, EMBF, false>), grid, dim3(512), 0, st, a, ra, fr, out4);        \
   } while (0)
-  if (emb) {
-    if (norm == 1) TLLM_R8(1, true);
-    else TLLM_R8(2, true);
-  } else if (norm == 0) TLLM_R8(0, false);
-  else if (norm == 1) TLLM_R8(1, false);
-  else TLLM_R8(2, false);
+  if (xr == 16) {
+    if (emb) {
+      if (norm == 1) TLLM_R8(16, 1, true);
+      else TLLM_R8(16, 2, true);
+    } else if (norm == 1) TLLM_R8(16, 1, false);
+    else TLLM_R8(16, 2, false);
+  } else if (emb) {
+    if (norm == 1) TLLM_R8(8, 1, true);
+    else TLLM_R8(8, 2, true);
+  } else if (norm == 0) TLLM_R8(8, 0, false);
+  else if (norm == 1) TLLM_R8(8, 1, false);
+  else TLLM_R8(8, 2, false);
 #undef TLLM_R8
 }
 
