@@ -466,6 +466,16 @@ def main() -> int:
                                                                            yarn=yarn, positions=pr, mode="decode", out=qo,
                                                                            norm_scale=scales[i % N_LAYERS]),
                          bytes_of["norm_qkv"](r), n=240)
+        # batches beyond 32 rows: the weight held, the rows streamed past it (one pass over the weight whatever the row count)
+        for r in (96, 192):
+            xr = torch.randn(r, HIDDEN, generator=g).bfloat16().to(dev)
+            pr = torch.randint(0, 8192, (r,), generator=g, dtype=torch.int64).to(dev)
+            qo = (torch.empty(r, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev),
+                  torch.empty(r, NKV * HD, dtype=torch.bfloat16, device=dev))
+            bench_kernel(f"qkv_rope_decode_B{r}",
+                         lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
+                                                                           yarn=yarn, positions=pr, mode="decode", out=qo),
+                         bytes_of["qkv"](r), n=96)
         # the first layer of a token step: the gather rides in the same launch (embedding_B8 + norm_qkv_rope_decode_B8 in one)
         qo = (torch.empty(B, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev),
               torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev))

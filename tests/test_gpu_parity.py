@@ -255,14 +255,16 @@ def _check_qkv(gpu, yarn, rows, mode, seed, prefill_positions=False, max_pos=819
     close(v, vr)
 
 
-@pytest.mark.parametrize("rows", [1, 8, 15, 16, 17, 32, 50, 100, 192])
+@pytest.mark.parametrize("rows", [1, 8, 15, 16, 17, 32, 33, 50, 64, 65, 96, 100, 192, 450])
 def test_qkv_rope_decode_parity(gpu, yarn, rows):
+    """Up to 8 / 32 rows the two streaming kernels; from 33 rows the kernel that holds the weight and streams the rows
+    past it (33: a one-row last block; 64 / 65 and 96: whole and ragged blocks; 450: more blocks than ring slots)."""
     _check_qkv(gpu, yarn, rows, "decode", seed=rows)
 
 
-@pytest.mark.parametrize("rows", [64, 65, 192, 193])
+@pytest.mark.parametrize("rows", [64, 65, 448, 449])
 def test_qkv_rope_auto_mode_either_side_of_the_row_threshold(gpu, yarn, rows):
-    """``mode="auto"``: the weight-streaming kernel up to 192 rows at the gpt-oss shape, the MFMA GEMM above."""
+    """``mode="auto"``: the weight-streaming kernels up to 448 rows at the gpt-oss shape, the MFMA GEMM above."""
     _check_qkv(gpu, yarn, rows, "auto", seed=40 + rows)
 
 
@@ -488,6 +490,34 @@ def test_streaming_decode_kernels_every_row_count(gpu, yarn, rows):
         T.out_residual_decode_forward(nan_ox, weight, ob, torch.zeros(full, 1, 2880, dtype=torch.bfloat16, device=gpu), weight_scale=wscale)
         out = T.out_residual_decode_forward(oxbuf[:rows].view(rows, 1, 4096), weight, ob, o["r"].view(rows, 1, 2880).to(gpu), weight_scale=wscale)
         close(out.view(rows, 2880), O.out_residual_ref(o["x"], wref, o["b"], o["r"]))
+
+
+@pytest.mark.parametrize("rows", [33, 47, 81])
+def test_rows_streaming_kernel_ragged_last_block(gpu, yarn, rows):
+    """Above 32 rows one kernel holds the weight and streams the activations past it in blocks of 16 rows; the last
+    block re-reads the last row instead of reading past it. The memory behind the last row is NaN, the launch before
+    ran on NaN activations (whatever it left in LDS would show), bf16 and fp8 weight, and the norm composed in front."""
+    d = O.make_inputs(rows, seed=1300 + rows)
+    w, b = d["w"].to(gpu), d["b"].to(gpu)
+    w8, ws = T.quantize_fp8_rows(w)
+    xbuf = torch.full((rows + 16, 2880), float("nan"), dtype=torch.bfloat16, device=gpu)
+    xbuf[:rows] = d["x"].to(gpu)
+    x, pos = xbuf[:rows], d["positions"].to(gpu)
+    nan_x = torch.full((96, 2880), float("nan"), dtype=torch.bfloat16, device=gpu)
+    nan_pos = torch.zeros(96, dtype=torch.int64, device=gpu)
+    for weight, wscale, wref in ((w, None, d["w"]), (w8, ws, O.dequant_fp8_ref(w8.cpu(), ws.cpu()))):
+        kw = dict(weight_scale=wscale) if wscale is not None else {}
+        T.qkv_rope_forward(nan_x, weight, b, 64, 8, 64, yarn=yarn, positions=nan_pos, mode="decode", **kw)
+        q, k, v = T.qkv_rope_forward(x, weight, b, 64, 8, 64, yarn=yarn, positions=pos, mode="decode", **kw)
+        qr, kr, vr = O.qkv_rope_ref(d["x"], wref, d["b"], d["positions"])
+        close(q, qr)
+        close(k, kr)
+        close(v, vr)
+    q, k, v = T.qkv_rope_forward(x, w, b, 64, 8, 64, yarn=yarn, positions=pos, mode="decode", norm_scale=d["norm_scale"].to(gpu), norm_eps=1e-5)
+    qr, kr, vr = O.qkv_rope_ref(O.rmsnorm_ref(d["x"], d["norm_scale"].float(), 1e-5).bfloat16(), d["w"], d["b"], d["positions"])
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
 
 
 def test_fused_norm_wait_for_the_other_wavefronts_never_expires(gpu, yarn):

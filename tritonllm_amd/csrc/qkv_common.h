@@ -55,6 +55,8 @@ int qkv_validate(const char* who, const void* x, const void* W, const void* q, c
 void launch_qkv_decode_r8(int xr, int norm, bool emb, bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 // ... and for 9..32 rows per workgroup, bf16 or fp8 weight, activations already normalised (qkv_decode_r32.hip).
 void launch_qkv_decode_r32(bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
+// ... and for any number of rows in one pass over the weight, activations already normalised (qkv_decode_rows.hip).
+void launch_qkv_decode_rows(bool w8, dim3 grid, hipStream_t st, const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& fr);
 
 // Any hidden size, any even head_dim: one workgroup per (head, row); each wavefront takes
 // rotation pairs (d, d + hd/2) in turn and reduces the two dot products by shuffle.

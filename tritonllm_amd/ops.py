@@ -35,9 +35,10 @@ _BF16 = torch.bfloat16
 
 # rows at or below this use the weight-streaming decode kernel, above it the MFMA GEMM
 DECODE_MAX_ROWS = 64
-# At the gpt-oss shape the streaming kernel takes 32 rows per pass over the weight, ~7.5 us a pass (96 rows 23 us, 128
-# rows 30 us), where the GEMM's one round of tiles costs 48-56 us however few rows there are: they meet near 224 rows.
-DECODE_MAX_ROWS_2880 = 192
+# At the gpt-oss shape the weight is read once whatever the row count (above 32 rows a kernel holds its share of the
+# weight and streams the rows past it: ~6.5 us + 0.09 us per row -- 96 rows 16 us, 192 rows 24 us, 384 rows 38-42 us),
+# where the GEMM's one round of tiles costs 50-56 us however few rows there are: they meet near 500 rows.
+DECODE_MAX_ROWS_2880 = 448
 
 
 def _decode_max_rows(hidden: int, head_dim: int) -> int:
