@@ -262,6 +262,22 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         mo = torch.empty(n, 2 * HIDDEN, HIDDEN, dtype=torch.bfloat16, device=dev)
         fn = lambda i: T.mxfp4_dequant(mb, ms, out=mo)
         nbytes = bytes_of["mxfp4"](ms.numel())
+    elif kind == "stack24":
+        # stack24_B<n>: token steps of the 24-layer per-token stack (configs[4]), four steps per graph replay
+        from tritonllm_amd.stack import LayerKernelStack
+        mlp_scales = [(1 + 0.1 * torch.randn(HIDDEN, generator=g)).bfloat16().to(dev) for _ in range(N_LAYERS + 1)]
+        xr = torch.randn(n, HIDDEN, generator=g).bfloat16().to(dev)
+        pr = torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
+        sx = (2.0 * torch.randn(4 * n, 2 * HIDDEN, generator=g)).bfloat16().to(dev)
+        st = LayerKernelStack(weights, biases, scales, mlp_scales[:N_LAYERS], mlp_scales[N_LAYERS], yarn, n, fuse_norm=not args.unfused)
+        fn = lambda i: st.token_step(xr, pr, sx)
+        fn(0)
+        gr = graph_of(fn, 4)
+        for _ in range(max(args.steps // 40, 6)):
+            gr.replay()
+        sec = min(time_graph(gr) for _ in range(5)) / 4
+        print(json.dumps({"kernel": name, "us_per_token_step": round(sec * 1e6, 2), "launches": st.launches_per_step()}))
+        return 0
     else:
         print(f"bench.py: unknown --only target {name}", file=sys.stderr)
         return 2
@@ -295,7 +311,7 @@ def main() -> int:
     ap.add_argument("--no-kernel-table", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="seconds of CPU work per CPU-baseline leg (all cores, one thread)")
     ap.add_argument("--only", default=None,
-                    help="run just one entry of the kernel table (e.g. qkv_rope_prefill_T2048) and print its row; for profiling")
+                    help="run just one entry of the kernel table (e.g. qkv_rope_prefill_T2048), or stack24_B<n>, and print its row; for profiling")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a rocprofv3 --pmc run of this command "
                          "holds a dispatch of known traffic to scale FETCH_SIZE / WRITE_SIZE by")

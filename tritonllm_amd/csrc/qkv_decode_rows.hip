@@ -41,6 +41,12 @@ __global__ __launch_bounds__(512) void qkv_decode_rows_kernel(QkvArgs a, RopeArg
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  {
+    // the kernel arguments the first loads need, fetched in one go with the others
+    const void* p0 = a.x;
+    const void* p1 = a.W;
+    asm volatile("" ::"s"(p0), "s"(p1));
+  }
   const int total_pairs = (a.n_q_heads + 2 * a.n_kv_heads) * 32;
   const int pair0 = blockIdx.x * PAIRS;
   const int nblk = static_cast<int>((a.rows + XB - 1) / XB);
