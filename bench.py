@@ -30,10 +30,10 @@ if ROOT not in sys.path:
 
 # HBM bytes per launch of the decode QKV kernel at B=8, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch), FETCH_SIZE scaled by the 2.000 a 256 MiB copy of known size reads on the same counter:
-# 14708.6 x 2.000 + 192.0 KiB with the fused norm, 14662.0 x 2.000 + 192.0 KiB without.
+# 14707.1 x 2.000 + 192.0 KiB with the fused norm, 14659.8 x 2.000 + 192.0 KiB without.
 # Summary and commands: profiles/qkv_decode_r8_kernel_B8_decode_step.md. Not re-measured by this script: when the
 # kernel changes, the profile has to be taken again.
-QKV_DECODE_TRAFFIC_BYTES = {"fused": int((14708.6 * 2.000 + 192.0) * 1024), "unfused": int((14662.0 * 2.000 + 192.0) * 1024)}
+QKV_DECODE_TRAFFIC_BYTES = {"fused": int((14707.1 * 2.000 + 192.0) * 1024), "unfused": int((14659.8 * 2.000 + 192.0) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published (no sparsity)
 
