@@ -523,7 +523,7 @@ def main() -> int:
         ow = [torch.empty(HIDDEN, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
         ow8 = [T.quantize_fp8_rows(w) for w in ow]
         ob = torch.empty(HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
-        for r in (1, 8, 32):
+        for r in (1, 8, 16, 32):
             ox = torch.empty(r, 1, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
             ores = torch.zeros(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev)
             bench_kernel(f"out_residual_decode_B{r}", lambda i, ox=ox, ores=ores: T.out_residual_decode_forward(ox, ow[i % N_LAYERS], ob, ores),

@@ -775,7 +775,7 @@ def _out_inputs(rows, seed, in_dim=4096, out_dim=2880):
                 b=(0.02 * torch.randn(out_dim, generator=g)).bfloat16(), r=torch.randn(rows, out_dim, generator=g).bfloat16())
 
 
-@pytest.mark.parametrize("rows", [1, 8, 11, 16, 17, 32, 45])
+@pytest.mark.parametrize("rows", [1, 8, 9, 11, 12, 13, 16, 17, 20, 21, 24, 25, 28, 29, 32, 33, 45, 64, 70])
 @pytest.mark.parametrize("fp8", [False, True])
 def test_out_residual_decode_parity(gpu, rows, fp8):
     d = _out_inputs(rows, 600 + rows)
@@ -793,7 +793,7 @@ def test_out_residual_decode_parity(gpu, rows, fp8):
     close(out.view(rows, 2880), want)
 
 
-@pytest.mark.parametrize("rows", [1, 5, 8])
+@pytest.mark.parametrize("rows", [1, 5, 8, 13, 32, 37])
 def test_out_residual_decode_strides_alignment_and_absent_operands(gpu, rows):
     """The C entry point with what the host wrapper never passes: a separate output buffer, row strides that rule
     out 8-byte accesses (2882) and ones that allow them (2884), an output that starts 2 bytes off an 8-byte boundary,

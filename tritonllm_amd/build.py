@@ -18,7 +18,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtllm_hip.so")
 INCLUDE = os.path.join(ROOT, "include")
 
-SOURCES = ["abi.hip", "rmsnorm.hip", "embedding.hip", "swiglu.hip", "rope.hip", "qkv_decode.hip", "qkv_decode_r8.hip", "qkv_decode_r32.hip", "qkv_decode_rows.hip", "qkv_prefill.hip", "out_decode.hip", "out_decode_r8.hip", "unembed.hip", "attn_decode.hip", "attn_prefill.hip", "mxfp4.hip"]
+SOURCES = ["abi.hip", "rmsnorm.hip", "embedding.hip", "swiglu.hip", "rope.hip", "qkv_decode.hip", "qkv_decode_r8.hip", "qkv_decode_r32.hip", "qkv_decode_rows.hip", "qkv_prefill.hip", "out_decode.hip", "out_decode_r8.hip", "out_decode_r32.hip", "unembed.hip", "attn_decode.hip", "attn_prefill.hip", "mxfp4.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 from ordinary float code.
 HIPCC_FLAGS = [

@@ -1,4 +1,4 @@
-// Argument block shared by the decode out-projection kernels (out_decode.hip, out_decode_r8.hip).
+// Argument block shared by the decode out-projection kernels (out_decode.hip, out_decode_r8.hip, out_decode_r32.hip).
 #pragma once
 #include "common.h"
 
@@ -18,5 +18,8 @@ struct OutArgs {
 
 // in_dim 4096, out_dim % 12 == 0, rows <= 8, bf16 weight or (a.w_scale != null) fp8; grid = (out_dim / 12)
 void launch_out_decode_r8(dim3 grid, hipStream_t st, const OutArgs& a);
+
+// in_dim 4096, out_dim % 12 == 0, bf16 weight, any number of rows in chunks of 32; grid = (out_dim / 12, ceil(rows / 32))
+void launch_out_decode_r32(dim3 grid, hipStream_t st, const OutArgs& a);
 
 }  // namespace tllm

@@ -3,7 +3,8 @@
 // One launch, no partial-sum workspace; `out` may be the residual buffer itself, as in the reference.
 //
 //   out_decode_r8_kernel    (out_decode_r8.hip) in_dim == 4096, out_dim % 12 == 0, up to 8 rows, bf16 or fp8 weight
-//   out_decode_cu_kernel    in_dim == 4096, out_dim % 12 == 0 (gpt-oss: [2880, 4096]), more rows: the weight-streaming layout
+//   out_decode_r32_kernel   (out_decode_r32.hip) the same shape, more rows in chunks of 32, bf16 weight
+//   out_decode_cu_kernel    in_dim == 4096, out_dim % 12 == 0 (gpt-oss: [2880, 4096]), more rows, fp8 weight: the weight-streaming layout
 //                           of the decode QKV kernel -- one workgroup per CU-sized share of the output features,
 //                           sixteen wavefronts splitting K, every load unconditional and issued up front, operands
 //                           through wavefront-private LDS patches into v_mfma_f32_32x32x16_bf16, one reduction.
@@ -221,6 +222,10 @@ extern "C" int tllm_out_residual_decode_bf16(const void* x, const void* W, const
     dim3 grid((unsigned)(out_dim / 12), (unsigned)chunks);
     if (rows <= 8) {
       launch_out_decode_r8(grid, st, a);
+      return check_launch("out_residual_decode");
+    }
+    if (!w8) {
+      launch_out_decode_r32(dim3((unsigned)(out_dim / 12), (unsigned)((rows + 31) / 32)), st, a);
       return check_launch("out_residual_decode");
     }
 #define TLLM_OUT(XR, CH)                                                                                   \

@@ -1,0 +1,208 @@
+// Decode-size attention out-projection + bias + residual for in_dim == 4096 and 9..32 activation rows per workgroup
+// (bf16 weight): the companion of out_decode_r8.hip for the larger decode batches
+//   out[r, n] = sum_k x[r, k] * W[n, k] + b[n] + res[r, n]        (out_residual_decode_forward, triton_kernels.py:1470-1517)
+//
+// Same skeleton: one workgroup per twelve output features (gpt-oss: 240 workgroups, one per CU), one 16-row MFMA tile
+// of weight rows on M against two column blocks of 16 activation rows on N (v_mfma_f32_16x16x32_bf16), every operand
+// loaded from global memory straight into LDS with the XOR swizzle chosen on the global side, fragments read back
+// once, partial tiles reduced in a fixed order by epilogue wavefronts that fetched bias and residual meanwhile.
+// What differs: 32 activation rows are 256 KB per workgroup, more than the LDS holds, so the activations arrive in
+// phases with the weight. Four streaming wavefronts, each with 1024 of the 4096 K: 32 k32 steps in eight phases of
+// four; in phase p the four together read 1024 contiguous bytes of every row (wavefront kq the 256 bytes at
+// p * 1024 + kq * 256). A phase of a wavefront is 8 KB of activations (32 rows x 256 bytes) and 3 KB of weight,
+// through a ring of three 11 KB regions: three phases are in flight, a phase is multiplied as soon as it has landed
+// and its region is then refilled with the phase three further on (a ring of two measures 1 % slower: the depth is
+// not what bounds the kernel, a CU takes in its 352 KB at 63 GB/s). Two epilogue wavefronts, one per column block.
+// XB = four-row activation blocks fetched per phase (rows past a chunk's last one repeat it; with fewer than 29 rows
+// the blocks that would hold no real row are not fetched at all).
+#include "out_common.h"
+
+namespace tllm {
+
+namespace r32o {
+constexpr int XR = 32;            // activation rows per workgroup
+constexpr int NS = 4;             // streaming wavefronts = K slices
+constexpr int NE = 2;             // epilogue wavefronts = column blocks
+constexpr int RW = 12;            // weight rows (output features) per workgroup
+constexpr int NPH = 8;            // phases of four k32 steps
+constexpr int RING = 3;           // resident phases per wavefront
+constexpr int XPH = 8 * 1024;     // activations of one phase: 32 rows x four k32 steps
+constexpr int WPH = 3 * 1024;     // weight of one phase: 12 rows x four k32 steps
+constexpr int REGION = XPH + WPH;
+}  // namespace r32o
+
+template <int XB>
+__global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8) {
+  using namespace r32o;
+  constexpr int LPP = XB + 3;                               // load instructions per phase
+  __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * RW;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
+  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+
+  if (wave >= NS) {
+    // ======================================================================= epilogue wavefront of column block cb
+    const int cb = wave - NS;
+    const int en = 16 * cb + (lane & 15), eg = lane >> 4;   // activation row of the chunk, quad of features
+    const bool evalid = eg < 3 && en < nvalid;
+    const int efeat = n0 + (evalid ? 4 * eg : 0);
+    const int64_t erow = row0 + (evalid ? en : 0);
+    // absent operands read a valid dummy address instead of being predicated
+    const bf16* bias_ptr = a.bias ? a.bias + efeat : a.x;
+    const bf16* res_ptr = a.res ? a.res + erow * a.res_rs + efeat : a.x;
+    bf16* out = a.out + erow * a.out_rs + efeat;
+    float bv[4], rv[4];
+    if (vec8) {
+      const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bias_ptr);
+      const bf16x4 r4 = *reinterpret_cast<const bf16x4*>(res_ptr);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        bv[i] = static_cast<float>(b4[i]);
+        rv[i] = static_cast<float>(r4[i]);
+      }
+    } else {
+      bf16 b1[4], r1[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        b1[i] = bias_ptr[i];
+        r1[i] = res_ptr[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        bv[i] = static_cast<float>(b1[i]);
+        rv[i] = static_cast<float>(r1[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (!a.bias) bv[i] = 0.f;
+      if (!a.res) rv[i] = 0.f;
+    }
+    unsigned red_o = static_cast<unsigned>(cb * 1024 + lane * 16);
+    // the wavefronts run alone from the barrier to the stores: everything that does not need the sums exists before it
+    asm volatile("" : "+v"(bv[0]), "+v"(bv[1]), "+v"(bv[2]), "+v"(bv[3]), "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]), "+v"(out), "+v"(red_o));
+    __syncthreads();                                        // partial tiles are in LDS
+    f32x4 t[NS];
+#pragma unroll
+    for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(ring + w * (RING * REGION) + red_o);
+    f32x4 acc = t[0];
+#pragma unroll
+    for (int w = 1; w < NS; ++w) {                          // fixed order: the result does not depend on timing
+      acc[0] += t[w][0];
+      acc[1] += t[w][1];
+      acc[2] += t[w][2];
+      acc[3] += t[w][3];
+    }
+    if (!evalid) return;
+    bf16x4 o;                                               // features efeat .. efeat + 3 of row en
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] + bv[i] + rv[i]);
+    if (vec8) {
+      *reinterpret_cast<bf16x4*>(out) = o;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[i] = o[i];
+    }
+    return;
+  }
+
+  // ========================================================================= streaming wavefront of K slice `kq`
+  const int kq = wave;
+  const int m = lane & 15, g = lane >> 4;
+  unsigned char* myring = ring + wave * (RING * REGION);
+
+  // lane -> (row of a 4-row block, position): it fetches chunk position ^ (row & 15) of that row's 256 bytes, so that
+  // the 16 rows a fragment read touches lie in 16 different bank groups
+  unsigned xoff[XB], goff[3];
+#pragma unroll
+  for (int j = 0; j < XB; ++j) {
+    const int r = 4 * j + (lane >> 4);
+    const int src = r < nvalid ? r : nvalid - 1;            // row inside the workgroup's 32 (the base below points at row0)
+    xoff[j] = static_cast<unsigned>(src * 8192 + kq * 256 + (((lane & 15) ^ (r & 15)) << 4));
+  }
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int r = 4 * j + (lane >> 4);
+    goff[j] = static_cast<unsigned>(n0 + r) * 8192u + kq * 256u + (((lane & 15) ^ r) << 4);
+  }
+  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x) + row0 * 8192;
+  const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
+  auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
+  auto issue_phase = [&](int p) {                           // the activations of the phase, then its weight
+    unsigned char* reg = myring + (p % RING) * REGION;
+    const unsigned char* xb = xbase + p * 1024;
+    const unsigned char* wb = wbase + p * 1024;
+#pragma unroll
+    for (int j = 0; j < XB; ++j) {
+      const unsigned dst = lds_addr(reg + j * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[j]), "s"(xb) : "memory", "m0");
+    }
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      const unsigned dst = lds_addr(reg + XPH + j * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff[j]), "s"(wb) : "memory", "m0");
+    }
+  };
+#pragma unroll
+  for (int p = 0; p < RING; ++p) issue_phase(p);
+
+  f32x4 acc[2];                                             // [column block]
+  acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int arow = m < RW ? m : m - RW;                     // tile rows past the twelfth re-read a real one (their sums are dropped)
+  const unsigned a_o = XPH + arow * 256;
+  const unsigned b0_o = m * 256, b1_o = (16 + m) * 256;
+#pragma unroll
+  for (int p = 0; p < NPH; ++p) {
+    // phase p has landed when only the loads of the phases after it that have been requested are outstanding
+    constexpr int kTwo = 2 * LPP, kOne = LPP;
+    if (p < NPH - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kTwo) : "memory");
+    else if (p == NPH - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kOne) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned char* reg = myring + (p % RING) * REGION;
+    bf16x8 fa[4], fb0[4], fb1[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      fa[st] = *reinterpret_cast<const bf16x8*>(reg + a_o + (((4 * st + g) ^ arow) << 4));
+      fb0[st] = *reinterpret_cast<const bf16x8*>(reg + b0_o + (((4 * st + g) ^ m) << 4));
+      if constexpr (XB > 4) fb1[st] = *reinterpret_cast<const bf16x8*>(reg + b1_o + (((4 * st + g) ^ m) << 4));
+    }
+    if (p + RING < NPH) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the region's fragments are in registers: it may be refilled
+      issue_phase(p + RING);
+    }
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[st], fb0[st], acc[0], 0, 0, 0);
+      if constexpr (XB > 4) acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[st], fb1[st], acc[1], 0, 0, 0);
+    }
+  }
+
+  // ---- partial tiles -> LDS (the wavefront's own region 0: every region's fragments have been read by now)
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  *reinterpret_cast<f32x4*>(myring + lane * 16) = acc[0];
+  *reinterpret_cast<f32x4*>(myring + 1024 + lane * 16) = acc[1];
+  __syncthreads();
+}
+
+// in_dim 4096, out_dim % 12 == 0, bf16 weight; grid = (out_dim / 12, ceil(rows / 32))
+void launch_out_decode_r32(dim3 grid, hipStream_t st, const OutArgs& a) {
+  auto al8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
+  const int vec8 = al8(a.out) && a.out_rs % 4 == 0 && (a.res == nullptr || (al8(a.res) && a.res_rs % 4 == 0)) && (a.bias == nullptr || al8(a.bias));
+  const int rows = static_cast<int>(a.rows < 32 ? a.rows : 32);          // of the fullest chunk
+  switch ((rows + 3) / 4) {
+    case 1: hipLaunchKernelGGL(out_decode_r32_kernel<1>, grid, dim3(384), 0, st, a, vec8); break;
+    case 2: hipLaunchKernelGGL(out_decode_r32_kernel<2>, grid, dim3(384), 0, st, a, vec8); break;
+    case 3: hipLaunchKernelGGL(out_decode_r32_kernel<3>, grid, dim3(384), 0, st, a, vec8); break;
+    case 4: hipLaunchKernelGGL(out_decode_r32_kernel<4>, grid, dim3(384), 0, st, a, vec8); break;
+    case 5: hipLaunchKernelGGL(out_decode_r32_kernel<5>, grid, dim3(384), 0, st, a, vec8); break;
+    case 6: hipLaunchKernelGGL(out_decode_r32_kernel<6>, grid, dim3(384), 0, st, a, vec8); break;
+    case 7: hipLaunchKernelGGL(out_decode_r32_kernel<7>, grid, dim3(384), 0, st, a, vec8); break;
+    default: hipLaunchKernelGGL(out_decode_r32_kernel<8>, grid, dim3(384), 0, st, a, vec8); break;
+  }
+}
+
+}  // namespace tllm
