@@ -879,6 +879,24 @@ def test_unembedding_decode_parity_small_vocab(gpu, rows, vocab, fp8):
     _argmax_ok(ids, want)
 
 
+@pytest.mark.parametrize("rows", [5, 11, 16, 19])
+@pytest.mark.parametrize("hidden", [64, 4096])
+def test_unembedding_other_hidden_sizes(gpu, rows, hidden):
+    """Hidden sizes other than gpt-oss's: above eight rows the kernel keeps sixteen activation rows in LDS where they
+    fit (2880 wide) and falls back to chunks of eight where they do not (4096 wide), logits and argmax alike."""
+    g = torch.Generator().manual_seed(880 + rows + hidden)
+    x = torch.randn(rows, hidden, generator=g).bfloat16()
+    w = (0.05 * torch.randn(3001, hidden, generator=g)).bfloat16()
+    xg = x.view(rows, 1, hidden).to(gpu)
+    want = O.linear_ref(x, w, None)
+    close(T.unembedding_decode_forward(xg, w.to(gpu)).view(rows, 3001), want)
+    _argmax_ok(T.unembedding_decode_argmax_forward(xg, w.to(gpu)), want)
+    w8, ws = T.quantize_fp8_rows(w.to(gpu))
+    want8 = O.linear_ref(x, O.dequant_fp8_ref(w8.cpu(), ws.cpu()), None)
+    close(T.unembedding_decode_fp8_forward(xg, w8, ws).view(rows, 3001), want8)
+    _argmax_ok(T.unembedding_decode_fp8_argmax_forward(xg, w8, ws), want8)
+
+
 def test_unembedding_full_vocabulary_and_module(gpu, monkeypatch):
     """The real size: [201088, 2880]. Logits against the oracle on a sample of columns (the full fp32 product on
     the CPU would take minutes), argmax against a planted winner, and the module's dispatch."""

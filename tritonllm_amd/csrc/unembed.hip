@@ -259,7 +259,7 @@ using namespace tllm;
 namespace {
 constexpr int kUnembedGrid = 256;      // one workgroup per CU
 
-int unembed_xr(int64_t rows) { return rows <= 8 ? 8 : 16; }
+int unembed_xr_most(int64_t rows) { return rows <= 8 ? 8 : 16; }
 
 // (wavefronts, K step, steps in flight), measured at B = 8 on the full vocabulary:
 //   bf16, up to 8 rows : 16 wavefronts, K step 64 (whole 128-byte lines), 4 in flight   185 us (8 wavefronts: 194)
@@ -272,15 +272,18 @@ size_t unembed_smem(int xr, bool w8, int64_t hidden) {
   return static_cast<size_t>(xr) * unembed_xrow((int)hidden) + unembed_nw(xr, w8) * unembed_patch(unembed_ks(xr, w8, hidden));
 }
 
-int unembed_xr(int64_t rows);
-size_t unembed_smem(int xr, bool w8, int64_t hidden);
+// Batch rows per workgroup: sixteen above eight rows where the LDS holds them (gpt-oss: 2880 wide), else chunks of eight
+// (each chunk streams the weight once more).
+int unembed_xr(int64_t rows, bool w8, int64_t hidden) {
+  return (rows > 8 && unembed_smem(16, w8, hidden) <= 160 * 1024) ? 16 : 8;
+}
 int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_t rows, int64_t hidden, int64_t vocab) {
   TLLM_REQUIRE(rows >= 0 && hidden >= 1 && vocab >= 1 && vocab < (1ll << 31) && hidden < (1ll << 24), TLLM_E_SHAPE,
                "%s: rows %lld, hidden %lld, vocab %lld", who, (long long)rows, (long long)hidden, (long long)vocab);
   if (rows == 0) return TLLM_OK;
   TLLM_REQUIRE(x && W, TLLM_E_ARG, "%s: x and W must not be NULL", who);
   TLLM_REQUIRE(hidden % 64 == 0, TLLM_E_SHAPE, "%s: hidden %lld must be a multiple of 64", who, (long long)hidden);
-  TLLM_REQUIRE(unembed_smem(unembed_xr(rows), w8, hidden) <= 160 * 1024, TLLM_E_SHAPE, "%s: hidden %lld too large for the LDS-resident activations", who,
+  TLLM_REQUIRE(unembed_smem(unembed_xr(rows, w8, hidden), w8, hidden) <= 160 * 1024, TLLM_E_SHAPE, "%s: hidden %lld too large for the LDS-resident activations", who,
                (long long)hidden);
   TLLM_REQUIRE(aligned16(x) && aligned16(W), TLLM_E_ALIGN, "%s: x and W must be 16-byte aligned", who);
   TLLM_REQUIRE((rows + 15) / 16 <= 65535, TLLM_E_SHAPE, "%s: rows %lld too many", who, (long long)rows);
@@ -289,7 +292,7 @@ int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_
 
 template <bool ARGMAX>
 int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t st) {
-  const int xr = unembed_xr(a.rows);
+  const int xr = unembed_xr(a.rows, w8, a.hidden);
   const size_t smem = unembed_smem(xr, w8, a.hidden);
   const dim3 grid(kUnembedGrid, (unsigned)((a.rows + xr - 1) / xr));
 #define TLLM_UNEMBED(XR, NW, KS, UD, W8F)                                                                                   \
@@ -328,9 +331,11 @@ extern "C" int tllm_unembedding_decode_bf16(const void* x, const void* W, const 
 
 extern "C" int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows) {
   if (rows <= 0) return 0;
-  const int xr = unembed_xr(rows);
+  const int xr = unembed_xr_most(rows);
   const int64_t chunks = (rows + xr - 1) / xr;
-  return chunks * kUnembedGrid * 16 * xr * 8;      // one (float, int) pair per wavefront (at most 16 per workgroup) and batch-row slot
+  // one (float, int) pair per wavefront (at most 16 per workgroup) and batch-row slot; chunks of eight rows, which a
+  // wide hidden size forces, never need more slots than chunks of sixteen
+  return chunks * kUnembedGrid * 16 * xr * 8;
 }
 
 // Both argmax entry points: the stream kernel leaves one candidate per wavefront and batch row in `workspace`, the
@@ -338,7 +343,7 @@ extern "C" int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows) {
 // call, so the workspace needs no clearing.
 static int unembed_argmax_run(const char* who, const void* x, const void* W, const float* w_scale, void* workspace, int64_t need,
                               int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
-  const int xr = unembed_xr(rows);
+  const int xr = unembed_xr(rows, w_scale != nullptr, hidden);
   UnembedArgs a{};
   a.x = (const bf16*)x;
   a.W = W;
