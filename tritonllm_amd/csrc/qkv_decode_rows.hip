@@ -59,17 +59,28 @@ __global__ __launch_bounds__(512) void qkv_decode_rows_kernel(QkvArgs a, RopeArg
   if (wave >= NS) {
     // ======================================================================= epilogue wavefront of tile `tile`
     const int tile = wave - NS;
+    const int eg = lane >> 4, en = lane & 15;               // quad of the tile, activation row of the block
+    // Between two barriers this wavefront is the workgroup's critical path (the streaming wavefronts need ~0.5 us per
+    // block), so nothing with a memory latency in it may sit there: what depends on the lane only is made once, the
+    // row's position is requested two blocks ahead, its cos / sin and output address are made one block ahead (before
+    // the barrier, while the streaming wavefronts multiply); between the barriers it sums, rotates and stores.
+    auto row0_of = [&](int b) { return static_cast<int64_t>(block_at(b < nblk ? b : nblk - 1)) * XB; };
+    auto nvalid_of = [&](int64_t row0) { return static_cast<int>(a.rows - row0 < XB ? a.rows - row0 : XB); };
+    StreamEpilogueLane<W8> ep;
+    ep.prepare(a, ra, fr, pair0, tile, eg, en, row0_of(0), nvalid_of(row0_of(0)));
+    int64_t pos_next = ep.request_row(a, ra, en, row0_of(1), nvalid_of(row0_of(1)));
     for (int b = 0; b < nblk; ++b) {
-      const int64_t row0 = static_cast<int64_t>(block_at(b)) * XB;
-      const int nvalid = static_cast<int>(a.rows - row0 < XB ? a.rows - row0 : XB);
-      StreamEpilogueLane<W8> ep;
-      ep.prepare(a, ra, fr, pair0, tile, lane >> 4, lane & 15, row0, nvalid);   // quad of the tile, activation row
+      const int64_t row1 = row0_of(b + 1), row2 = row0_of(b + 2);   // past the end: the last block again
+      StreamEpilogueLane<W8> next = ep;
+      next.prepare_row(a, ra, fr, pos_next, en, row1, nvalid_of(row1));
       unsigned red_o = static_cast<unsigned>((b & 1) * (NS * PART) + tile * 1024 + lane * 16);
       asm volatile("" : "+v"(red_o));
       asm volatile("s_barrier" ::: "memory");               // the partial tiles of block b are in LDS
       f32x4 t[NS];
 #pragma unroll
       for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(part + w * PART + red_o);
+      // requested before this block's stores go out: the wait for it, one round on, then does not wait for them
+      const int64_t pos_after = ep.request_row(a, ra, en, row2, nvalid_of(row2));
       f32x4 acc = t[0];
 #pragma unroll
       for (int w = 1; w < NS; ++w) {                        // fixed order: the result does not depend on timing
@@ -79,6 +90,8 @@ __global__ __launch_bounds__(512) void qkv_decode_rows_kernel(QkvArgs a, RopeArg
         acc[3] += t[w][3];
       }
       ep.finish(acc, out4);
+      ep = next;
+      pos_next = pos_after;
     }
     return;
   }
