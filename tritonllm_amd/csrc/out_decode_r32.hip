@@ -12,7 +12,7 @@
 // p * 1024 + kq * 256). A phase of a wavefront is 8 KB of activations (32 rows x 256 bytes) and 3 KB of weight,
 // through a ring of three 11 KB regions: three phases are in flight, a phase is multiplied as soon as it has landed
 // and its region is then refilled with the phase three further on (a ring of two measures 1 % slower: the depth is
-// not what bounds the kernel, a CU takes in its 352 KB at 63 GB/s). Two epilogue wavefronts, one per column block.
+// not what bounds the kernel). Two epilogue wavefronts, one per column block.
 // XB = four-row activation blocks fetched per phase (rows past a chunk's last one repeat it; with fewer than 29 rows
 // the blocks that would hold no real row are not fetched at all).
 #include "out_common.h"

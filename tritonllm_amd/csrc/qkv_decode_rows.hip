@@ -12,9 +12,9 @@
 // are in flight while one is multiplied. After a block's last unit the wavefronts park their partial tiles in one of
 // two buffers and meet the epilogue wavefronts at a barrier; those finish the block (sum, bias, rotation, one
 // rounding, stores) while the next block is multiplied.
-// Per CU: 115 KB of weight from HBM once, and rows x 5760 bytes of activations from the L2s -- the latter is what
-// bounds the kernel from a few dozen rows up (a CU is served 60-80 GB/s), and why the prefill GEMM, which shares
-// activation tiles between fewer CUs, takes over at a few hundred rows.
+// Per CU: 115 KB of weight from HBM once, and rows x 5760 bytes of activations from the L2s. A block of 16 rows costs
+// ~1.4 us, most of it the streaming wavefronts' own chain (wait, fragment reads, dependent MFMAs, barrier) rather than
+// the bytes; the prefill GEMM, whose tiles share activations between fewer CUs, takes over at a few hundred rows.
 // W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (triton_kernels.py:261-268, 927-965): the
 // fragments are widened to bf16 (exact) once, on their way into the registers; the row scale multiplies the finished sum.
 #include "qkv_decode_stream.h"
