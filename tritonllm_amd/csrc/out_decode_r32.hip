@@ -1,5 +1,5 @@
 // Decode-size attention out-projection + bias + residual for in_dim == 4096 and 9..32 activation rows per workgroup
-// (bf16 weight): the companion of out_decode_r8.hip for the larger decode batches
+// (bf16 or fp8 weight): the companion of out_decode_r8.hip for the larger decode batches
 //   out[r, n] = sum_k x[r, k] * W[n, k] + b[n] + res[r, n]        (out_residual_decode_forward, triton_kernels.py:1470-1517)
 //
 // Same skeleton: one workgroup per twelve output features (gpt-oss: 240 workgroups, one per CU), one 16-row MFMA tile
@@ -13,6 +13,9 @@
 // through a ring of three 11 KB regions: three phases are in flight, a phase is multiplied as soon as it has landed
 // and its region is then refilled with the phase three further on (a ring of two measures 1 % slower: the depth is
 // not what bounds the kernel). Two epilogue wavefronts, one per column block.
+// W8: fp8 (OCP e4m3) weight with one fp32 scale per output row (the reference's ATTN_FP8 option,
+// triton_kernels.py:1385-1408): a weight row of a phase is 128 bytes (two loads of eight rows), fragments are widened
+// to bf16 (exact) between the LDS read and the MFMA, the row scale multiplies the finished sum.
 // XB = four-row activation blocks fetched per phase (rows past a chunk's last one repeat it; with fewer than 29 rows
 // the blocks that would hold no real row are not fetched at all).
 #include "out_common.h"
@@ -31,10 +34,11 @@ constexpr int WPH = 3 * 1024;     // weight of one phase: 12 rows x four k32 ste
 constexpr int REGION = XPH + WPH;
 }  // namespace r32o
 
-template <int XB>
+template <int XB, bool W8>
 __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8) {
   using namespace r32o;
-  constexpr int LPP = XB + 3;                               // load instructions per phase
+  constexpr int LW = W8 ? 2 : 3;                            // weight load instructions per phase
+  constexpr int LPP = XB + LW;                              // load instructions per phase
   __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -81,6 +85,12 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
       if (!a.bias) bv[i] = 0.f;
       if (!a.res) rv[i] = 0.f;
     }
+    float ws[4] = {1.f, 1.f, 1.f, 1.f};                    // W8: the row scales of the lane's four features
+    if constexpr (W8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ws[i] = a.w_scale[efeat + i];
+      asm volatile("" : "+v"(ws[0]), "+v"(ws[1]), "+v"(ws[2]), "+v"(ws[3]));
+    }
     unsigned red_o = static_cast<unsigned>(cb * 1024 + lane * 16);
     // the wavefronts run alone from the barrier to the stores: everything that does not need the sums exists before it
     asm volatile("" : "+v"(bv[0]), "+v"(bv[1]), "+v"(bv[2]), "+v"(bv[3]), "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]), "+v"(out), "+v"(red_o));
@@ -99,7 +109,7 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     if (!evalid) return;
     bf16x4 o;                                               // features efeat .. efeat + 3 of row en
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] + bv[i] + rv[i]);
+    for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] * ws[i] + bv[i] + rv[i]);
     if (vec8) {
       *reinterpret_cast<bf16x4*>(out) = o;
     } else {
@@ -116,17 +126,25 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
 
   // lane -> (row of a 4-row block, position): it fetches chunk position ^ (row & 15) of that row's 256 bytes, so that
   // the 16 rows a fragment read touches lie in 16 different bank groups
-  unsigned xoff[XB], goff[3];
+  unsigned xoff[XB], goff[LW];
 #pragma unroll
   for (int j = 0; j < XB; ++j) {
     const int r = 4 * j + (lane >> 4);
     const int src = r < nvalid ? r : nvalid - 1;            // row inside the workgroup's 32 (the base below points at row0)
     xoff[j] = static_cast<unsigned>(src * 8192 + kq * 256 + (((lane & 15) ^ (r & 15)) << 4));
   }
+  // (W8: a weight row of a phase is 128 bytes = 8 chunks and a load covers eight rows: lane -> row 8 j + lane / 8,
+  // position lane % 8, chunk position ^ (row & 7); rows 12..15 of the second load repeat row 11, unread)
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    const int r = 4 * j + (lane >> 4);
-    goff[j] = static_cast<unsigned>(n0 + r) * 8192u + kq * 256u + (((lane & 15) ^ r) << 4);
+  for (int j = 0; j < LW; ++j) {
+    if constexpr (W8) {
+      int r = 8 * j + (lane >> 3);
+      r = r < RW ? r : RW - 1;
+      goff[j] = static_cast<unsigned>(n0 + r) * 4096u + kq * 128u + (((lane & 7) ^ (r & 7)) << 4);
+    } else {
+      const int r = 4 * j + (lane >> 4);
+      goff[j] = static_cast<unsigned>(n0 + r) * 8192u + kq * 256u + (((lane & 15) ^ r) << 4);
+    }
   }
   const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x) + row0 * 8192;
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
@@ -134,14 +152,14 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   auto issue_phase = [&](int p) {                           // the activations of the phase, then its weight
     unsigned char* reg = myring + (p % RING) * REGION;
     const unsigned char* xb = xbase + p * 1024;
-    const unsigned char* wb = wbase + p * 1024;
+    const unsigned char* wb = wbase + p * (W8 ? 512 : 1024);
 #pragma unroll
     for (int j = 0; j < XB; ++j) {
       const unsigned dst = lds_addr(reg + j * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[j]), "s"(xb) : "memory", "m0");
     }
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
+    for (int j = 0; j < LW; ++j) {
       const unsigned dst = lds_addr(reg + XPH + j * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff[j]), "s"(wb) : "memory", "m0");
     }
@@ -153,7 +171,14 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
   acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int arow = m < RW ? m : m - RW;                     // tile rows past the twelfth re-read a real one (their sums are dropped)
-  const unsigned a_o = XPH + arow * 256;
+  const unsigned a_o = XPH + arow * (W8 ? 128 : 256);
+  // W8: the lane's eight fp8 of step st are bytes 32 st + 8 g of the 128-byte row: half g & 1 of chunk 2 st + g / 2,
+  // which sits at position chunk ^ (row & 7)
+  auto w8frag = [&](const unsigned char* reg, int st) {
+    typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+    const u32x2 raw = *reinterpret_cast<const u32x2*>(reg + a_o + (((2 * st + (g >> 1)) ^ (arow & 7)) << 4) + (g & 1) * 8);
+    return fp8x8_to_bf16x8(raw[0], raw[1]);
+  };
   const unsigned b0_o = m * 256, b1_o = (16 + m) * 256;
 #pragma unroll
   for (int p = 0; p < NPH; ++p) {
@@ -166,7 +191,8 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     bf16x8 fa[4], fb0[4], fb1[4];
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
-      fa[st] = *reinterpret_cast<const bf16x8*>(reg + a_o + (((4 * st + g) ^ arow) << 4));
+      if constexpr (W8) fa[st] = w8frag(reg, st);
+      else fa[st] = *reinterpret_cast<const bf16x8*>(reg + a_o + (((4 * st + g) ^ arow) << 4));
       fb0[st] = *reinterpret_cast<const bf16x8*>(reg + b0_o + (((4 * st + g) ^ m) << 4));
       if constexpr (XB > 4) fb1[st] = *reinterpret_cast<const bf16x8*>(reg + b1_o + (((4 * st + g) ^ m) << 4));
     }
@@ -188,21 +214,27 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   __syncthreads();
 }
 
-// in_dim 4096, out_dim % 12 == 0, bf16 weight; grid = (out_dim / 12, ceil(rows / 32))
+// in_dim 4096, out_dim % 12 == 0, bf16 weight or (a.w_scale != null) fp8; grid = (out_dim / 12, ceil(rows / 32))
 void launch_out_decode_r32(dim3 grid, hipStream_t st, const OutArgs& a) {
   auto al8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
   const int vec8 = al8(a.out) && a.out_rs % 4 == 0 && (a.res == nullptr || (al8(a.res) && a.res_rs % 4 == 0)) && (a.bias == nullptr || al8(a.bias));
   const int rows = static_cast<int>(a.rows < 32 ? a.rows : 32);          // of the fullest chunk
+#define TLLM_OUT32(XB)                                                                                        \
+  do {                                                                                                        \
+    if (a.w_scale) hipLaunchKernelGGL((out_decode_r32_kernel<XB, true>), grid, dim3(384), 0, st, a, vec8);   \
+    else hipLaunchKernelGGL((out_decode_r32_kernel<XB, false>), grid, dim3(384), 0, st, a, vec8);            \
+  } while (0)
   switch ((rows + 3) / 4) {
-    case 1: hipLaunchKernelGGL(out_decode_r32_kernel<1>, grid, dim3(384), 0, st, a, vec8); break;
-    case 2: hipLaunchKernelGGL(out_decode_r32_kernel<2>, grid, dim3(384), 0, st, a, vec8); break;
-    case 3: hipLaunchKernelGGL(out_decode_r32_kernel<3>, grid, dim3(384), 0, st, a, vec8); break;
-    case 4: hipLaunchKernelGGL(out_decode_r32_kernel<4>, grid, dim3(384), 0, st, a, vec8); break;
-    case 5: hipLaunchKernelGGL(out_decode_r32_kernel<5>, grid, dim3(384), 0, st, a, vec8); break;
-    case 6: hipLaunchKernelGGL(out_decode_r32_kernel<6>, grid, dim3(384), 0, st, a, vec8); break;
-    case 7: hipLaunchKernelGGL(out_decode_r32_kernel<7>, grid, dim3(384), 0, st, a, vec8); break;
-    default: hipLaunchKernelGGL(out_decode_r32_kernel<8>, grid, dim3(384), 0, st, a, vec8); break;
+    case 1: TLLM_OUT32(1); break;
+    case 2: TLLM_OUT32(2); break;
+    case 3: TLLM_OUT32(3); break;
+    case 4: TLLM_OUT32(4); break;
+    case 5: TLLM_OUT32(5); break;
+    case 6: TLLM_OUT32(6); break;
+    case 7: TLLM_OUT32(7); break;
+    default: TLLM_OUT32(8); break;
   }
+#undef TLLM_OUT32
 }
 
 }  // namespace tllm
