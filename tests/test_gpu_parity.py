@@ -794,25 +794,30 @@ def test_out_residual_decode_parity(gpu, rows, fp8):
 
 
 @pytest.mark.parametrize("rows", [1, 5, 8, 13, 32, 37])
-def test_out_residual_decode_strides_alignment_and_absent_operands(gpu, rows):
+@pytest.mark.parametrize("fp8", [False, True])
+def test_out_residual_decode_strides_alignment_and_absent_operands(gpu, rows, fp8):
     """The C entry point with what the host wrapper never passes: a separate output buffer, row strides that rule
     out 8-byte accesses (2882) and ones that allow them (2884), an output that starts 2 bytes off an 8-byte boundary,
-    no bias, no residual. Untouched padding columns must stay untouched."""
+    no bias, no residual; bf16 weight and fp8 weight with row scales. Untouched padding columns must stay untouched."""
     from tritonllm_amd import _lib
     L = _lib.lib()
     d = _out_inputs(rows, 650 + rows)
     x, w, b = d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu)
+    w_ref, ws = d["w"], None
+    if fp8:
+        w, ws = T.quantize_fp8_rows(w)
+        w_ref = O.dequant_fp8_ref(w.cpu(), ws.cpu())
     for stride, shift, with_bias, with_res in ((2884, 0, True, True), (2882, 0, True, True), (2884, 1, True, True),
                                                (2880, 0, False, True), (2880, 0, True, False), (2880, 0, False, False)):
         res = torch.zeros(rows, stride, dtype=torch.bfloat16, device=gpu)
         res[:, :2880] = d["r"].to(gpu)
         buf = torch.full((rows * stride + 8,), 7.0, dtype=torch.bfloat16, device=gpu)
         out = buf[shift:shift + rows * stride].view(rows, stride)
-        rc = L.tllm_out_residual_decode_bf16(x.data_ptr(), w.data_ptr(), None, b.data_ptr() if with_bias else None,
+        rc = L.tllm_out_residual_decode_bf16(x.data_ptr(), w.data_ptr(), ws.data_ptr() if fp8 else None, b.data_ptr() if with_bias else None,
                                              res.data_ptr() if with_res else None, out.data_ptr(), stride, stride, rows, 4096, 2880, None)
         assert rc == 0, L.tllm_last_error()
         torch.cuda.synchronize()
-        want = O.out_residual_ref(d["x"], d["w"], d["b"] if with_bias else torch.zeros_like(d["b"]),
+        want = O.out_residual_ref(d["x"], w_ref, d["b"] if with_bias else torch.zeros_like(d["b"]),
                                   d["r"] if with_res else torch.zeros_like(d["r"]))
         close(out[:, :2880], want)
         assert torch.all(out[:, 2880:] == 7.0) and torch.all(buf[:shift] == 7.0) and torch.all(buf[shift + rows * stride:] == 7.0)
