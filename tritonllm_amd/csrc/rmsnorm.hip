@@ -111,13 +111,42 @@ __global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const bf16x8* x, cons
   }
 }
 
-// One 256-lane workgroup per row; VPT = 16-byte vectors per thread.
+// The scale vectors of 16-byte vector `vec` as they lie in memory (one 16-byte load for bf16, two for fp32), so that a
+// kernel can request them before it needs them.
+template <bool kScaleBf16>
+struct ScaleRaw {
+  bf16x8 b;
+  f32x4 f0, f1;
+  __device__ __forceinline__ void load(const void* scale, int vec) {
+    if constexpr (kScaleBf16) {
+      b = reinterpret_cast<const bf16x8*>(scale)[vec];
+    } else {
+      const f32x4* sp = reinterpret_cast<const f32x4*>(scale) + 2 * vec;
+      f0 = sp[0];
+      f1 = sp[1];
+    }
+  }
+  __device__ __forceinline__ float at(int j) const {
+    if constexpr (kScaleBf16) return static_cast<float>(b[j]);
+    else return j < 4 ? f0[j] : f1[j - 4];
+  }
+};
+
+// One 256-lane workgroup per row; VPT = 16-byte vectors per thread. The few-row case is all latency, so every load --
+// the row and the scale -- goes out before anything waits (left at its use, behind the barrier, the scale's load would
+// add a memory round trip to the chain: 2.36 -> 2.28 us at 8 rows, 2.43 -> 2.34 at 32, same box).
 template <int VPT, bool kScaleBf16, bool GATHER>
 __global__ __launch_bounds__(256) void rmsnorm_block_kernel(const bf16x8* x, const void* __restrict__ scale,
                                                             bf16x8* out, int nvec, float hidden_f, float eps, GatherSrc g) {
   __shared__ float part[4];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
+  ScaleRaw<kScaleBf16> sc[VPT];
+  if constexpr (GATHER) {
+    // the row's address hangs on the token id: the scale can travel meanwhile
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) sc[i].load(scale, tid + i * 256 < nvec ? tid + i * 256 : 0);
+  }
   const bf16x8* xr = GATHER ? gather_row(g, x, row, nvec, tid == 0) : x + row * nvec;
   bf16x8 v[VPT];
 #pragma unroll
@@ -129,6 +158,10 @@ __global__ __launch_bounds__(256) void rmsnorm_block_kernel(const bf16x8* x, con
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[i][j] = static_cast<bf16>(0.f);
     }
+  }
+  if constexpr (!GATHER) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) sc[i].load(scale, tid + i * 256 < nvec ? tid + i * 256 : 0);
   }
   if constexpr (GATHER) {
 #pragma unroll
@@ -149,7 +182,10 @@ __global__ __launch_bounds__(256) void rmsnorm_block_kernel(const bf16x8* x, con
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int idx = tid + i * 256;
-    if (idx < nvec) __builtin_nontemporal_store(normalize8<kScaleBf16>(v[i], rinv, scale, idx), orow + idx);   // streamed out: measured 5-18 % faster
+    bf16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = static_cast<bf16>(static_cast<float>(v[i][j]) * rinv * sc[i].at(j));
+    if (idx < nvec) __builtin_nontemporal_store(o, orow + idx);   // streamed out: measured 5-18 % faster at prompt sizes, level at a few rows
   }
 }
 
