@@ -122,19 +122,16 @@ __device__ __forceinline__ void rope_cos_sin(const RopeArgs& r, const YarnFreqs&
   }
 }
 
-// Eight fp8 (OCP e4m3) values in two dwords -> eight bf16, exactly: e4m3 -> fp32 has at most four significant bits, so
-// the upper halves of the fp32 values are the bf16 values.
+// Eight fp8 (OCP e4m3) values in two dwords -> eight bf16, exactly (bf16 holds every e4m3 value): gfx950's packed
+// conversion takes two fp8 of one 16-bit half to two bf16, times a scale of 1 -- four instructions for the eight values
+// (through fp32 pairs and a byte permute it was eight). The results are taken as whole registers.
 __device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
   typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
-  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
-  const unsigned raw[2] = {lo, hi};
   u32x4 o;
-#pragma unroll
-  for (int d = 0; d < 2; ++d) {
-    const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[d]), true);
-    o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
-    o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
-  }
+  o[0] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false));
+  o[1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true));
+  o[2] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false));
+  o[3] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true));
   return __builtin_bit_cast(bf16x8, o);
 }
 

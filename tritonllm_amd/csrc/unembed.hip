@@ -136,21 +136,10 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
         for (int i = 0; i < LPS; ++i) {
           const int r = (i * 64 + lane) / CPS, kc = (i * 64 + lane) % CPS;
           if constexpr (W8) {
-            typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
-            typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
-            const i32x4 raw = __builtin_bit_cast(i32x4, buf[d][i]);
-            bf16x8 w0, w1;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[q], false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(raw[q], true);
-              bf16x8& dst = q < 2 ? w0 : w1;
-              dst[4 * (q & 1) + 0] = static_cast<bf16>(p0[0]);
-              dst[4 * (q & 1) + 1] = static_cast<bf16>(p0[1]);
-              dst[4 * (q & 1) + 2] = static_cast<bf16>(p1[0]);
-              dst[4 * (q & 1) + 3] = static_cast<bf16>(p1[1]);
-            }
-            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32) = w0;
-            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32 + 16) = w1;
+            typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+            const u32x4 raw = __builtin_bit_cast(u32x4, buf[d][i]);                    // sixteen fp8
+            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32) = fp8x8_to_bf16x8(raw[0], raw[1]);
+            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32 + 16) = fp8x8_to_bf16x8(raw[2], raw[3]);
           } else {
             *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 16) = buf[d][i];
           }
