@@ -70,7 +70,11 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   __syncthreads();
 
   // ---- this wavefront's tiles: t = gw, gw + G, gw + 2G, ...
-  const int gw = blockIdx.x * UNW + wave, G = gridDim.x * UNW;
+  // Wavefront w of workgroup b is number w * gridDim.x + b: when the tiles do not divide evenly (201088 rows are 6284
+  // tiles for 4096 wavefronts) the ones that take one tile more are the first wavefronts of EVERY workgroup, not all
+  // the wavefronts of the first workgroups -- every CU then streams to the end of the launch.
+  const int G = gridDim.x * UNW;
+  const int gw = wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x);
   const int ntiles = (a.vocab + 31) >> 5;
   const int my_tiles = gw < ntiles ? (ntiles - gw + G - 1) / G : 0;
   const int total = my_tiles * nsteps;                        // steps of the whole stream
