@@ -30,6 +30,35 @@ __global__ __launch_bounds__(256) void embedding_vec_kernel(const bf16x8* __rest
   }
 }
 
+// A decode batch: a handful of tokens. One workgroup per token, a row's vectors dealt over its 256 lanes with every load
+// requested before the first store -- the launch is one id load and one row round trip deep.
+template <typename IdT, int VPT>
+__global__ __launch_bounds__(256) void embedding_few_kernel(const bf16x8* __restrict__ table, const IdT* __restrict__ ids,
+                                                            bf16x8* __restrict__ out, int nvec, int64_t vocab, int32_t* oob_flag) {
+  const int tid = threadIdx.x;
+  const int64_t t = blockIdx.x;
+  const int64_t id = static_cast<int64_t>(ids[t]);
+  const bool ok = id >= 0 && id < vocab;
+  const bf16x8* src = table + (ok ? id : 0) * nvec;
+  bf16x8 v[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int idx = tid + i * 256;
+    v[i] = src[idx < nvec ? idx : 0];
+  }
+  bf16x8* dst = out + t * nvec;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int idx = tid + i * 256;
+    if (!ok) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[i][j] = static_cast<bf16>(0.f);
+    }
+    if (idx < nvec) dst[idx] = v[i];
+  }
+  if (!ok && oob_flag && tid == 0) *oob_flag = 1;
+}
+
 template <typename IdT>
 __global__ __launch_bounds__(256) void embedding_scalar_kernel(const uint16_t* __restrict__ table, const IdT* __restrict__ ids,
                                                                uint16_t* __restrict__ out, int64_t n_tokens, int64_t hidden,
@@ -54,7 +83,25 @@ extern "C" int tllm_embedding_bf16(const void* table, const void* ids, int ids_i
   TLLM_REQUIRE(table && ids && out, TLLM_E_ARG, "embedding: null pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec_ok = hidden % 8 == 0 && aligned16(table) && aligned16(out) && hidden / 8 < (1ll << 31);
-  if (vec_ok) {
+  if (vec_ok && n_tokens <= 64 && hidden / 8 <= 4 * 256) {
+    const int nvec = static_cast<int>(hidden / 8);
+    const int vpt = (nvec + 255) / 256;
+    dim3 grid(static_cast<unsigned>(n_tokens)), block(256);
+#define TLLM_FEW(V)                                                                                                              \
+  do {                                                                                                                           \
+    if (ids_is_i64)                                                                                                              \
+      hipLaunchKernelGGL((embedding_few_kernel<int64_t, V>), grid, block, 0, st, (const bf16x8*)table, (const int64_t*)ids,      \
+                         (bf16x8*)out, nvec, vocab, oob_flag);                                                                   \
+    else                                                                                                                         \
+      hipLaunchKernelGGL((embedding_few_kernel<int32_t, V>), grid, block, 0, st, (const bf16x8*)table, (const int32_t*)ids,      \
+                         (bf16x8*)out, nvec, vocab, oob_flag);                                                                   \
+  } while (0)
+    if (vpt == 1) TLLM_FEW(1);
+    else if (vpt == 2) TLLM_FEW(2);
+    else if (vpt == 3) TLLM_FEW(3);
+    else TLLM_FEW(4);
+#undef TLLM_FEW
+  } else if (vec_ok) {
     const int64_t blocks = (n_tokens + 3) / 4;
     dim3 grid(static_cast<unsigned>(blocks < 16384 ? blocks : 16384)), block(256);
     const int nvec = static_cast<int>(hidden / 8);
