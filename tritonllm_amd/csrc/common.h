@@ -1,5 +1,6 @@
 // Shared device/host helpers for the gfx950 layer kernels.
 #pragma once
+#include <type_traits>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -32,10 +33,21 @@ int check_launch(const char* what);
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- device helpers --------------------------------------------------------
+// Sum over the 64 lanes, the same value in every lane. Inside a row of 16 lanes through DPP operands (lane ^ 1, lane ^ 2,
+// the mirrored half row, the mirrored row: four adds, no LDS crossbar), across the four rows through scalar registers.
+// (Six __shfl_xor steps are six ds_bpermute round trips, ~0.2 us on the critical path of a few-row kernel.)
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  v += dpp(v, std::integral_constant<int, 0xB1>{});        // quad_perm [1, 0, 3, 2]
+  v += dpp(v, std::integral_constant<int, 0x4E>{});        // quad_perm [2, 3, 0, 1]
+  v += dpp(v, std::integral_constant<int, 0x141>{});       // row_half_mirror
+  v += dpp(v, std::integral_constant<int, 0x140>{});       // row_mirror
+  const int b = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return (r0 + r1) + (r2 + r3);
 }
 
 // Kernel-argument copy of the rotary source (TllmRope with the YaRN block by value).
