@@ -211,8 +211,7 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
         sc[4 * kb + i] = s;
         bmax = fmaxf(bmax, s);
       }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    bmax = max_over_lane_bits_16_32(bmax);
     const float m_new = fmaxf(m_run, bmax);
     const float alpha = __expf(m_run - m_new);
     float psum = 0.f;
@@ -223,8 +222,7 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
       psum += p;
       pa[j] = static_cast<bf16>(p);
     }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
+    psum = sum_over_lane_bits_16_32(psum);
     l_run = l_run * alpha + psum;
     m_run = m_new;
 

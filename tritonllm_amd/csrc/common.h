@@ -50,6 +50,41 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// The lane's own value and that of lane ^ 16 (lane ^ 32), in some order -- enough for a sum or a maximum. gfx950's row
+// and half-wavefront swaps are vector-ALU instructions; __shfl_xor goes through the LDS crossbar and waits for it.
+// (The two results are taken out of the returned pair as one 64-bit value: element access on it reads element 0 twice
+// with this compiler.)
+__device__ __forceinline__ void lane_xor16_pair(float x, float* a, float* b) {
+  const int xi = __builtin_bit_cast(int, x);
+  const unsigned long long u = __builtin_bit_cast(unsigned long long, __builtin_amdgcn_permlane16_swap(xi, xi, false, false));
+  *a = __uint_as_float(static_cast<unsigned>(u));
+  *b = __uint_as_float(static_cast<unsigned>(u >> 32));
+}
+__device__ __forceinline__ void lane_xor32_pair(float x, float* a, float* b) {
+  const int xi = __builtin_bit_cast(int, x);
+  const unsigned long long u = __builtin_bit_cast(unsigned long long, __builtin_amdgcn_permlane32_swap(xi, xi, false, false));
+  *a = __uint_as_float(static_cast<unsigned>(u));
+  *b = __uint_as_float(static_cast<unsigned>(u >> 32));
+}
+// x + (x of lane ^ 8), x + (x of lane ^ 16) + ..., as sums and maxima over the lanes that differ in the given bits
+__device__ __forceinline__ float lane_xor8_value(float x) {   // row_ror:8 inside a row of 16 lanes
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float sum_over_lane_bits_16_32(float x) {
+  float a, b;
+  lane_xor16_pair(x, &a, &b);
+  x = a + b;
+  lane_xor32_pair(x, &a, &b);
+  return a + b;
+}
+__device__ __forceinline__ float max_over_lane_bits_16_32(float x) {
+  float a, b;
+  lane_xor16_pair(x, &a, &b);
+  x = fmaxf(a, b);
+  lane_xor32_pair(x, &a, &b);
+  return fmaxf(a, b);
+}
+
 // Kernel-argument copy of the rotary source (TllmRope with the YaRN block by value).
 struct RopeArgs {
   const float* cos_table;

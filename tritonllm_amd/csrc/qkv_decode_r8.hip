@@ -341,8 +341,7 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
       float ssq = 0.f;
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) ssq += sumsq(fb[s]);
-      ssq += __shfl_xor(ssq, 16, 64);
-      ssq += __shfl_xor(ssq, 32, 64);
+      ssq = sum_over_lane_bits_16_32(ssq);
       const float rinv = publish_and_meet(ssq);             // lanes 0..15: row m1 == lane
 #ifdef TLLM_R8_STAMPS
       R8_STAMP(3);
@@ -381,9 +380,8 @@ __global__ __launch_bounds__(512) void qkv_decode_r8_kernel(QkvArgs a, RopeArgs 
       float ssq = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) ssq += (j == 7 && h == 1) ? 0.f : sumsq(own[j]);
-      ssq += __shfl_xor(ssq, 8, 64);
-      ssq += __shfl_xor(ssq, 16, 64);
-      ssq += __shfl_xor(ssq, 32, 64);
+      ssq += lane_xor8_value(ssq);
+      ssq = sum_over_lane_bits_16_32(ssq);
       const float rinv = publish_and_meet(ssq);             // lanes 0..7: row m1 == lane
 #ifdef TLLM_R8_STAMPS
       R8_STAMP(3);
