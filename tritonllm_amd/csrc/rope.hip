@@ -67,6 +67,53 @@ __global__ __launch_bounds__(256) void rope_kernel(bf16x8* q, bf16x8* k, int64_t
   }
 }
 
+// A decode batch: one token per workgroup, gridDim.y workgroups sharing its heads, one item per lane. The item's two
+// vectors are requested before anything else, so that the position load and the cos / sin arithmetic of the first n_freq
+// lanes run while they are on their way; one barrier, then rotate and store.
+__global__ __launch_bounds__(256) void rope_few_kernel(bf16x8* q, bf16x8* k, int n_q_heads, int n_kv_heads, int head_dim, RopeArgs ra,
+                                                       YarnFreqs fr) {
+  __shared__ float s_cos[TLLM_MAX_ROPE_FREQS];
+  __shared__ float s_sin[TLLM_MAX_ROPE_FREQS];
+  const int tid = threadIdx.x;
+  const int n_freq = head_dim >> 1;
+  const int64_t row = blockIdx.x;
+  const int vph = n_freq >> 3;                       // 128-bit vectors per half head
+  const int items = (n_q_heads + n_kv_heads) * vph;
+  const int it = blockIdx.y * 256 + tid;
+  const bool valid = it < items;
+  const int itc = valid ? it : 0;
+  const int h = itc / vph, j = itc - h * vph;
+  bf16x8* base;
+  if (h < n_q_heads)
+    base = q + (row * n_q_heads + h) * (2 * vph);
+  else
+    base = k + (row * n_kv_heads + (h - n_q_heads)) * (2 * vph);
+  const bf16x8 lo = base[j], hi = base[vph + j];     // lanes past the last item read item 0 and store nothing
+
+  for (int i = tid; i < n_freq; i += 256) {
+    const int64_t pos = rope_position(ra, row);
+    float c, s;
+    rope_cos_sin(ra, fr, pos, i, &c, &s);
+    s_cos[i] = c;
+    s_sin[i] = s;
+  }
+  __syncthreads();
+  if (!valid) return;
+
+  const float* cs = s_cos + 8 * j;
+  const float* sn = s_sin + 8 * j;
+  bf16x8 olo, ohi;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float x1 = static_cast<float>(lo[e]), x2 = static_cast<float>(hi[e]);
+    const float c = cs[e], s = sn[e];
+    olo[e] = static_cast<bf16>(x1 * c - x2 * s);
+    ohi[e] = static_cast<bf16>(x2 * c + x1 * s);
+  }
+  base[j] = olo;
+  base[vph + j] = ohi;
+}
+
 __global__ __launch_bounds__(256) void yarn_table_kernel(float* cos_out, float* sin_out, int64_t start, int64_t n_pos, int n_freq,
                                                          float concentration, YarnFreqs fr) {
   const int64_t total = n_pos * n_freq;
@@ -102,8 +149,12 @@ extern "C" int tllm_rope_bf16(void* q, void* k, int64_t rows, int n_q_heads, int
     const int items = (n_q_heads + n_kv_heads) * (head_dim >> 4);     // per token
     int parts = (items + 255) / 256;
     parts = parts < 1 ? 1 : (parts > 64 ? 64 : parts);
-    hipLaunchKernelGGL(rope_kernel<1>, dim3((unsigned)rows, (unsigned)parts), dim3(256), 0, static_cast<hipStream_t>(stream), (bf16x8*)q,
-                       (bf16x8*)k, rows, n_q_heads, n_kv_heads, head_dim, ra, fr);
+    if (items <= parts * 256)     // one item per lane
+      hipLaunchKernelGGL(rope_few_kernel, dim3((unsigned)rows, (unsigned)parts), dim3(256), 0, static_cast<hipStream_t>(stream),
+                         (bf16x8*)q, (bf16x8*)k, n_q_heads, n_kv_heads, head_dim, ra, fr);
+    else
+      hipLaunchKernelGGL(rope_kernel<1>, dim3((unsigned)rows, (unsigned)parts), dim3(256), 0, static_cast<hipStream_t>(stream), (bf16x8*)q,
+                         (bf16x8*)k, rows, n_q_heads, n_kv_heads, head_dim, ra, fr);
     return check_launch("rope");
   }
   const int64_t blocks = (rows + kRopeTok - 1) / kRopeTok;
