@@ -119,6 +119,10 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
     kind, _, size = name.rpartition("_")
     n = int(size[1:])
     flops = nbytes = None
+    tables = kind == "qkv_rope_prefill_tables"           # cos / sin from the precomputed tables, as the reference passes them
+    if tables:
+        kind = "qkv_rope_prefill"
+        rope_t = T.RotaryEmbedding(HD, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=dev)
     if kind in ("qkv_rope_prefill", "qkv_rope_decode", "norm_qkv_rope_decode", "qkv_rope_decode_w8", "norm_qkv_rope_decode_w8"):
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         pp = torch.arange(n, dtype=torch.int64, device=dev) if kind.endswith("prefill") else \
@@ -128,10 +132,11 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         mode = "prefill" if kind.endswith("prefill") else "decode"
         fused, w8 = kind.startswith("norm_"), kind.endswith("_w8")
         wq = [T.quantize_fp8_rows(w) for w in weights] if w8 else None
+        how = dict(cos=rope_t.cos.clone(), sin=rope_t.sin.clone(), max_context_length=rope_t.max_context_length) if tables else dict(yarn=yarn)
         fn = lambda i: T.qkv_rope_forward(xp, wq[i % N_LAYERS][0] if w8 else weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
-                                          yarn=yarn, positions=pp, mode=mode, out=qo,
+                                          positions=pp, mode=mode, out=qo,
                                           norm_scale=scales[i % N_LAYERS] if fused else None,
-                                          weight_scale=wq[i % N_LAYERS][1] if w8 else None)
+                                          weight_scale=wq[i % N_LAYERS][1] if w8 else None, **how)
         flops, nbytes = 2.0 * n * HIDDEN * QKV_DIM, bytes_of[("norm_qkv" if fused else "qkv") + ("_w8" if w8 else "")](n)
     elif kind == "embed_norm_qkv_rope_decode":
         idp = torch.randint(0, VOCAB_BENCH, (n,), generator=g, dtype=torch.int32).to(dev)

@@ -158,6 +158,8 @@ __device__ __forceinline__ void rope_positions_16_uniform(const RopeArgs& r, con
   }
 }
 
+// TABLE: cos / sin come from the caller's tables (two loads per value) instead of the YaRN parameters.
+template <bool TABLE>
 __global__ __launch_bounds__(512) void qkv_prefill_quads_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
   constexpr int BM = 128;
   constexpr int WS = w_stages(BM);          // weight stages (3)
@@ -315,10 +317,14 @@ __global__ __launch_bounds__(512) void qkv_prefill_quads_kernel(QkvArgs a, RopeA
   constexpr int CSN = 8;
   static_assert(NW * 2 * CSN == EROWS && EROWS == BM, "eight wavefronts x two rows x eight rounds cover the tile");
   float2 csr[CSN];
-  if (a.has_rope) {
+  if (TABLE || a.has_rope) {
     const int f = lane & 31;
     int64_t pos_even[CSN], pos_odd[CSN];
     rope_positions_16_uniform(ra, a.W, row0 + 16 * wave, a.rows, pos_even, pos_odd);
+    // TABLE: the loads go out whether there is a rotation or not (without one they read the weight's first bytes), so
+    // that the waits below can count on them, and no branch surrounds a load.
+    const float* cos_t = a.has_rope ? ra.cos_table : reinterpret_cast<const float*>(a.W);
+    const float* sin_t = a.has_rope ? ra.sin_table : reinterpret_cast<const float*>(a.W);
 #pragma unroll
     for (int j = 0; j < CSN; ++j) {
       int64_t p = lane < 32 ? pos_even[j] : pos_odd[j];
@@ -327,12 +333,23 @@ __global__ __launch_bounds__(512) void qkv_prefill_quads_kernel(QkvArgs a, RopeA
         if (grow >= a.rows) grow = a.rows - 1;
         p += grow < ra.tokens_per_batch ? grow : grow % ra.tokens_per_batch;
       }
-      float c, sn;
-      rope_cos_sin(ra, fr, rope_wrap(p, ra.max_ctx), f, &c, &sn);
-      csr[j] = make_float2(c, sn);
+      if constexpr (TABLE) {
+        const int64_t at = a.has_rope ? rope_wrap(p, ra.max_ctx) * ra.table_row_stride + f : f;
+        // The youngest loads of the prologue: a wait counts them in until they have landed, which they have by the
+        // loop's second slice (they return behind the look-ahead loads issued before them).
+        csr[j] = make_float2(cos_t[at], sin_t[at]);
+      } else {
+        float c, sn;
+        yarn_cos_sin(rope_wrap(p, ra.max_ctx), fr.v[f], ra.concentration, &c, &sn);
+        csr[j] = make_float2(c, sn);
+      }
     }
   }
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");   // slice 0 has landed when only those are outstanding
+  // slice 0 has landed when only those are outstanding
+  if constexpr (TABLE)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW + 2 * CSN) : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");
   __syncthreads();
 #pragma unroll
   for (int tb = 0; tb < TB; ++tb) fx[0][tb] = *reinterpret_cast<const bf16x8*>(xring + fx_o[tb]);
@@ -421,6 +438,7 @@ __device__ __forceinline__ void w_tile_row(int i, int* head_local, int* dim) {
   }
 }
 
+template <bool TABLE>
 __global__ __launch_bounds__(512) void qkv_prefill_kernel256(QkvArgs a, RopeArgs ra, YarnFreqs fr, int tiles_m, int tiles_n, int swizzle) {
   constexpr int BM = 256;
   constexpr int WS = w_stages(BM);          // weight stages (2)
@@ -598,11 +616,23 @@ __global__ __launch_bounds__(512) void qkv_prefill_kernel256(QkvArgs a, RopeArgs
       int64_t pos[EROWS / 16];
 #pragma unroll
       for (int j = 0; j < EROWS / 16; ++j) pos[j] = pos_s[EROWS * pass + (tid >> 5) + 16 * j];
+      if constexpr (TABLE) {
+        float c[EROWS / 16], sn[EROWS / 16];                   // all sixteen loads out before the first is looked at
 #pragma unroll
-      for (int j = 0; j < EROWS / 16; ++j) {
-        float c, sn;
-        rope_cos_sin(ra, fr, rope_wrap(pos[j], ra.max_ctx), f, &c, &sn);
-        cs_tab[((tid >> 5) + 16 * j) * CSROW + f] = make_float2(c, sn);
+        for (int j = 0; j < EROWS / 16; ++j) {
+          const int64_t at = rope_wrap(pos[j], ra.max_ctx) * ra.table_row_stride + f;
+          c[j] = ra.cos_table[at];
+          sn[j] = ra.sin_table[at];
+        }
+#pragma unroll
+        for (int j = 0; j < EROWS / 16; ++j) cs_tab[((tid >> 5) + 16 * j) * CSROW + f] = make_float2(c[j], sn[j]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < EROWS / 16; ++j) {
+          float c, sn;
+          yarn_cos_sin(rope_wrap(pos[j], ra.max_ctx), fr.v[f], ra.concentration, &c, &sn);
+          cs_tab[((tid >> 5) + 16 * j) * CSROW + f] = make_float2(c, sn);
+        }
       }
     }
     __syncthreads();
@@ -688,11 +718,13 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   }
   static bool attr_set = false;   // raising the dynamic-LDS limit is idempotent; a benign race at worst repeats it
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_quads_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       prefill_smem(128));
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_prefill_kernel256), hipFuncAttributeMaxDynamicSharedMemorySize, prefill_smem(256));
-    TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_prefill: cannot raise LDS limit: %s", hipGetErrorString(e));
+    const void* k128[] = {reinterpret_cast<const void*>(qkv_prefill_quads_kernel<false>), reinterpret_cast<const void*>(qkv_prefill_quads_kernel<true>)};
+    const void* k256[] = {reinterpret_cast<const void*>(qkv_prefill_kernel256<false>), reinterpret_cast<const void*>(qkv_prefill_kernel256<true>)};
+    for (int t = 0; t < 2; ++t) {
+      hipError_t e = hipFuncSetAttribute(k128[t], hipFuncAttributeMaxDynamicSharedMemorySize, prefill_smem(128));
+      if (e == hipSuccess) e = hipFuncSetAttribute(k256[t], hipFuncAttributeMaxDynamicSharedMemorySize, prefill_smem(256));
+      TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_prefill: cannot raise LDS limit: %s", hipGetErrorString(e));
+    }
     attr_set = true;
   }
   const int heads = n_q_heads + 2 * n_kv_heads;
@@ -709,10 +741,19 @@ extern "C" int tllm_qkv_rope_prefill_bf16(const void* x, const void* W, const vo
   // Super-block of tiles per XCD: 8 x 4 (token tiles x column tiles). Measured at T = 2048: 8 x 4 and 16 x 2 66 us,
   // 4 x 8 71 us, 2 x 16 and no grouping 75 us; from T = 4096 up (256-token tiles) the shape makes no difference.
   const int swizzle = (tiles_m % 8 == 0 && tiles_n % 4 == 0) ? 8 : 0;
-  if (BM == 256)
-    hipLaunchKernelGGL(qkv_prefill_kernel256, dim3((unsigned)tiles), dim3(512), prefill_smem(256), st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
-  else
-    hipLaunchKernelGGL(qkv_prefill_quads_kernel, dim3((unsigned)tiles), dim3(512), prefill_smem(128), st, a, ra, fr, (int)tiles_m, tiles_n,
-                       swizzle);
+  // cos / sin from the caller's tables or, with YaRN parameters, computed in the kernel
+  const bool table = !ra.use_yarn;
+  const dim3 grid((unsigned)tiles), block(512);
+  if (BM == 256) {
+    if (table)
+      hipLaunchKernelGGL(qkv_prefill_kernel256<true>, grid, block, prefill_smem(256), st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
+    else
+      hipLaunchKernelGGL(qkv_prefill_kernel256<false>, grid, block, prefill_smem(256), st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
+  } else {
+    if (table)
+      hipLaunchKernelGGL(qkv_prefill_quads_kernel<true>, grid, block, prefill_smem(128), st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
+    else
+      hipLaunchKernelGGL(qkv_prefill_quads_kernel<false>, grid, block, prefill_smem(128), st, a, ra, fr, (int)tiles_m, tiles_n, swizzle);
+  }
   return check_launch("qkv_rope_prefill");
 }
