@@ -612,6 +612,21 @@ def test_qkv_rope_prefill_256_token_tiles(gpu, yarn, rows):
     _check_qkv(gpu, yarn, rows, "prefill", seed=rows, prefill_positions=rows % 2 == 0, max_pos=131072)
 
 
+@pytest.mark.parametrize("rows", [300, 2304])
+def test_qkv_rope_prefill_cos_sin_tables(gpu, rows):
+    """The prefill kernels' table variants (cos / sin loaded, as the reference passes them, triton_kernels.py:90) at both
+    tile heights, arbitrary positions, against the oracle; plain tensors, which the host side cannot trace back to YaRN
+    parameters."""
+    d = O.make_inputs(rows, seed=7000 + rows, prefill=False, max_pos=131072)
+    cos_t, sin_t = O.yarn_cos_sin(torch.arange(O.MAX_CTX))
+    q, k, v = T.qkv_rope_forward(d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64, cos=cos_t.to(gpu), sin=sin_t.to(gpu),
+                                 positions=d["positions"].to(gpu), mode="prefill")
+    qr, kr, vr = O.qkv_rope_ref(d["x"], d["w"], d["b"], d["positions"])
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+
+
 def test_qkv_decode_and_prefill_agree(gpu, yarn):
     d = O.make_inputs(40, seed=21)
     args = (d["x"].to(gpu), d["w"].to(gpu), d["b"].to(gpu), 64, 8, 64)

@@ -353,9 +353,7 @@ __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(AttnArgs a, int 
   const bool has = lane < live;
   const float m_s = has ? m_raw : kNegBig;
   const float l_s = has ? l_raw : 0.f;
-  float m_all = m_s;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, o, 64));
+  const float m_all = wave_max(m_s);
   const float f_s = __expf(m_s - m_all);                     // 0 for the lanes without a split
   const float l_all = wave_sum(l_s * f_s);
   float o = 0.f;
@@ -366,7 +364,9 @@ __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(AttnArgs a, int 
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const float f = __shfl(f_s, s0 + u < live ? s0 + u : 0, 64);
+      // the split index is the same in every lane: a scalar lane read, not a trip through the LDS crossbar
+      const float f = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f_s),
+                                                                          __builtin_amdgcn_readfirstlane(s0 + u < live ? s0 + u : 0)));
       o += (s0 + u < live) ? v[u] * f : 0.f;
     }
   }

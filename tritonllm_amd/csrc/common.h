@@ -50,6 +50,21 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// Maximum over the 64 lanes, the same value in every lane; the same route as wave_sum.
+__device__ __forceinline__ float wave_max(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0xB1>{}));
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x4E>{}));
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x141>{}));
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x140>{}));
+  const int b = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
 // The lane's own value and that of lane ^ 16 (lane ^ 32), in some order -- enough for a sum or a maximum. gfx950's row
 // and half-wavefront swaps are vector-ALU instructions; __shfl_xor goes through the LDS crossbar and waits for it.
 // (The two results are taken out of the returned pair as one 64-bit value: element access on it reads element 0 twice
