@@ -497,6 +497,19 @@ def main() -> int:
                          lambda i, xr=xr, pr=pr, qo=qo: T.qkv_rope_forward(xr, weights[i % N_LAYERS], biases[i % N_LAYERS], NQ, NKV, HD,
                                                                            yarn=yarn, positions=pr, mode="decode", out=qo),
                          bytes_of["qkv"](r), n=96)
+        # other model shapes (the reference's decode kernel is generic over hidden_size and head_dim, triton_kernels.py:1127-1158):
+        # hidden 4096 with head_dim 64 takes the general MFMA decode kernel, head_dim 128 the general scalar kernel
+        for tag, hid, nq, nkv, hd in (("h4096_hd64", 4096, 64, 8, 64), ("h4096_hd128", 4096, 32, 8, 128)):
+            od = (nq + 2 * nkv) * hd
+            ws = [torch.empty(od, hid, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(8)]
+            bs = torch.empty(od, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
+            xr = torch.randn(B, hid, generator=g).bfloat16().to(dev)
+            yg = T.YarnParams(head_dim=hd, base=150000.0)
+            bench_kernel(f"qkv_rope_decode_{tag}_B{B}",
+                         lambda i, xr=xr, ws=ws, bs=bs, nq=nq, nkv=nkv, hd=hd, yg=yg: T.qkv_rope_forward(xr, ws[i % 8], bs, nq, nkv, hd, yarn=yg,
+                                                                                                         positions=positions, mode="decode"),
+                         od * hid * 2 + od * 2 + B * (hid * 2 + od * 2), n=96)
+            del ws
         # the first layer of a token step: the gather rides in the same launch (embedding_B8 + norm_qkv_rope_decode_B8 in one)
         qo = (torch.empty(B, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev),
               torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev))

@@ -134,8 +134,11 @@ int tllm_rope_bf16(void* q, void* k, int64_t rows, int n_q_heads, int n_kv_heads
  * k_row_stride = n_ctx*n_kv*hd and kv_slot_stride = n_kv*hd this is the
  * reference's write of the new token into the KV cache.
  *
- * _decode: weight-streaming kernel for few rows (any rows accepted; the
- *   weight is streamed once per 32 rows). Needs no workspace: unlike the
+ * _decode: weight-streaming kernels for few rows (any rows accepted). At the
+ *   gpt-oss shape (hidden 2880, head_dim 64) the weight is read once whatever
+ *   the row count; other shapes (hidden % 32 == 0, head_dim % 16 == 0: an MFMA
+ *   kernel, once per 16 rows; anything else: a scalar kernel) are generic as
+ *   the reference's kernel is. Needs no workspace: unlike the
  *   reference's split-K pair of launches (partials at triton_kernels.py:1200)
  *   the K reduction stays inside a workgroup.
  *   replaces qkv_rope_cache_decode_forward triton_kernels.py:1109-1255 and,

@@ -661,6 +661,25 @@ def test_qkv_offset_form_tables_and_no_rope(gpu, yarn):
         close(v, plain[:, 4608:])
 
 
+@pytest.mark.parametrize("hd,nq,nkv", [(128, 4, 2), (32, 5, 1), (16, 3, 3)])
+@pytest.mark.parametrize("rows", [5, 20])
+def test_qkv_decode_other_head_dims(gpu, hd, nq, nkv, rows):
+    """The general MFMA decode kernel at head dims other than 64 (rotation partners head_dim / 2 apart, head_dim / 16
+    workgroups per head), hidden a multiple of 32 with a K tail; 20 rows = two row chunks, the second ragged."""
+    g = torch.Generator().manual_seed(1000 + hd + rows)
+    hidden = 608
+    x = torch.randn(rows, hidden, generator=g).bfloat16()
+    w = (0.05 * torch.randn((nq + 2 * nkv) * hd, hidden, generator=g)).bfloat16()
+    b = (0.05 * torch.randn((nq + 2 * nkv) * hd, generator=g)).bfloat16()
+    y = T.YarnParams(head_dim=hd, base=10000.0)
+    pos = torch.randint(0, 8192, (rows,), generator=g)
+    qr, kr, vr = O.qkv_rope_ref(x, w, b, pos, nq, nkv, hd, base=10000.0, scaling_factor=1.0)
+    q, k, v = T.qkv_rope_forward(x.to(gpu), w.to(gpu), b.to(gpu), nq, nkv, hd, yarn=y, positions=pos.to(gpu), mode="decode")
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+
+
 def test_qkv_generic_shapes(gpu):
     g = torch.Generator().manual_seed(23)
     hidden, nq, nkv, hd = 100, 3, 1, 32                     # hidden % 32 != 0, head_dim != 64 -> generic kernel

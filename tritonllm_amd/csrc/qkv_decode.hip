@@ -116,23 +116,25 @@ void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& f
 }
 
 // ------------------------------------------------------------------------------------------------
-// MFMA kernel for any hidden % 32 == 0 (head_dim 64). A workgroup owns 16 weight rows of one head --
-// dims [8p, 8p+8) and their partners [32+8p, 32+8p+8) -- and up to 16 activation rows; its wavefronts
+// MFMA kernel for any hidden % 32 == 0 and head_dim % 16 == 0 (the reference's decode kernel is generic over both,
+// triton_kernels.py:1127-1158). A workgroup owns 16 weight rows of one head -- dims [8p, 8p+8) and their partners
+// [half+8p, half+8p+8), half = head_dim / 2 -- and up to 16 activation rows; its wavefronts
 // split K in runs of SPW k32-steps whose loads are all issued before the first multiply.
-// v_mfma_f32_16x16x32_bf16: tile row 4*qd + i is dim 8p + 2*qd + (i & 1), plus 32 when i >= 2, so
+// v_mfma_f32_16x16x32_bf16: tile row 4*qd + i is dim 8p + 2*qd + (i & 1), plus half when i >= 2, so
 // each lane's four accumulators are two complete (lo, hi) pairs.
 template <int NW, int SPW>
 __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   __shared__ float red[NW][4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int head = blockIdx.x >> 2, piece = blockIdx.x & 3;
+  const int half = a.head_dim >> 1, pieces = half >> 3;
+  const int head = blockIdx.x / pieces, piece = blockIdx.x - head * pieces;
   const int64_t row0 = static_cast<int64_t>(blockIdx.y) * 16;
   const int kvec = a.hidden >> 3;       // 16-byte vectors per row
   const int nsteps = a.hidden >> 5;     // MFMA k-steps of 32
   const int m = lane & 15, g = lane >> 4;
 
-  const int dim_a = 8 * piece + 2 * (m >> 2) + (m & 1) + ((m & 2) ? 32 : 0);
-  const bf16x8* wrow = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * 64 + dim_a) * kvec + g;
+  const int dim_a = 8 * piece + 2 * (m >> 2) + (m & 1) + ((m & 2) ? half : 0);
+  const bf16x8* wrow = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * a.head_dim + dim_a) * kvec + g;
   // Lanes past the last activation row re-read a live lane's row (same addresses, no extra traffic);
   // their output column is dropped.
   const int64_t xrow_idx = row0 + m;
@@ -169,13 +171,13 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 
   // the lane holds activation row xrow_idx and dims d0, d0 + 1 (acc[0], acc[1]) with their partners (acc[2], acc[3])
   const int d0 = 8 * piece + 2 * g;
-  const int col = head * 64 + d0;
+  const int col = head * a.head_dim + d0;
   float lo0 = acc[0], lo1 = acc[1], hi0 = acc[2], hi1 = acc[3];
   if (a.bias) {
     lo0 += static_cast<float>(a.bias[col]);
     lo1 += static_cast<float>(a.bias[col + 1]);
-    hi0 += static_cast<float>(a.bias[col + 32]);
-    hi1 += static_cast<float>(a.bias[col + 33]);
+    hi0 += static_cast<float>(a.bias[col + half]);
+    hi1 += static_cast<float>(a.bias[col + half + 1]);
   }
   if (rotate) {
     const int64_t pos = rope_position(ra, xrow_idx);
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   phi[0] = static_cast<bf16>(hi0);
   phi[1] = static_cast<bf16>(hi1);
   *reinterpret_cast<bf16x2*>(out + d0) = plo;
-  *reinterpret_cast<bf16x2*>(out + d0 + 32) = phi;
+  *reinterpret_cast<bf16x2*>(out + d0 + half) = phi;
 }
 
 }  // namespace tllm
@@ -326,8 +328,8 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
   if (rows == 0) return TLLM_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int heads = n_q_heads + 2 * n_kv_heads;
-  const bool mfma_ok = head_dim == 64 && hidden % 32 == 0 && aligned16(x) && aligned16(W);
-  if (mfma_ok && hidden == 2880 && aligned16(b) && static_cast<int64_t>(heads) * 64 * hidden < (1ll << 31)) {
+  const bool mfma_ok = head_dim % 16 == 0 && hidden % 32 == 0 && aligned16(x) && aligned16(W);
+  if (mfma_ok && head_dim == 64 && hidden == 2880 && aligned16(b) && static_cast<int64_t>(heads) * 64 * hidden < (1ll << 31)) {
     // 32-bit element offsets inside W and x are enough here; outputs are written element-wise, any alignment
     return launch_decode_2880("qkv_rope_decode", a, ra, fr, 0, false, rows, heads, st);
   }
@@ -337,7 +339,7 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
   if (mfma_ok && out4) {
     const int64_t chunks = (rows + 15) / 16;
     TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
-    hipLaunchKernelGGL((qkv_decode_kernel<4, 16>), dim3((unsigned)(heads * 4), (unsigned)chunks), dim3(4 * 64), 0, st, a, ra, fr);
+    hipLaunchKernelGGL((qkv_decode_kernel<4, 16>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(4 * 64), 0, st, a, ra, fr);
     return check_launch("qkv_rope_decode");
   }
   launch_qkv_generic(a, ra, fr, st);
