@@ -60,15 +60,6 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   const int kvec = a.hidden >> 3;                             // 16-byte chunks per activation row
   const int nsteps = a.hidden / KS;                           // K steps
 
-  // ---- prologue: the activation rows into LDS (rows past the end repeat the last one; never stored)
-  for (int c = tid; c < XR * kvec; c += UNW * 64) {
-    int r = c / kvec;
-    const int kc = c - r * kvec;
-    const int rs = r < nvalid ? r : nvalid - 1;
-    *reinterpret_cast<bf16x8*>(xs + r * xrow_b + kc * 16) = reinterpret_cast<const bf16x8*>(a.x)[(row0 + rs) * kvec + kc];
-  }
-  __syncthreads();
-
   // ---- this wavefront's tiles: t = gw, gw + G, gw + 2G, ...
   // Wavefront w of workgroup b is number w * gridDim.x + b: when the tiles do not divide evenly (201088 rows are 6284
   // tiles for 4096 wavefronts) the ones that take one tile more are the first wavefronts of EVERY workgroup, not all
@@ -121,6 +112,16 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
 #pragma unroll
   for (int d = 0; d < UD; ++d) issue(d);
 
+  // ---- the activation rows into LDS (rows past the end repeat the last one; never stored), behind the first weight
+  // requests: those take the longest to come back, and the first multiply needs both
+  for (int c = tid; c < XR * kvec; c += UNW * 64) {
+    int r = c / kvec;
+    const int kc = c - r * kvec;
+    const int rs = r < nvalid ? r : nvalid - 1;
+    *reinterpret_cast<bf16x8*>(xs + r * xrow_b + kc * 16) = reinterpret_cast<const bf16x8*>(a.x)[(row0 + rs) * kvec + kc];
+  }
+  __syncthreads();
+
   f32x16 acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
@@ -163,7 +164,6 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        issue(d);                                             // buf[d] is free again: the step UD ahead
         if (++c_step == nsteps) {                             // tile finished: lane owns vocabulary row c_tile*32 + m
           const int v = c_tile * 32 + m;
           float sc = 1.f;
@@ -187,6 +187,11 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
           c_tile += G;
         }
       }
+      // buf[d] is free again: the step UD ahead. Outside the branch above, so that every path through the loop
+      // issues the same loads and the compiler's waits can count on all UD steps being in flight (with the request
+      // inside the branch it has to assume that the steps before this one were skipped, and every UD-th step waited
+      // for everything in flight).
+      issue(d);
     }
   }
 
