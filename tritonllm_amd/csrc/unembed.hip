@@ -65,7 +65,12 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   // tiles for 4096 wavefronts) the ones that take one tile more are the first wavefronts of EVERY workgroup, not all
   // the wavefronts of the first workgroups -- every CU then streams to the end of the launch.
   const int G = gridDim.x * UNW;
-  const int gw = wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x);
+  // The logits of a tile leave as 64-byte runs, half a cache line: neighbouring tiles go to neighbouring wavefronts of
+  // one workgroup, which reach the end of their tiles at about the same time, so that the two halves of a line meet in
+  // the same L2 and leave it as one write (182.8 -> 178.9 us; four or eight neighbouring tiles per workgroup are slower,
+  // 184 / 194 us: their reads then pull on the same memory pages). The argmax form stores nothing and keeps the plain deal.
+  constexpr int ADJ = ARGMAX ? 1 : 2;
+  const int gw = ADJ * ((wave / ADJ) * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)) + (wave % ADJ);
   const int ntiles = (a.vocab + 31) >> 5;
   const int my_tiles = gw < ntiles ? (ntiles - gw + G - 1) / G : 0;
   const int total = my_tiles * nsteps;                        // steps of the whole stream
