@@ -897,6 +897,34 @@ def _argmax_ok(ids, logits_ref):
     assert torch.equal(ids[clear], top2.indices[clear, 0])
 
 
+def test_unembedding_argmax_ties_negative_maxima_and_zeros(gpu):
+    """The winner among the per-wavefront candidates is picked through one sortable key per candidate: exact ties (the
+    same vocabulary row planted in tiles that different wavefronts and workgroups own) must go to the lowest index, a
+    row whose logits are all negative must still find its maximum, and a row of zeros (every logit +-0) must return
+    token 0."""
+    g = torch.Generator().manual_seed(4242)
+    vocab = 140000                                            # 4375 tiles: more than one per wavefront
+    x = torch.randn(4, 2880, generator=g).bfloat16()
+    x[1] = -x[0]
+    x[2] = 0
+    w = (0.02 * torch.randn(vocab, 2880, generator=g)).bfloat16()
+    planted = [131071, 777, 65536, 40000]
+    for i in planted:
+        w[i] = x[0]                                           # logit |x0|^2 for row 0, the most negative one for row 1
+    x[3] = x[3].abs()
+    ids = T.unembedding_decode_argmax_forward(x.view(4, 1, 2880).to(gpu), w.to(gpu)).cpu().long()
+    want = O.linear_ref(x, w, None)
+    assert ids[0].item() == min(planted)
+    assert ids[2].item() == 0
+    _argmax_ok(ids[[1, 3]], want[[1, 3]])
+    # all logits of a row negative: w = -|w|, x >= 0
+    wn = -w.abs()
+    idn = T.unembedding_decode_argmax_forward(x[3:4].view(1, 1, 2880).to(gpu), wn.to(gpu))
+    wantn = O.linear_ref(x[3:4], wn, None)
+    assert wantn.max() < 0
+    _argmax_ok(idn, wantn)
+
+
 @pytest.mark.parametrize("rows,vocab", [(1, 4096), (8, 5000), (13, 4097), (16, 20000), (20, 3001)])
 @pytest.mark.parametrize("fp8", [False, True])
 def test_unembedding_decode_parity_small_vocab(gpu, rows, vocab, fp8):

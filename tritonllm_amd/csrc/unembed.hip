@@ -225,39 +225,65 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   }
 }
 
-// One workgroup per batch row: the winner among the per-wavefront candidates. Lowest index wins a tie.
-__global__ __launch_bounds__(256) void unembed_argmax_reduce_kernel(const float* part_max, const int* part_idx, int* token_ids, int n_part,
-                                                                    int xr) {
-  __shared__ float s_v[256];
-  __shared__ int s_i[256];
-  const int row = blockIdx.x;
+// One workgroup per batch row: the winner among the per-wavefront candidates (at most 4096). Lowest index wins a tie.
+// A candidate becomes one 64-bit key -- the value's bits made monotonic in the upper word, the complement of its index
+// in the lower -- so that the winner is a plain maximum. Every thread requests its (up to four) candidates before it
+// looks at any; wavefront maximum through DPP operands and scalar lane reads, sixteen wavefront results through LDS.
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k) {
+  auto dpp = [](unsigned x, auto ctrl) {
+    return static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  auto step = [&](auto ctrl) {
+    const unsigned long long o = (static_cast<unsigned long long>(dpp(static_cast<unsigned>(k >> 32), ctrl)) << 32) | dpp(static_cast<unsigned>(k), ctrl);
+    k = o > k ? o : k;
+  };
+  step(std::integral_constant<int, 0xB1>{});               // quad_perm [1, 0, 3, 2]
+  step(std::integral_constant<int, 0x4E>{});               // quad_perm [2, 3, 0, 1]
+  step(std::integral_constant<int, 0x141>{});              // row_half_mirror
+  step(std::integral_constant<int, 0x140>{});              // row_mirror: every lane of a row of 16 now holds the row's maximum
+  unsigned long long best = 0;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(k >> 32), 16 * r));
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(k), 16 * r));
+    const unsigned long long o = (static_cast<unsigned long long>(hi) << 32) | lo;
+    best = o > best ? o : best;
+  }
+  return best;
+}
+
+constexpr int kArgmaxReduceThreads = 1024;
+
+__global__ __launch_bounds__(kArgmaxReduceThreads) void unembed_argmax_reduce_kernel(const float* part_max, const int* part_idx, int* token_ids,
+                                                                                     int n_part, int xr) {
+  __shared__ unsigned long long s_k[kArgmaxReduceThreads / 64];
+  const int row = blockIdx.x, tid = threadIdx.x;
   const int chunk = row / xr, brow = row - chunk * xr;
-  float bv = -3.0e38f;
-  int bi = 0x7fffffff;
-  for (int p = threadIdx.x; p < n_part; p += 256) {
-    const int64_t slot = (static_cast<int64_t>(chunk) * n_part + p) * xr + brow;
-    const float v = part_max[slot];
-    const int i = part_idx[slot];
-    if (v > bv || (v == bv && i < bi)) {
-      bv = v;
-      bi = i;
-    }
+  constexpr int PER = 4;                                    // n_part <= 4096
+  float v[PER];
+  int idx[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int p = tid + j * kArgmaxReduceThreads;
+    const int64_t slot = (static_cast<int64_t>(chunk) * n_part + (p < n_part ? p : n_part - 1)) * xr + brow;
+    v[j] = part_max[slot];
+    idx[j] = part_idx[slot];
   }
-  s_v[threadIdx.x] = bv;
-  s_i[threadIdx.x] = bi;
+  unsigned long long k = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const unsigned b = __float_as_uint(v[j] + 0.0f);        // -0 + 0 = +0: the two zeros compare equal, so they must make one key
+    const unsigned mono = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    const unsigned long long o = (static_cast<unsigned long long>(mono) << 32) | static_cast<unsigned>(~idx[j]);
+    k = (tid + j * kArgmaxReduceThreads < n_part && o > k) ? o : k;
+  }
+  k = wave_max_u64(k);
+  if ((tid & 63) == 0) s_k[tid >> 6] = k;
   __syncthreads();
-  for (int o = 128; o > 0; o >>= 1) {
-    if (threadIdx.x < o) {
-      const float v = s_v[threadIdx.x + o];
-      const int i = s_i[threadIdx.x + o];
-      if (v > s_v[threadIdx.x] || (v == s_v[threadIdx.x] && i < s_i[threadIdx.x])) {
-        s_v[threadIdx.x] = v;
-        s_i[threadIdx.x] = i;
-      }
-    }
-    __syncthreads();
+  if (tid < 64) {
+    k = wave_max_u64(tid < kArgmaxReduceThreads / 64 ? s_k[tid] : 0ull);
+    if (tid == 0) token_ids[row] = static_cast<int>(~static_cast<unsigned>(k));
   }
-  if (threadIdx.x == 0) token_ids[row] = s_i[0];
 }
 
 }  // namespace tllm
@@ -364,7 +390,8 @@ static int unembed_argmax_run(const char* who, const void* x, const void* W, con
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc = unembed_launch<true>(who, a, w_scale != nullptr, st);
   if (rc != TLLM_OK) return rc;
-  hipLaunchKernelGGL(unembed_argmax_reduce_kernel, dim3((unsigned)rows), dim3(256), 0, st, a.part_max, a.part_idx, token_ids,
+  static_assert(kUnembedGrid * 16 <= 4 * kArgmaxReduceThreads, "the reduce kernel takes up to four candidates per thread");
+  hipLaunchKernelGGL(unembed_argmax_reduce_kernel, dim3((unsigned)rows), dim3(kArgmaxReduceThreads), 0, st, a.part_max, a.part_idx, token_ids,
                      kUnembedGrid * unembed_nw(xr, w_scale != nullptr), xr);
   return check_launch(who);
 }
