@@ -60,19 +60,28 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   const int kvec = a.hidden >> 3;                             // 16-byte chunks per activation row
   const int nsteps = a.hidden / KS;                           // K steps
 
-  // ---- this wavefront's tiles: t = gw, gw + G, gw + 2G, ...
-  // Wavefront w of workgroup b is number w * gridDim.x + b: when the tiles do not divide evenly (201088 rows are 6284
-  // tiles for 4096 wavefronts) the ones that take one tile more are the first wavefronts of EVERY workgroup, not all
-  // the wavefronts of the first workgroups -- every CU then streams to the end of the launch.
+  // ---- this wavefront's tiles, one per round of G = all wavefronts of the launch. Within a round the tiles go
+  // wavefront index first, workgroup second: when the tiles do not divide evenly (201088 rows are 6284 tiles for 4096
+  // wavefronts) the ones that take one tile more are the first wavefronts of EVERY workgroup, not all the wavefronts of
+  // the first workgroups -- every CU then streams to the end of the launch.
   const int G = gridDim.x * UNW;
   // The logits of a tile leave as 64-byte runs, half a cache line: neighbouring tiles go to neighbouring wavefronts of
   // one workgroup, which reach the end of their tiles at about the same time, so that the two halves of a line meet in
   // the same L2 and leave it as one write (182.8 -> 178.9 us; four or eight neighbouring tiles per workgroup are slower,
-  // 184 / 194 us: their reads then pull on the same memory pages). The argmax form stores nothing and keeps the plain deal.
-  constexpr int ADJ = ARGMAX ? 1 : 2;
-  const int gw = ADJ * ((wave / ADJ) * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)) + (wave % ADJ);
+  // 184 / 194 us: their reads then pull on the same memory pages). A pair of wavefronts (2q, 2q + 1) of all workgroups
+  // covers a row of 2 * gridDim.x tiles per round; a row that the vocabulary does not fill is dealt one tile per
+  // workgroup instead, so that no CU takes two tiles more than another. The argmax form stores nothing and deals singly.
+  constexpr bool ADJ2 = !ARGMAX;
+  const int nwg = static_cast<int>(gridDim.x), wg = static_cast<int>(blockIdx.x);
   const int ntiles = (a.vocab + 31) >> 5;
-  const int my_tiles = gw < ntiles ? (ntiles - gw + G - 1) / G : 0;
+  auto tile_of = [&](int round) {
+    const int base = round * G + (wave >> 1) * (2 * nwg);     // first tile of this wavefront pair's row
+    if (ADJ2 && ntiles - base >= 2 * nwg) return base + 2 * wg + (wave & 1);
+    return base + (wave & 1) * nwg + wg;
+  };
+  const int full_rounds = ntiles / G;                         // rounds in which every wavefront has a tile
+  const int my_tiles = full_rounds + (tile_of(full_rounds) < ntiles ? 1 : 0);
+  const int gw = wave * nwg + wg;                             // this wavefront's number (its slot in the argmax workspace)
   const int total = my_tiles * nsteps;                        // steps of the whole stream
 
   // One load instruction moves 1 KB; the 32 x (KS elements) block of a step is dealt to the lanes as 16-byte
@@ -91,7 +100,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
 
   bf16x8 buf[UD][LPS];
   const bf16x8* lp[LPS];                                      // load cursor: row bases of the tile being requested
-  int l_tile = gw, l_step = 0, l_count = 0;
+  int l_round = 0, l_tile = tile_of(0), l_step = 0, l_count = 0;
 #pragma unroll
   for (int i = 0; i < LPS; ++i) lp[i] = row_base(my_tiles > 0 ? l_tile : 0, i);
   // Unconditional on purpose (a load under a branch makes the compiler wait for it where the paths join): past
@@ -108,7 +117,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
       ++l_count;
       if (++l_step == nsteps) {
         l_step = 0;
-        l_tile += G;
+        l_tile = tile_of(++l_round);
 #pragma unroll
         for (int i = 0; i < LPS; ++i) lp[i] = row_base(l_tile < ntiles ? l_tile : ntiles - 1, i);
       }
@@ -141,7 +150,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
 
   const unsigned char* xfrag = xs + (m & (XR - 1)) * xrow_b + h * 16;   // activations on M: tile rows >= XR repeat, never stored
   const unsigned char* wfrag = patch + m * UPROW + h * 16;              // vocabulary rows on N
-  int c_tile = gw, c_step = 0;
+  int c_round = 0, c_tile = tile_of(0), c_step = 0;
   for (int g0 = 0; g0 < total; g0 += UD) {
 #pragma unroll
     for (int d = 0; d < UD; ++d) {
@@ -189,7 +198,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
           c_step = 0;
-          c_tile += G;
+          c_tile = tile_of(++c_round);
         }
       }
       // buf[d] is free again: the step UD ahead. Outside the branch above, so that every path through the loop
