@@ -8,6 +8,11 @@ Every step uses the next of 24 distinct layer weight sets (708 MB of QKV weights
 weights come from HBM, not from the 256 MB Infinity Cache. The K timed steps are captured
 in one HIP graph and replayed, which is how the reference runs its decode loop.
 
+Timing: `value` / `ms_per_step` are EXACTLY --steps steps between two synchronisations (median of 31 such samples);
+`steady_state` repeats those samples on a GPU that is already busy. Every other figure (`roofline`, `kernels`,
+`stack24`, `prefill_chains`, `attention_blocks24`) is a steady-state launch-to-launch time: HIP-graph replays timed
+back to back behind an untimed one, at least 8 ms of them (the first ~130 us after a synchronisation run slower).
+
 Prints ONE JSON line: whole-job tokens/s, plus `roofline` for the dominant kernel (the
 decode QKV stream), `cpu_baseline` (the eager bf16 PyTorch restatement of the reference
 chain timed on the host cores) and a `kernels` table with every kernel at its decode and
@@ -113,7 +118,7 @@ def name_of_stamps(fused: bool) -> str:
     return "qkv_decode_r8_kernel<2,false,false>" if fused else "qkv_decode_r8_kernel<0,false,false>"
 
 
-def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg, _lib) -> int:
+def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, steady_graph, weights, biases, scales, table, g, gg, _lib) -> int:
     """One kernel-table entry on its own (a clean target for rocprofv3)."""
     name = args.only
     kind, _, size = name.rpartition("_")
@@ -280,7 +285,7 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         gr = graph_of(fn, 4)
         for _ in range(max(args.steps // 40, 6)):
             gr.replay()
-        sec = min(time_graph(gr) for _ in range(5)) / 4
+        sec = steady_graph(gr) / 4
         print(json.dumps({"kernel": name, "us_per_token_step": round(sec * 1e6, 2), "launches": st.launches_per_step()}))
         return 0
     else:
@@ -291,7 +296,7 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights,
         fn(i)
     gr = graph_of(fn, reps)
     gr.replay()
-    sec = min(time_graph(gr) for _ in range(5)) / reps
+    sec = steady_graph(gr) / reps
     row = {"kernel": name, "us": round(sec * 1e6, 3), "launches_per_replay": reps}
     if nbytes is not None:
         row["GB/s"] = round(nbytes / sec / 1e9, 1)
@@ -382,10 +387,13 @@ def main() -> int:
                 fn(i)
         return gr
 
-    def time_graph(gr, reps: int = 1) -> float:
-        """Seconds for `reps` replays, HIP events on the current stream."""
+    def time_graph(gr, reps: int = 1, lead_in: bool = False) -> float:
+        """Seconds for `reps` replays, HIP events on the current stream. With `lead_in` one untimed replay goes out
+        just before the first event, so that the timed replays start on a GPU that is already busy."""
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
+        if lead_in:
+            gr.replay()
         e0.record()
         for _ in range(reps):
             gr.replay()
@@ -393,8 +401,17 @@ def main() -> int:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3
 
+    def steady_graph(gr, tries: int = 5, target_s: float = 0.008) -> float:
+        """Seconds per replay in steady state: the first ~130 us after a synchronisation run slower (a kernel that is
+        launched on an idle GPU finds its clocks down: the T = 2048 prefill QKV kernel reads 57.8-59.5 us per launch in
+        replays of 48 and 55.2-55.4 us in replays of 240, the unembedding 185 us in replays of 10 and 177 in replays of
+        24), so the replays are timed back to back behind an untimed one, at least `target_s` of them."""
+        one = time_graph(gr)
+        reps = max(1, min(200, int(target_s / max(one, 1e-6)) + 1))
+        return min(time_graph(gr, reps, lead_in=True) for _ in range(tries)) / reps
+
     if args.only:
-        return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, time_graph, weights, biases, scales, table, g, gg, _lib)
+        return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, steady_graph, weights, biases, scales, table, g, gg, _lib)
 
     # ---------------------------------------------------------------- the timed job
     # One sample = EXACTLY --steps steps, captured as one HIP graph and timed with HIP events between two
@@ -417,6 +434,12 @@ def main() -> int:
     elapsed = samples[len(samples) // 2]           # median sample: seconds for --steps steps
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = B * args.steps / elapsed
+    # The same K steps on a GPU that is already busy (an untimed replay of the same graph goes out just before the first
+    # event): what a serving loop sees. `value` stays the figure between two synchronisations, whose first ~130 us find
+    # the GPU's clocks down -- 5 % of a 20-step sample, 0.3 % of a 4800-step one.
+    busy = sorted(time_graph(jobs[(sm * args.steps) % N_LAYERS], 1, lead_in=True) for sm in range(n_samples))[n_samples // 2]
+    steady_state = {"ms_per_step": round(busy / args.steps * 1e3, 6), "tokens/s": round(B * args.steps / busy, 1),
+                    "how": "median over the same samples, each timed right behind an untimed replay of its own graph"}
 
     # ---------------------------------------------------------------- dominant kernel, live
     n_launch = 20 * N_LAYERS
@@ -434,7 +457,7 @@ def main() -> int:
         kernel_name = "qkv_decode_r8_kernel<2,false,false> (RMSNorm + QKV + bias + YaRN RoPE, B=8, weight streamed from HBM)"
     qkv_graph = graph_of(dominant, n_launch)
     qkv_graph.replay()
-    qkv_s = min(time_graph(qkv_graph) for _ in range(5)) / n_launch
+    qkv_s = steady_graph(qkv_graph) / n_launch
     roofline = {
         "kernel": kernel_name,
         "bound": "hbm", "achieved": round(qkv_bytes / qkv_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -460,7 +483,7 @@ def main() -> int:
                 fn(i)
             gr = graph_of(fn, n)
             gr.replay()
-            sec = min(time_graph(gr) for _ in range(5)) / n
+            sec = steady_graph(gr) / n
             row = {"us": round(sec * 1e6, 3)}
             if nbytes is not None:
                 row["GB/s"] = round(nbytes / sec / 1e9, 1)
@@ -578,11 +601,11 @@ def main() -> int:
         # unembedding over the full vocabulary (the embedding table doubles as the [201088, 2880] weight: 1.16 GB per launch)
         for r in (1, 8):
             ux = torch.empty(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
-            bench_kernel(f"unembedding_decode_B{r}", lambda i, ux=ux: T.unembedding_decode_forward(ux, table), bytes_of["unembed"](r), n=10)
+            bench_kernel(f"unembedding_decode_B{r}", lambda i, ux=ux: T.unembedding_decode_forward(ux, table), bytes_of["unembed"](r), n=24)
             bench_kernel(f"unembedding_argmax_B{r}", lambda i, ux=ux: T.unembedding_decode_argmax_forward(ux, table),
-                         bytes_of["unembed_argmax"](r), n=10)
+                         bytes_of["unembed_argmax"](r), n=24)
         uw8, uws = T.quantize_fp8_rows(table)
-        bench_kernel("unembedding_decode_w8_B8", lambda i, ux=ux: T.unembedding_decode_forward(ux, uw8, uws), bytes_of["unembed_w8"](8), n=10)
+        bench_kernel("unembedding_decode_w8_B8", lambda i, ux=ux: T.unembedding_decode_forward(ux, uw8, uws), bytes_of["unembed_w8"](8), n=24)
         del uw8, uws
         # stand-alone rotary at the decode size (one token per batch row, independent positions)
         rope_off = torch.zeros(1, dtype=torch.int64, device=dev)
@@ -649,7 +672,7 @@ def main() -> int:
             token_step(0)
             gr = graph_of(token_step, 4)
             gr.replay()
-            sec = min(time_graph(gr) for _ in range(5)) / 4
+            sec = steady_graph(gr) / 4
             stack[f"B{r}"] = {"us_per_token_step": round(sec * 1e6, 2), "tokens/s": round(r / sec, 1), "launches": st.launches_per_step(),
                               "weight_GB/s": round(N_LAYERS * QKV_DIM * HIDDEN * 2 / sec / 1e9, 1)}
 
@@ -679,7 +702,7 @@ def main() -> int:
             attn_step(0)
             gr = graph_of(attn_step, 2)
             gr.replay()
-            sec = min(time_graph(gr) for _ in range(5)) / 2
+            sec = steady_graph(gr) / 2
             attn_stack[f"B{r}_ctx{ctx}"] = {"us_per_token_step": round(sec * 1e6, 2), "us_per_layer": round(sec * 1e6 / N_LAYERS, 2),
                                             "tokens/s": round(r / sec, 1)}
             del ck, cv
@@ -711,7 +734,7 @@ def main() -> int:
             chain(0)
             gr = graph_of(chain, 24)
             gr.replay()
-            sec = min(time_graph(gr) for _ in range(5)) / 24
+            sec = steady_graph(gr) / 24
             prefill_chains[f"T{tt}"] = {"chain": ("gather/RMSNorm (one launch)" if with_gather else "RMSNorm") + " + QKV/bias/RoPE" + (" + SwiGLU[32768,5760]" if swiglu_rows else ""),
                                         "us": round(sec * 1e6, 2), "tokens/s": round(tt / sec, 1)}
             del xp, tn, qo, sx, so
@@ -740,7 +763,7 @@ def main() -> int:
             prompt_step(0)
             gr = graph_of(prompt_step, 1)
             gr.replay()
-            sec = min(time_graph(gr) for _ in range(3))
+            sec = steady_graph(gr, tries=3)
             attn_stack[f"prompt_T{tt}"] = {"us_per_prompt": round(sec * 1e6, 1), "us_per_layer": round(sec * 1e6 / N_LAYERS, 2),
                                            "tokens/s": round(tt / sec, 1)}
             del xp, tn, qb, ck, cv
@@ -807,7 +830,7 @@ def main() -> int:
                    "batch": B, "layers_rotated": N_LAYERS,
                    "rmsnorm": "own launch" if args.unfused else "inside the QKV decode kernel",
                    "gather": "inside the QKV decode kernel (x = table rows)" if args.fuse_gather else "own launch (x ~ N(0,1) as the configuration states)"},
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "prefill_chains": prefill_chains, "attention_blocks24": attn_stack,
+        "steady_state": steady_state, "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels, "stack24": stack, "prefill_chains": prefill_chains, "attention_blocks24": attn_stack,
         "samples": n_samples, "sample_ms_min_median_max": [round(samples[0] * 1e3, 4), round(elapsed * 1e3, 4), round(samples[-1] * 1e3, 4)],
         "wall_s_all_samples": round(wall, 4),
     }
