@@ -38,6 +38,7 @@ struct UnembedArgs {
   int* part_idx;
   int64_t rows;
   int hidden, vocab;
+  int pair_stores;        // the logits rows allow 4-byte stores at even columns
 };
 
 __host__ __device__ constexpr int unembed_patch(int ks) { return 32 * (ks * 2 + 16); }   // wavefront patch: 32 rows of KS bf16 + padding
@@ -46,8 +47,16 @@ __host__ __device__ constexpr int unembed_xrow(int hidden) { return hidden * 2 +
 
 // UNW wavefronts per workgroup: sixteen where LDS allows (up to 8 batch rows: measured 6.3 against 6.0 TB/s with eight),
 // eight with 16 batch rows resident.
-template <int XR, int UNW, int KS, int UD, bool W8, bool ARGMAX>
+// SR (fp8 weight, even vocabulary): a row of fp8 is hidden bytes, 22.5 cache lines at gpt-oss's width, so that row pieces
+// never line up with cache lines; two neighbouring rows together are 2 * hidden bytes -- whole lines. The weight is then
+// read as [vocab / 2, 2 * hidden]: a tile is 32 such pairs (64 vocabulary rows), a step is 128 bytes = one aligned line of
+// every pair (the bf16 kernel's pattern exactly, streamed with the nontemporal hint), and the bytes of a step belong to
+// the pair's first row while they lie below `hidden` and to its second row from there on -- two accumulator tiles, the
+// K offset into the activations chosen per MFMA. A lane ends up with the logits of rows 2p and 2p + 1: one 4-byte store,
+// whole 128-byte lines per wavefront. (A bare read in this pattern: 86 us for the 580 MB; in 192-byte row pieces: 96-98.)
+template <int XR, int UNW, int KS, int UD, bool W8, bool ARGMAX, bool SR = false>
 __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
+  static_assert(!SR || (W8 && KS == 128), "pairs of rows: fp8 weight, 128 bytes per pair and step");
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 31, h = lane >> 5;
@@ -58,7 +67,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
   const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
   const int kvec = a.hidden >> 3;                             // 16-byte chunks per activation row
-  const int nsteps = a.hidden / KS;                           // K steps
+  const int nsteps = SR ? 2 * a.hidden / KS : a.hidden / KS;  // K steps of a tile
 
   // ---- this wavefront's tiles, one per round of G = all wavefronts of the launch. Within a round the tiles go
   // wavefront index first, workgroup second: when the tiles do not divide evenly (201088 rows are 6284 tiles for 4096
@@ -71,9 +80,10 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   // 184 / 194 us: their reads then pull on the same memory pages). A pair of wavefronts (2q, 2q + 1) of all workgroups
   // covers a row of 2 * gridDim.x tiles per round; a row that the vocabulary does not fill is dealt one tile per
   // workgroup instead, so that no CU takes two tiles more than another. The argmax form stores nothing and deals singly.
-  constexpr bool ADJ2 = !ARGMAX;
+  constexpr bool ADJ2 = !ARGMAX && !SR;                       // (pairs of rows leave as whole lines anyway)
   const int nwg = static_cast<int>(gridDim.x), wg = static_cast<int>(blockIdx.x);
-  const int ntiles = (a.vocab + 31) >> 5;
+  const int nunits = SR ? a.vocab >> 1 : a.vocab;            // rows (pairs of rows) of the weight as it is streamed
+  const int ntiles = (nunits + 31) >> 5;
   auto tile_of = [&](int round) {
     const int base = round * G + (wave >> 1) * (2 * nwg);     // first tile of this wavefront pair's row
     if (ADJ2 && ntiles - base >= 2 * nwg) return base + 2 * wg + (wave & 1);
@@ -89,12 +99,12 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   // 128-byte line; KS = 192: 24 lanes per 384-byte run).
   constexpr int CPS = (W8 ? KS : KS * 2) / 16;                // 16-byte chunks per row per step, as the weight lies in memory
   constexpr int LPS = 32 * CPS / 64;                          // load instructions per step
-  const int64_t wrow_vec = W8 ? (a.hidden >> 4) : (a.hidden >> 3);   // 16-byte chunks per weight row
+  const int64_t wrow_vec = (W8 && !SR) ? (a.hidden >> 4) : (a.hidden >> 3);   // 16-byte chunks per weight row (pair of rows)
   const bf16x8* wv = reinterpret_cast<const bf16x8*>(a.W);
   auto row_base = [&](int tile, int i) -> const bf16x8* {    // first chunk this lane fetches of load i in tile `tile`
     const int c = i * 64 + lane;
     int v = tile * 32 + c / CPS;
-    v = v < a.vocab ? v : a.vocab - 1;                        // ragged last tile: repeat the last row (never stored)
+    v = v < nunits ? v : nunits - 1;                          // ragged last tile: repeat the last row (never stored)
     return wv + static_cast<int64_t>(v) * wrow_vec + (c % CPS);
   };
 
@@ -110,7 +120,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
     for (int i = 0; i < LPS; ++i) {
       // fp8 rows are 22.5 lines long, so a step's row pieces share lines with the next step's: read through the cache
       // they are fetched from HBM once (FETCH_SIZE 601 MB for 580 MB of weight; with the streaming hint 730 MB)
-      if constexpr (W8) buf[d][i] = lp[i][l_step * CPS];
+      if constexpr (W8 && !SR) buf[d][i] = lp[i][l_step * CPS];
       else buf[d][i] = __builtin_nontemporal_load(lp[i] + l_step * CPS);
     }
     if (l_count + 1 < total) {
@@ -136,9 +146,9 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   }
   __syncthreads();
 
-  f32x16 acc;
+  f32x16 acc, acc2;                                           // acc2 (SR): the pair's second row
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
   constexpr int NB = XR / 2;                                  // accumulator registers that carry batch rows: row(v) = 8*(v>>2) + 4*h + (v&3)
   float best[NB];
   int best_i[NB];
@@ -170,15 +180,82 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        if constexpr (SR) {
+          const int kb0 = c_step * KS;                        // the step's first byte inside the pair = K of the first row
+          // One branch per step, not per MFMA: inside a case the sixteen fragment reads go out together.
+          if (kb0 + KS <= a.hidden) {                         // uniform: the whole step belongs to the first row
 #pragma unroll
-        for (int t = 0; t < KS / 16; ++t) {
-          const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + c_step * (KS * 2) + t * 32);
-          const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+            for (int t = 0; t < KS / 16; ++t) {
+              const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + (kb0 + 16 * t) * 2);
+              const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+            }
+          } else if (kb0 >= a.hidden) {                       // ... to the second row
+#pragma unroll
+            for (int t = 0; t < KS / 16; ++t) {
+              const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + (kb0 - a.hidden + 16 * t) * 2);
+              const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
+              acc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc2, 0, 0, 0);
+            }
+          } else {                                            // the step in which the first row ends (hidden is a multiple of 16: no MFMA straddles)
+#pragma unroll
+            for (int t = 0; t < KS / 16; ++t) {
+              const int kb = kb0 + 16 * t;
+              const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
+              if (kb < a.hidden) {
+                const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + kb * 2);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+              } else {
+                const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + (kb - a.hidden) * 2);
+                acc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc2, 0, 0, 0);
+              }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int t = 0; t < KS / 16; ++t) {
+            const bf16x8 fa = *reinterpret_cast<const bf16x8*>(xfrag + c_step * (KS * 2) + t * 32);
+            const bf16x8 fb = *reinterpret_cast<const bf16x8*>(wfrag + t * 32);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (++c_step == nsteps) {                             // tile finished: lane owns vocabulary row c_tile*32 + m
+        if (SR && ++c_step == nsteps) {                       // tile finished: lane owns vocabulary rows 2 p and 2 p + 1, p = c_tile*32 + m
+          const int v0 = 2 * (c_tile * 32 + m), v1 = v0 + 1;  // the vocabulary is even here: both are inside it, or neither
+          const float sc0 = a.w_scale[v0 < a.vocab ? v0 : a.vocab - 2], sc1 = a.w_scale[v1 < a.vocab ? v1 : a.vocab - 1];
+#pragma unroll
+          for (int r = 0; r < NB; ++r) {
+            const int brow = 8 * (r >> 2) + 4 * h + (r & 3);
+            const float val0 = acc[r] * sc0, val1 = acc2[r] * sc1;
+            if constexpr (ARGMAX) {
+              if (v0 < a.vocab && val0 > best[r]) {           // ascending order: '>' keeps the lowest index
+                best[r] = val0;
+                best_i[r] = v0;
+              }
+              if (v0 < a.vocab && val1 > best[r]) {
+                best[r] = val1;
+                best_i[r] = v1;
+              }
+            } else if (v0 < a.vocab && brow < nvalid) {
+              bf16* lrow = a.logits + (row0 + brow) * a.ld + v0;
+              if (a.pair_stores) {
+                bf16x2 pr;
+                pr[0] = static_cast<bf16>(val0);
+                pr[1] = static_cast<bf16>(val1);
+                *reinterpret_cast<bf16x2*>(lrow) = pr;
+              } else {
+                lrow[0] = static_cast<bf16>(val0);
+                lrow[1] = static_cast<bf16>(val1);
+              }
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.f;
+          c_step = 0;
+          c_tile = tile_of(++c_round);
+        }
+        if (!SR && ++c_step == nsteps) {                      // tile finished: lane owns vocabulary row c_tile*32 + m
           const int v = c_tile * 32 + m;
           float sc = 1.f;
           if constexpr (W8) sc = a.w_scale[v < a.vocab ? v : a.vocab - 1];
@@ -336,16 +413,20 @@ int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_
 template <bool ARGMAX>
 int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t st) {
   const int xr = unembed_xr(a.rows, w8, a.hidden);
-  const size_t smem = unembed_smem(xr, w8, a.hidden);
+  // fp8 weight, up to 8 rows, even vocabulary: pairs of rows (whole cache lines), eight wavefronts, 128 bytes per pair and step
+  const size_t smem_pairs = static_cast<size_t>(8) * unembed_xrow(a.hidden) + 8 * unembed_patch(128);
+  const bool pairs = w8 && xr == 8 && a.vocab % 2 == 0 && smem_pairs <= 160 * 1024;
+  const size_t smem = pairs ? smem_pairs : unembed_smem(xr, w8, a.hidden);
   const dim3 grid(kUnembedGrid, (unsigned)((a.rows + xr - 1) / xr));
-#define TLLM_UNEMBED(XR, NW, KS, UD, W8F)                                                                                   \
+#define TLLM_UNEMBED(XR, NW, KS, UD, W8F, ...)                                                                              \
   do {                                                                                                                      \
-    auto kern = unembed_kernel<XR, NW, KS, UD, W8F, ARGMAX>;                                                                \
+    auto kern = unembed_kernel<XR, NW, KS, UD, W8F, ARGMAX, ##__VA_ARGS__>;                                                 \
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "%s: cannot raise LDS limit: %s", who, hipGetErrorString(e));              \
     hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, a);                                                             \
   } while (0)
-  if (xr == 8 && !w8) TLLM_UNEMBED(8, 16, 64, 4, false);
+  if (pairs) TLLM_UNEMBED(8, 8, 128, 2, true, true);          // steps in flight 1 / 2 / 3 / 4: 122 / 99 / 105 / 107 us; 12 wavefronts x 3: 103, 10 x 2: 103, 6 x 2: 115
+  else if (xr == 8 && !w8) TLLM_UNEMBED(8, 16, 64, 4, false);
   else if (xr == 8 && unembed_ks(8, true, a.hidden) == 192) TLLM_UNEMBED(8, 8, 192, 2, true);
   else if (xr == 8) TLLM_UNEMBED(8, 8, 64, 4, true);
   else if (w8) TLLM_UNEMBED(16, 8, 64, 4, true);
@@ -369,6 +450,7 @@ extern "C" int tllm_unembedding_decode_bf16(const void* x, const void* W, const 
   a.rows = rows;
   a.hidden = (int)hidden;
   a.vocab = (int)vocab;
+  a.pair_stores = reinterpret_cast<uintptr_t>(logits) % 4 == 0 && logits_row_stride % 2 == 0;
   return unembed_launch<false>("unembedding_decode", a, w_scale != nullptr, static_cast<hipStream_t>(stream));
 }
 
