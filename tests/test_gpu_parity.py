@@ -897,6 +897,28 @@ def _argmax_ok(ids, logits_ref):
     assert torch.equal(ids[clear], top2.indices[clear, 0])
 
 
+def test_unembedding_fp8_logits_rows_that_allow_2_byte_stores_only(gpu):
+    """The fp8 kernel for an even vocabulary stores the logits of two neighbouring vocabulary rows as one 4-byte pair
+    where the logits buffer allows it; here it does not (odd row stride, first element 2 bytes into a word)."""
+    from tritonllm_amd._lib import lib
+    g = torch.Generator().manual_seed(8642)
+    rows, vocab = 5, 3000
+    x = torch.randn(rows, 2880, generator=g).bfloat16()
+    w = (0.02 * torch.randn(vocab, 2880, generator=g)).bfloat16()
+    w8, ws = T.quantize_fp8_rows(w.to(gpu))
+    want = O.linear_ref(x, O.dequant_fp8_ref(w8.cpu(), ws.cpu()), None)
+    ld = vocab + 3
+    buf = torch.full((rows * ld + 8,), float("nan"), dtype=torch.bfloat16, device=gpu)
+    xg = x.to(gpu)
+    rc = lib().tllm_unembedding_decode_bf16(xg.data_ptr(), w8.data_ptr(), ws.data_ptr(), buf.data_ptr() + 2, ld, rows, 2880, vocab,
+                                            torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = buf[1:1 + rows * ld].view(rows, ld)
+    close(got[:, :vocab], want)
+    assert torch.isnan(got[:, vocab:].float()).all() and torch.isnan(buf[0].float())   # nothing outside the rows was written
+
+
 def test_unembedding_argmax_ties_negative_maxima_and_zeros(gpu):
     """The winner among the per-wavefront candidates is picked through one sortable key per candidate: exact ties (the
     same vocabulary row planted in tiles that different wavefronts and workgroups own) must go to the lowest index, a

@@ -21,7 +21,8 @@
 // winner. Ties go to the lowest index.
 //
 // W8: fp8 (OCP e4m3) weight with one fp32 scale per vocabulary row (triton_kernels.py:261-268): widened to bf16
-// on the way into the patch, the row scale multiplies the finished sum. Half the bytes.
+// on the way into the patch, the row scale multiplies the finished sum. Half the bytes. With an even vocabulary the
+// weight is streamed as pairs of rows (SR, below), whose bytes are whole cache lines.
 #include <mutex>
 
 #include "common.h"
@@ -383,7 +384,8 @@ int unembed_xr_most(int64_t rows) { return rows <= 8 ? 8 : 16; }
 
 // (wavefronts, K step, steps in flight), measured at B = 8 on the full vocabulary:
 //   bf16, up to 8 rows : 16 wavefronts, K step 64 (whole 128-byte lines), 4 in flight   185 us (8 wavefronts: 194)
-//   fp8,  up to 8 rows :  8 wavefronts, K step 192, 2 in flight                          133 us (16 x 64 x 4: 167)
+//   fp8,  up to 8 rows :  even vocabulary: pairs of rows, 8 wavefronts, 128 bytes per pair and step, 2 in flight   99 us
+//                         odd vocabulary: 8 wavefronts, K step 192, 2 in flight           113 us (16 x 64 x 4: 124)
 //   16 rows            :  8 wavefronts (LDS holds the 16 activation rows), K step 64, 4 in flight
 // K steps that split 128-byte lines (96 elements of bf16, 32) cost 25-50 %.
 int unembed_nw(int xr, bool w8) { return (xr == 8 && !w8) ? 16 : 8; }
