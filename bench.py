@@ -124,11 +124,25 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, steady_graph, weight
     kind, _, size = name.rpartition("_")
     n = int(size[1:])
     flops = nbytes = None
+    if kind in ("qkv_rope_decode_h4096_hd64", "qkv_rope_decode_h4096_hd128"):
+        # shapes other than gpt-oss's: the general decode kernels (8 rotating weights of [6144, 4096])
+        nq, nkv, hd = (64, 8, 64) if kind.endswith("hd64") else (32, 8, 128)
+        od = (nq + 2 * nkv) * hd
+        ws = [torch.empty(od, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(8)]
+        bs = torch.empty(od, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
+        xr = torch.randn(n, 4096, generator=g).bfloat16().to(dev)
+        pr = torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
+        yg = T.YarnParams(head_dim=hd, base=150000.0)
+        fn = lambda i: T.qkv_rope_forward(xr, ws[i % 8], bs, nq, nkv, hd, yarn=yg, positions=pr, mode="decode")
+        nbytes = od * 4096 * 2 + od * 2 + n * (4096 * 2 + od * 2)
+        kind = "generic"
     tables = kind == "qkv_rope_prefill_tables"           # cos / sin from the precomputed tables, as the reference passes them
     if tables:
         kind = "qkv_rope_prefill"
         rope_t = T.RotaryEmbedding(HD, 150000, torch.float32, initial_context_length=4096, scaling_factor=32.0, device=dev)
-    if kind in ("qkv_rope_prefill", "qkv_rope_decode", "norm_qkv_rope_decode", "qkv_rope_decode_w8", "norm_qkv_rope_decode_w8"):
+    if kind == "generic":
+        pass
+    elif kind in ("qkv_rope_prefill", "qkv_rope_decode", "norm_qkv_rope_decode", "qkv_rope_decode_w8", "norm_qkv_rope_decode_w8"):
         xp = torch.empty(n, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         pp = torch.arange(n, dtype=torch.int64, device=dev) if kind.endswith("prefill") else \
             torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
