@@ -401,12 +401,12 @@ def main() -> int:
                 fn(i)
         return gr
 
-    def time_graph(gr, reps: int = 1, lead_in: bool = False) -> float:
-        """Seconds for `reps` replays, HIP events on the current stream. With `lead_in` one untimed replay goes out
-        just before the first event, so that the timed replays start on a GPU that is already busy."""
+    def time_graph(gr, reps: int = 1, lead_in: int = 0) -> float:
+        """Seconds for `reps` replays, HIP events on the current stream. `lead_in` untimed replays go out just before
+        the first event, so that the timed replays start on a GPU that is already busy."""
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        if lead_in:
+        for _ in range(int(lead_in)):
             gr.replay()
         e0.record()
         for _ in range(reps):
@@ -422,7 +422,7 @@ def main() -> int:
         24), so the replays are timed back to back behind an untimed one, at least `target_s` of them."""
         one = time_graph(gr)
         reps = max(1, min(200, int(target_s / max(one, 1e-6)) + 1))
-        return min(time_graph(gr, reps, lead_in=True) for _ in range(tries)) / reps
+        return min(time_graph(gr, reps, lead_in=max(1, reps // 4)) for _ in range(tries)) / reps
 
     if args.only:
         return run_only(args, T, torch, dev, yarn, bytes_of, graph_of, steady_graph, weights, biases, scales, table, g, gg, _lib)
@@ -451,9 +451,10 @@ def main() -> int:
     # The same K steps on a GPU that is already busy (an untimed replay of the same graph goes out just before the first
     # event): what a serving loop sees. `value` stays the figure between two synchronisations, whose first ~130 us find
     # the GPU's clocks down -- 5 % of a 20-step sample, 0.3 % of a 4800-step one.
-    busy = sorted(time_graph(jobs[(sm * args.steps) % N_LAYERS], 1, lead_in=True) for sm in range(n_samples))[n_samples // 2]
+    lead = max(1, int(0.002 / elapsed) + 1)                  # at least 2 ms of untimed replays before the first event
+    busy = sorted(time_graph(jobs[(sm * args.steps) % N_LAYERS], 1, lead_in=lead) for sm in range(n_samples))[n_samples // 2]
     steady_state = {"ms_per_step": round(busy / args.steps * 1e3, 6), "tokens/s": round(B * args.steps / busy, 1),
-                    "how": "median over the same samples, each timed right behind an untimed replay of its own graph"}
+                    "how": f"median over the same samples, each timed right behind {lead} untimed replay(s) of its own graph (>= 2 ms)"}
 
     # ---------------------------------------------------------------- dominant kernel, live
     n_launch = 20 * N_LAYERS
