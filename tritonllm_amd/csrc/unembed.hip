@@ -4,11 +4,11 @@
 // twins :200-302 and :404-512). With W = [201088, 2880] bf16 this is a 1.16 GB stream per token -- the largest
 // single read of a decode step -- so the kernel is built around keeping HBM busy and nothing else:
 //
-//   * one workgroup of sixteen (eight) wavefronts per CU, alive for the whole launch; the few activation rows sit in LDS,
+//   * one workgroup of ten (eight) wavefronts per CU, alive for the whole launch; the few activation rows sit in LDS,
 //     read once per workgroup;
 //   * a wavefront owns whole 32-row vocabulary tiles (dealt round-robin, so every CU gets the same share +-1) and
 //     walks K in steps of 64: four 1 KB loads per step, each lane fetching 16 bytes so that eight lanes cover one
-//     128-byte line of one row (fully coalesced), four steps (16 KB per wavefront, 128 KB per CU) always in
+//     128-byte line of one row (fully coalesced), three steps (12 KB per wavefront, 120 KB per CU) always in
 //     flight, the stream running on across tile boundaries;
 //   * a step's 32 x 64 block goes through a wavefront-private LDS patch into MFMA operand layout:
 //     v_mfma_f32_32x32x16_bf16 with the activations on M and the vocabulary rows on N, so a lane owns one
@@ -46,8 +46,7 @@ __host__ __device__ constexpr int unembed_patch(int ks) { return 32 * (ks * 2 + 
 
 __host__ __device__ constexpr int unembed_xrow(int hidden) { return hidden * 2 + 16; }   // activation row in LDS, bytes
 
-// UNW wavefronts per workgroup: sixteen where LDS allows (up to 8 batch rows: measured 6.3 against 6.0 TB/s with eight),
-// eight with 16 batch rows resident.
+// UNW wavefronts per workgroup and UD steps in flight: see the table at unembed_nw() below.
 // SR (fp8 weight, even vocabulary): a row of fp8 is hidden bytes, 22.5 cache lines at gpt-oss's width, so that row pieces
 // never line up with cache lines; two neighbouring rows together are 2 * hidden bytes -- whole lines. The weight is then
 // read as [vocab / 2, 2 * hidden]: a tile is 32 such pairs (64 vocabulary rows), a step is 128 bytes = one aligned line of
@@ -383,12 +382,13 @@ constexpr int kUnembedGrid = 256;      // one workgroup per CU
 int unembed_xr_most(int64_t rows) { return rows <= 8 ? 8 : 16; }
 
 // (wavefronts, K step, steps in flight), measured at B = 8 on the full vocabulary:
-//   bf16, up to 8 rows : 16 wavefronts, K step 64 (whole 128-byte lines), 4 in flight   185 us (8 wavefronts: 194)
+//   bf16, up to 8 rows : 10 wavefronts, K step 64 (whole 128-byte lines), 3 in flight   174.5 us (8 x 3: 175.1, 12 x 2: 175.4,
+//                         16 x 4: 177.5, 10 x 2: 176.5, 8 x 192-element steps x 2: 182.8; the K step must divide hidden)
 //   fp8,  up to 8 rows :  even vocabulary: pairs of rows, 8 wavefronts, 128 bytes per pair and step, 2 in flight   99 us
 //                         odd vocabulary: 8 wavefronts, K step 192, 2 in flight           113 us (16 x 64 x 4: 124)
 //   16 rows            :  8 wavefronts (LDS holds the 16 activation rows), K step 64, 4 in flight
 // K steps that split 128-byte lines (96 elements of bf16, 32) cost 25-50 %.
-int unembed_nw(int xr, bool w8) { return (xr == 8 && !w8) ? 16 : 8; }
+int unembed_nw(int xr, bool w8) { return (xr == 8 && !w8) ? 10 : 8; }
 int unembed_ks(int xr, bool w8, int64_t hidden) { return (xr == 8 && w8 && hidden % 192 == 0) ? 192 : 64; }
 size_t unembed_smem(int xr, bool w8, int64_t hidden) {
   return static_cast<size_t>(xr) * unembed_xrow((int)hidden) + unembed_nw(xr, w8) * unembed_patch(unembed_ks(xr, w8, hidden));
@@ -428,7 +428,7 @@ int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t s
     hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, a);                                                             \
   } while (0)
   if (pairs) TLLM_UNEMBED(8, 8, 128, 2, true, true);          // steps in flight 1 / 2 / 3 / 4: 122 / 99 / 105 / 107 us; 12 wavefronts x 3: 103, 10 x 2: 103, 6 x 2: 115
-  else if (xr == 8 && !w8) TLLM_UNEMBED(8, 16, 64, 4, false);
+  else if (xr == 8 && !w8) TLLM_UNEMBED(8, 10, 64, 3, false);
   else if (xr == 8 && unembed_ks(8, true, a.hidden) == 192) TLLM_UNEMBED(8, 8, 192, 2, true);
   else if (xr == 8) TLLM_UNEMBED(8, 8, 64, 4, true);
   else if (w8) TLLM_UNEMBED(16, 8, 64, 4, true);
