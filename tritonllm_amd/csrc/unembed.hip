@@ -386,7 +386,7 @@ int unembed_xr_most(int64_t rows) { return rows <= 8 ? 8 : 16; }
 //                         16 x 4: 177.5, 10 x 2: 176.5, 8 x 192-element steps x 2: 182.8; the K step must divide hidden)
 //   fp8,  up to 8 rows :  even vocabulary: pairs of rows, 8 wavefronts, 128 bytes per pair and step, 2 in flight   99 us
 //                         odd vocabulary: 8 wavefronts, K step 192, 2 in flight           113 us (16 x 64 x 4: 124)
-//   16 rows            :  8 wavefronts (LDS holds the 16 activation rows), K step 64, 4 in flight
+//   16 rows            :  8 wavefronts (LDS holds the 16 activation rows), K step 64, 3 in flight (bf16: 183.4 us; 4: 185.3, 2: 188.7)
 // K steps that split 128-byte lines (96 elements of bf16, 32) cost 25-50 %.
 int unembed_nw(int xr, bool w8) { return (xr == 8 && !w8) ? 10 : 8; }
 int unembed_ks(int xr, bool w8, int64_t hidden) { return (xr == 8 && w8 && hidden % 192 == 0) ? 192 : 64; }
@@ -432,7 +432,7 @@ int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t s
   else if (xr == 8 && unembed_ks(8, true, a.hidden) == 192) TLLM_UNEMBED(8, 8, 192, 2, true);
   else if (xr == 8) TLLM_UNEMBED(8, 8, 64, 4, true);
   else if (w8) TLLM_UNEMBED(16, 8, 64, 4, true);
-  else TLLM_UNEMBED(16, 8, 64, 4, false);
+  else TLLM_UNEMBED(16, 8, 64, 3, false);
 #undef TLLM_UNEMBED
   return check_launch(who);
 }
