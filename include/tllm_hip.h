@@ -194,7 +194,9 @@ int tllm_embed_norm_qkv_rope_decode_bf16(const void* ids, int ids_is_i64, const 
  * triton_kernels.py:261-268; its use in the fused decode kernel, :927-940 and :963-965, argument
  * weight_scale of qkv_rope_cache_decode_forward :1109). Half the bytes of the bf16 kernel; activations stay
  * bf16, accumulation fp32. norm_scale may be NULL (no fused RMSNorm) or as in tllm_norm_qkv_rope_decode_bf16.
- * Exists for hidden == 2880, head_dim == 64 (TLLM_E_SHAPE otherwise). */
+ * hidden == 2880 with head_dim == 64: the weight-streaming kernels; any other hidden % 32 == 0 with
+ * head_dim % 16 == 0: the general MFMA decode kernel, norm_scale must be NULL there and q / k / v 4-byte aligned
+ * with even strides (TLLM_E_SHAPE / TLLM_E_ALIGN otherwise). */
 int tllm_qkv_rope_decode_w8_bf16(const void* x, const void* norm_scale, int scale_is_bf16, float eps,
                                  const void* W8, const float* w_scale, const void* b, void* q, void* k, void* v,
                                  int64_t q_row_stride, int64_t k_row_stride, int64_t v_row_stride,

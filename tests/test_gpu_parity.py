@@ -680,6 +680,36 @@ def test_qkv_decode_other_head_dims(gpu, hd, nq, nkv, rows):
     close(v, vr)
 
 
+@pytest.mark.parametrize("hd,nq,nkv", [(128, 4, 2), (64, 6, 1), (32, 5, 1)])
+@pytest.mark.parametrize("rows", [5, 20])
+def test_qkv_decode_fp8_weight_other_shapes(gpu, hd, nq, nkv, rows):
+    """fp8 weight with per-row scales at shapes other than gpt-oss's (the reference's fp8 branch is generic,
+    triton_kernels.py:927-940): the general MFMA decode kernel, against the oracle on the dequantised weight; with a
+    norm requested the host side runs the RMSNorm launch first."""
+    g = torch.Generator().manual_seed(2000 + hd + rows)
+    hidden = 608
+    x = torch.randn(rows, hidden, generator=g).bfloat16()
+    w = (0.05 * torch.randn((nq + 2 * nkv) * hd, hidden, generator=g)).bfloat16()
+    b = (0.05 * torch.randn((nq + 2 * nkv) * hd, generator=g)).bfloat16()
+    sc = (1 + 0.1 * torch.randn(hidden, generator=g)).bfloat16()
+    y = T.YarnParams(head_dim=hd, base=10000.0)
+    pos = torch.randint(0, 8192, (rows,), generator=g)
+    w8, ws = T.quantize_fp8_rows(w.to(gpu))
+    wd = O.dequant_fp8_ref(w8.cpu(), ws.cpu())
+    qr, kr, vr = O.qkv_rope_ref(x, wd, b, pos, nq, nkv, hd, base=10000.0, scaling_factor=1.0)
+    q, k, v = T.qkv_rope_forward(x.to(gpu), w8, b.to(gpu), nq, nkv, hd, yarn=y, positions=pos.to(gpu), mode="decode", weight_scale=ws)
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+    t_ref = O.rmsnorm_ref(x, sc.float(), 1e-5).bfloat16()
+    qr, kr, vr = O.qkv_rope_ref(t_ref, wd, b, pos, nq, nkv, hd, base=10000.0, scaling_factor=1.0)
+    q, k, v = T.qkv_rope_forward(x.to(gpu), w8, b.to(gpu), nq, nkv, hd, yarn=y, positions=pos.to(gpu), mode="decode", weight_scale=ws,
+                                 norm_scale=sc.to(gpu), norm_eps=1e-5)
+    close(q, qr)
+    close(k, kr)
+    close(v, vr)
+
+
 def test_qkv_generic_shapes(gpu):
     g = torch.Generator().manual_seed(23)
     hidden, nq, nkv, hd = 100, 3, 1, 32                     # hidden % 32 != 0, head_dim != 64 -> generic kernel

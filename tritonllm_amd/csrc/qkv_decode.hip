@@ -122,7 +122,10 @@ void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& f
 // split K in runs of SPW k32-steps whose loads are all issued before the first multiply.
 // v_mfma_f32_16x16x32_bf16: tile row 4*qd + i is dim 8p + 2*qd + (i & 1), plus half when i >= 2, so
 // each lane's four accumulators are two complete (lo, hi) pairs.
-template <int NW, int SPW>
+// W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (the reference's fp8 branch is as generic as its
+// bf16 one, triton_kernels.py:927-940): eight bytes per lane and step, widened to bf16 in registers (exact), the row
+// scale applied to the finished sum.
+template <int NW, int SPW, bool W8 = false>
 __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   __shared__ float red[NW][4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -135,6 +138,10 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 
   const int dim_a = 8 * piece + 2 * (m >> 2) + (m & 1) + ((m & 2) ? half : 0);
   const bf16x8* wrow = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * a.head_dim + dim_a) * kvec + g;
+  typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+  // fp8: the row is hidden bytes; a k32 step is 32 of them, the lane's eight at 8 g
+  const u32x2* wrow8 = reinterpret_cast<const u32x2*>(reinterpret_cast<const unsigned char*>(a.W) +
+                                                      (static_cast<int64_t>(head) * a.head_dim + dim_a) * a.hidden) + g;
   // Lanes past the last activation row re-read a live lane's row (same addresses, no extra traffic);
   // their output column is dropped.
   const int64_t xrow_idx = row0 + m;
@@ -146,11 +153,17 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int s0 = wave * SPW; s0 < nsteps; s0 += NW * SPW) {
     bf16x8 wa[SPW], xb[SPW];
+    u32x2 wa8[SPW];
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {       // clamped, never predicated: a tail step re-reads the last one and is masked below
       const int step = s0 + i < nsteps ? s0 + i : nsteps - 1;
-      wa[i] = __builtin_nontemporal_load(wrow + step * 4);
+      if constexpr (W8) wa8[i] = __builtin_nontemporal_load(wrow8 + step * 4);
+      else wa[i] = __builtin_nontemporal_load(wrow + step * 4);
       xb[i] = xrow[step * 4];
+    }
+    if constexpr (W8) {
+#pragma unroll
+      for (int i = 0; i < SPW; ++i) wa[i] = fp8x8_to_bf16x8(wa8[i][0], wa8[i][1]);
     }
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
@@ -173,6 +186,12 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   const int d0 = 8 * piece + 2 * g;
   const int col = head * a.head_dim + d0;
   float lo0 = acc[0], lo1 = acc[1], hi0 = acc[2], hi1 = acc[3];
+  if constexpr (W8) {
+    lo0 *= a.w_scale[col];
+    lo1 *= a.w_scale[col + 1];
+    hi0 *= a.w_scale[col + half];
+    hi1 *= a.w_scale[col + half + 1];
+  }
   if (a.bias) {
     lo0 += static_cast<float>(a.bias[col]);
     lo1 += static_cast<float>(a.bias[col + 1]);
@@ -310,8 +329,36 @@ extern "C" int tllm_qkv_rope_decode_w8_bf16(const void* x, const void* norm_scal
                                             int64_t k_row_stride, int64_t v_row_stride, int64_t kv_slot_stride, int64_t rows,
                                             int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim, const TllmRope* rope,
                                             void* stream) {
-  return decode_2880_entry("qkv_rope_decode_w8", x, norm_scale, scale_is_bf16, eps, W8, w_scale, true, b, q, k, v, q_row_stride,
-                           k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads, n_kv_heads, head_dim, rope, stream);
+  if (hidden == 2880 && head_dim == 64)
+    return decode_2880_entry("qkv_rope_decode_w8", x, norm_scale, scale_is_bf16, eps, W8, w_scale, true, b, q, k, v, q_row_stride,
+                             k_row_stride, v_row_stride, kv_slot_stride, rows, hidden, n_q_heads, n_kv_heads, head_dim, rope, stream);
+  // other shapes: the general MFMA decode kernel with the fp8 weight (no fused norm there)
+  QkvArgs a;
+  RopeArgs ra;
+  YarnFreqs fr;
+  int rc = qkv_validate("qkv_rope_decode_w8", x, W8, q, k, v, q_row_stride, k_row_stride, v_row_stride, kv_slot_stride, rows, hidden,
+                        n_q_heads, n_kv_heads, head_dim, rope, &a, &ra, &fr);
+  if (rc != TLLM_OK) return rc;
+  TLLM_REQUIRE(norm_scale == nullptr, TLLM_E_SHAPE,
+               "qkv_rope_decode_w8: the fused RMSNorm exists for hidden 2880 / head_dim 64 only: call tllm_rmsnorm_bf16 first");
+  TLLM_REQUIRE(head_dim % 16 == 0 && hidden % 32 == 0, TLLM_E_SHAPE,
+               "qkv_rope_decode_w8: head_dim %d must be a multiple of 16 and hidden %lld of 32", head_dim, (long long)hidden);
+  TLLM_REQUIRE(aligned16(x) && aligned16(W8), TLLM_E_ALIGN, "qkv_rope_decode_w8: x and W must be 16-byte aligned");
+  TLLM_REQUIRE(w_scale != nullptr && reinterpret_cast<uintptr_t>(w_scale) % 4 == 0, TLLM_E_ARG,
+               "qkv_rope_decode_w8: w_scale must be a 4-byte aligned device pointer");
+  const bool out4 = (reinterpret_cast<uintptr_t>(q) % 4 == 0) && (reinterpret_cast<uintptr_t>(k) % 4 == 0) &&
+                    (reinterpret_cast<uintptr_t>(v) % 4 == 0) && q_row_stride % 2 == 0 && k_row_stride % 2 == 0 &&
+                    v_row_stride % 2 == 0 && kv_slot_stride % 2 == 0;
+  TLLM_REQUIRE(out4, TLLM_E_ALIGN, "qkv_rope_decode_w8: q, k, v must be 4-byte aligned with even strides at this shape");
+  a.bias = (const bf16*)b;
+  a.w_scale = w_scale;
+  if (rows == 0) return TLLM_OK;
+  const int heads = n_q_heads + 2 * n_kv_heads;
+  const int64_t chunks = (rows + 15) / 16;
+  TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode_w8: rows %lld too many for the decode kernel", (long long)rows);
+  hipLaunchKernelGGL((qkv_decode_kernel<4, 16, true>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(4 * 64), 0,
+                     static_cast<hipStream_t>(stream), a, ra, fr);
+  return check_launch("qkv_rope_decode_w8");
 }
 
 extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const void* b, void* q, void* k, void* v, int64_t q_row_stride,

@@ -281,8 +281,9 @@ def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_
             x2 = rmsnorm_forward(x2, scale, eps)
             norm = None
     if w_scale is not None:
-        if not (kind == "decode" and x2.shape[1] == 2880 and hd == 64):
-            raise NotImplementedError("fp8 weights with per-row scales: the HIP path has the decode kernel for hidden 2880 / head_dim 64 only")
+        if kind != "decode" or x2.shape[1] % 32 != 0 or hd % 16 != 0:
+            raise NotImplementedError("fp8 weights with per-row scales: the HIP path has decode kernels only, for hidden a multiple "
+                                      "of 32 and head_dim a multiple of 16")
         scale, eps = norm if norm is not None else (None, 0.0)
         rc = lib().tllm_qkv_rope_decode_w8_bf16(
             x2.data_ptr(), ptr(scale), int(scale is not None and scale.dtype == _BF16), float(eps), weight.data_ptr(),
