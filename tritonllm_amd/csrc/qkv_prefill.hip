@@ -335,8 +335,8 @@ __global__ __launch_bounds__(512) void qkv_prefill_quads_kernel(QkvArgs a, RopeA
       }
       if constexpr (TABLE) {
         const int64_t at = a.has_rope ? rope_wrap(p, ra.max_ctx) * ra.table_row_stride + f : f;
-        // The youngest loads of the prologue: a wait counts them in until they have landed, which they have by the
-        // loop's second slice (they return behind the look-ahead loads issued before them).
+        // The youngest loads of the prologue: every wait below is for older loads and so at most stricter than it
+        // needs to be until these have landed, which they have by the loop's second slice.
         csr[j] = make_float2(cos_t[at], sin_t[at]);
       } else {
         float c, sn;
@@ -346,10 +346,9 @@ __global__ __launch_bounds__(512) void qkv_prefill_quads_kernel(QkvArgs a, RopeA
     }
   }
   // slice 0 has landed when only those are outstanding
-  if constexpr (TABLE)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW + 2 * CSN) : "memory");
-  else
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");
+  // (TABLE: the sixteen table loads are younger still and are not counted in, so this wait also takes some of the
+  // look-ahead loads in -- measured: no difference -- and does not depend on how many loads the compiler makes of them)
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((WS - 2) * LPWW + LPW) : "memory");
   __syncthreads();
 #pragma unroll
   for (int tb = 0; tb < TB; ++tb) fx[0][tb] = *reinterpret_cast<const bf16x8*>(xring + fx_o[tb]);
