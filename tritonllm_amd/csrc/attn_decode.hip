@@ -93,6 +93,7 @@ __device__ __forceinline__ int attn_live_splits(const AttnArgs& a, int* lo_out, 
 template <bool ROWS>
 __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(AttnArgs a) {
   __shared__ __align__(16) unsigned char vt[(ROWS ? RW : AW) * VTILE];
+  __shared__ __align__(16) unsigned char kt[(ROWS ? RW : AW) * VTILE];   // K tile, the same shape
   __shared__ float s_m[ROWS ? 1 : AW][16], s_l[ROWS ? 1 : AW][16];
   __shared__ float s_acc[ROWS ? 1 : AW][ROWS ? 1 : 16][64 + 1];
 
@@ -142,6 +143,7 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
   const bf16* kbase = a.k + b * a.kv_bs + static_cast<int64_t>(kvh) * 64;
   const bf16* vbase = a.v + b * a.kv_bs + static_cast<int64_t>(kvh) * 64;
   unsigned char* vtile = vt + wave * VTILE;
+  unsigned char* ktile = kt + wave * VTILE;
 
   float m_run = kNegBig, l_run = 0.f;                          // of head r16 (replicated over the four lane groups)
   f32x4_t acc[4];                                              // O: lane (d = 16 nb + r16, heads 4 g + i)
@@ -157,23 +159,21 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
   auto ld = [](const unsigned char* p) {
     return ROWS ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p)) : *reinterpret_cast<const bf16x8*>(p);
   };
-  bf16x8 ka[2][2], vr[4];
+  // K and V both arrive row-major, eight neighbouring lanes covering one 128-byte row piece; K's A-operand fragments
+  // (lane = (key, k group)) are then read out of LDS. Loaded straight into operand layout, neighbouring lanes ask for
+  // different rows -- 64 requests of 16 bytes per instruction, which the memory side serves at three quarters of the rate.
+  bf16x8 kr[4], vr[4];
   auto load_block = [&](int k0) {
     const int last = s_hi - k0 - 1;                            // last valid row of the block (>= 31 except in the final one)
     const unsigned char* kb0 = reinterpret_cast<const unsigned char*>(kbase + static_cast<int64_t>(k0) * a.kv_ts);
     const unsigned char* vb0 = reinterpret_cast<const unsigned char*>(vbase + static_cast<int64_t>(k0) * a.kv_ts);
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int r = 16 * kb + r16;
-      const unsigned off = static_cast<unsigned>(r < last ? r : last) * ts_b + 16u * g;
-      ka[kb][0] = ld(kb0 + off);
-      ka[kb][1] = ld(kb0 + off + 64);
-    }
-#pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = i * 64 + lane;
       const int r = c >> 3;
-      vr[i] = ld(vb0 + static_cast<unsigned>(r < last ? r : last) * ts_b + 16u * (c & 7));
+      const unsigned off = static_cast<unsigned>(r < last ? r : last) * ts_b + 16u * (c & 7);
+      kr[i] = ld(kb0 + off);
+      vr[i] = ld(vb0 + off);
     }
   };
 
@@ -183,17 +183,23 @@ __global__ __launch_bounds__((ROWS ? RW : AW) * 64) void attn_decode_kernel(Attn
   for (int blk = first; blk < nblk; blk += STEP) {
     const int k0 = s_lo + 32 * blk;
     // ---- S^T for the block's two 16-key halves
-    f32x4_t st[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb][0], qb0, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-      st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb][1], qb1, st[kb], 0, 0, 0);
-    }
-    // V tile into LDS (row-major, as loaded)
+    // K and V tiles into LDS (row-major, as loaded)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = i * 64 + lane;
+      *reinterpret_cast<bf16x8*>(ktile + (c >> 3) * VROW + (c & 7) * 16) = kr[i];
       *reinterpret_cast<bf16x8*>(vtile + (c >> 3) * VROW + (c & 7) * 16) = vr[i];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    f32x4_t st[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const unsigned char* krow = ktile + (16 * kb + r16) * VROW + 16 * g;
+      const bf16x8 ka0 = *reinterpret_cast<const bf16x8*>(krow), ka1 = *reinterpret_cast<const bf16x8*>(krow + 64);
+      st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka0, qb0, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka1, qb1, st[kb], 0, 0, 0);
     }
     // The next block's loads go out before this one's arithmetic. Unconditional (a load under a branch makes the
     // compiler wait for it where the paths join): the last round simply requests its own block again.
