@@ -125,9 +125,16 @@ void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& f
 // W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (the reference's fp8 branch is as generic as its
 // bf16 one, triton_kernels.py:927-940): eight bytes per lane and step, widened to bf16 in registers (exact), the row
 // scale applied to the finished sum.
+// bf16 weight: a run's 16 rows x SPW x 64 bytes arrive row by row -- one load instruction = one row's contiguous run, 64
+// lanes x 16 bytes -- and pass a wavefront-private LDS patch on their way into A-operand layout (loaded straight into
+// that layout every lane's 16 bytes are a request of their own, and the memory side serves such a stream at three
+// quarters of the rate).
 template <int NW, int SPW, bool W8 = false>
 __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   __shared__ float red[NW][4][64];
+  constexpr int WROW = SPW * 64 + 16;                       // patch row: a run's bytes of one weight row + padding (conflict-free fragment reads)
+  extern __shared__ __align__(16) unsigned char wpatch_all[];   // bf16 weight: [NW][16][WROW]
+  static_assert(W8 || SPW == 16, "a load instruction covers one row's run of 16 steps");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int half = a.head_dim >> 1, pieces = half >> 3;
   const int head = blockIdx.x / pieces, piece = blockIdx.x - head * pieces;
@@ -157,9 +164,28 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {       // clamped, never predicated: a tail step re-reads the last one and is masked below
       const int step = s0 + i < nsteps ? s0 + i : nsteps - 1;
-      if constexpr (W8) wa8[i] = __builtin_nontemporal_load(wrow8 + step * 4);
-      else wa[i] = __builtin_nontemporal_load(wrow + step * 4);
+      if constexpr (W8) {
+        wa8[i] = __builtin_nontemporal_load(wrow8 + step * 4);
+      } else {
+        // load i = tile row i: lane l fetches chunk s0 * 4 + l of that row (clamped at the row's end: a tail run re-reads
+        // the last chunk; those steps are masked below)
+        const int chunk = s0 * 4 + lane < kvec ? s0 * 4 + lane : kvec - 1;
+        const int dim_i = 8 * piece + 2 * (i >> 2) + (i & 1) + ((i & 2) ? half : 0);
+        wa[i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * a.head_dim + dim_i) * kvec + chunk);
+      }
       xb[i] = xrow[step * 4];
+    }
+    if constexpr (!W8) {
+      unsigned char* wp = wpatch_all + wave * (16 * WROW);
+#pragma unroll
+      for (int i = 0; i < SPW; ++i) *reinterpret_cast<bf16x8*>(wp + i * WROW + lane * 16) = wa[i];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int i = 0; i < SPW; ++i) wa[i] = *reinterpret_cast<const bf16x8*>(wp + m * WROW + (4 * i + g) * 16);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the next run's writes come after these reads
+      __builtin_amdgcn_wave_barrier();
     }
     if constexpr (W8) {
 #pragma unroll
@@ -386,7 +412,16 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
   if (mfma_ok && out4) {
     const int64_t chunks = (rows + 15) / 16;
     TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
-    hipLaunchKernelGGL((qkv_decode_kernel<4, 16>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(4 * 64), 0, st, a, ra, fr);
+    constexpr size_t kPatchBytes = 4 * 16 * (16 * 64 + 16);     // four wavefronts' weight patches: 66 560 bytes
+    static bool attr_set = false;   // raising the dynamic-LDS limit is idempotent; a benign race at worst repeats it
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_decode_kernel<4, 16>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)kPatchBytes);
+      TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_decode: cannot raise LDS limit: %s", hipGetErrorString(e));
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((qkv_decode_kernel<4, 16>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(4 * 64), kPatchBytes, st, a, ra,
+                       fr);
     return check_launch("qkv_rope_decode");
   }
   launch_qkv_generic(a, ra, fr, st);
