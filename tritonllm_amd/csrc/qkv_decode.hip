@@ -412,15 +412,19 @@ extern "C" int tllm_qkv_rope_decode_bf16(const void* x, const void* W, const voi
   if (mfma_ok && out4) {
     const int64_t chunks = (rows + 15) / 16;
     TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode: rows %lld too many for the decode kernel", (long long)rows);
-    constexpr size_t kPatchBytes = 4 * 16 * (16 * 64 + 16);     // four wavefronts' weight patches: 66 560 bytes
+    // wavefronts per workgroup 1 / 2 / 4 / 8: 14.0 / 14.7 / 15.5 / 17.2 us at hidden 4096, 8 rows (one wavefront then walks K in
+    // runs of 512, one after the other; two register sets taken in turn, so that the next run's loads are out while a run is
+    // multiplied, changed nothing: 14.1 us, at 292 registers one wavefront per SIMD)
+    constexpr int GNW = 1;
+    constexpr size_t kPatchBytes = GNW * 16 * (16 * 64 + 16);   // the wavefronts' weight patches
     static bool attr_set = false;   // raising the dynamic-LDS limit is idempotent; a benign race at worst repeats it
     if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_decode_kernel<4, 16>), hipFuncAttributeMaxDynamicSharedMemorySize,
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_decode_kernel<GNW, 16>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          (int)kPatchBytes);
       TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "qkv_rope_decode: cannot raise LDS limit: %s", hipGetErrorString(e));
       attr_set = true;
     }
-    hipLaunchKernelGGL((qkv_decode_kernel<4, 16>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(4 * 64), kPatchBytes, st, a, ra,
+    hipLaunchKernelGGL((qkv_decode_kernel<GNW, 16>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(GNW * 64), kPatchBytes, st, a, ra,
                        fr);
     return check_launch("qkv_rope_decode");
   }
