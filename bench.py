@@ -124,17 +124,20 @@ def run_only(args, T, torch, dev, yarn, bytes_of, graph_of, steady_graph, weight
     kind, _, size = name.rpartition("_")
     n = int(size[1:])
     flops = nbytes = None
-    if kind in ("qkv_rope_decode_h4096_hd64", "qkv_rope_decode_h4096_hd128"):
-        # shapes other than gpt-oss's: the general decode kernels (8 rotating weights of [6144, 4096])
+    if kind in ("qkv_rope_decode_h4096_hd64", "qkv_rope_decode_h4096_hd128", "qkv_rope_decode_w8_h4096_hd64"):
+        # shapes other than gpt-oss's: the general decode kernel (8 rotating weights of [6144, 4096], bf16 or fp8)
         nq, nkv, hd = (64, 8, 64) if kind.endswith("hd64") else (32, 8, 128)
+        w8 = "_w8_" in kind
         od = (nq + 2 * nkv) * hd
         ws = [torch.empty(od, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(8)]
+        wq = [T.quantize_fp8_rows(w) for w in ws] if w8 else None
         bs = torch.empty(od, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
         xr = torch.randn(n, 4096, generator=g).bfloat16().to(dev)
         pr = torch.randint(0, 8192, (n,), generator=g, dtype=torch.int64).to(dev)
         yg = T.YarnParams(head_dim=hd, base=150000.0)
-        fn = lambda i: T.qkv_rope_forward(xr, ws[i % 8], bs, nq, nkv, hd, yarn=yg, positions=pr, mode="decode")
-        nbytes = od * 4096 * 2 + od * 2 + n * (4096 * 2 + od * 2)
+        fn = lambda i: T.qkv_rope_forward(xr, wq[i % 8][0] if w8 else ws[i % 8], bs, nq, nkv, hd, yarn=yg, positions=pr, mode="decode",
+                                          weight_scale=wq[i % 8][1] if w8 else None)
+        nbytes = od * 4096 * (1 if w8 else 2) + od * (6 if w8 else 2) + n * (4096 * 2 + od * 2)
         kind = "generic"
     tables = kind == "qkv_rope_prefill_tables"           # cos / sin from the precomputed tables, as the reference passes them
     if tables:
@@ -536,7 +539,7 @@ def main() -> int:
                                                                            yarn=yarn, positions=pr, mode="decode", out=qo),
                          bytes_of["qkv"](r), n=96)
         # other model shapes (the reference's decode kernel is generic over hidden_size and head_dim, triton_kernels.py:1127-1158):
-        # hidden 4096 with head_dim 64 takes the general MFMA decode kernel, head_dim 128 the general scalar kernel
+        # hidden 4096 with head_dim 64 or 128 takes the general MFMA decode kernel, with a bf16 or an fp8 weight
         for tag, hid, nq, nkv, hd in (("h4096_hd64", 4096, 64, 8, 64), ("h4096_hd128", 4096, 32, 8, 128)):
             od = (nq + 2 * nkv) * hd
             ws = [torch.empty(od, hid, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(8)]
@@ -547,6 +550,13 @@ def main() -> int:
                          lambda i, xr=xr, ws=ws, bs=bs, nq=nq, nkv=nkv, hd=hd, yg=yg: T.qkv_rope_forward(xr, ws[i % 8], bs, nq, nkv, hd, yarn=yg,
                                                                                                          positions=positions, mode="decode"),
                          od * hid * 2 + od * 2 + B * (hid * 2 + od * 2), n=96)
+            if hd == 64:
+                wq8 = [T.quantize_fp8_rows(w) for w in ws]
+                bench_kernel(f"qkv_rope_decode_w8_{tag}_B{B}",
+                             lambda i, xr=xr, wq8=wq8, bs=bs, nq=nq, nkv=nkv, hd=hd, yg=yg: T.qkv_rope_forward(
+                                 xr, wq8[i % 8][0], bs, nq, nkv, hd, yarn=yg, positions=positions, mode="decode", weight_scale=wq8[i % 8][1]),
+                             od * hid + od * 6 + B * (hid * 2 + od * 2), n=96)
+                del wq8
             del ws
         # the first layer of a token step: the gather rides in the same launch (embedding_B8 + norm_qkv_rope_decode_B8 in one)
         qo = (torch.empty(B, NQ * HD, dtype=torch.bfloat16, device=dev), torch.empty(B, NKV * HD, dtype=torch.bfloat16, device=dev),

@@ -125,16 +125,16 @@ void launch_qkv_generic(const QkvArgs& a, const RopeArgs& ra, const YarnFreqs& f
 // W8: the weight is fp8 (OCP e4m3) with one fp32 scale per output row (the reference's fp8 branch is as generic as its
 // bf16 one, triton_kernels.py:927-940): eight bytes per lane and step, widened to bf16 in registers (exact), the row
 // scale applied to the finished sum.
-// bf16 weight: a run's 16 rows x SPW x 64 bytes arrive row by row -- one load instruction = one row's contiguous run, 64
-// lanes x 16 bytes -- and pass a wavefront-private LDS patch on their way into A-operand layout (loaded straight into
-// that layout every lane's 16 bytes are a request of their own, and the memory side serves such a stream at three
+// A run's 16 weight rows x SPW steps arrive row by row -- one load instruction = one row's contiguous run, 64 lanes x 16
+// bytes (fp8: x 8) -- and pass a wavefront-private LDS patch on their way into A-operand layout (loaded straight into
+// that layout every lane's bytes are a request of their own, and the memory side serves such a stream at three
 // quarters of the rate).
 template <int NW, int SPW, bool W8 = false>
 __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs ra, YarnFreqs fr) {
   __shared__ float red[NW][4][64];
-  constexpr int WROW = SPW * 64 + 16;                       // patch row: a run's bytes of one weight row + padding (conflict-free fragment reads)
-  extern __shared__ __align__(16) unsigned char wpatch_all[];   // bf16 weight: [NW][16][WROW]
-  static_assert(W8 || SPW == 16, "a load instruction covers one row's run of 16 steps");
+  constexpr int WROW = SPW * (W8 ? 32 : 64) + 16;           // patch row: a run's bytes of one weight row + padding (conflict-free fragment reads)
+  extern __shared__ __align__(16) unsigned char wpatch_all[];   // [NW][16][WROW]
+  static_assert(SPW == 16, "a load instruction covers one row's run of 16 steps");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int half = a.head_dim >> 1, pieces = half >> 3;
   const int head = blockIdx.x / pieces, piece = blockIdx.x - head * pieces;
@@ -143,12 +143,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
   const int nsteps = a.hidden >> 5;     // MFMA k-steps of 32
   const int m = lane & 15, g = lane >> 4;
 
-  const int dim_a = 8 * piece + 2 * (m >> 2) + (m & 1) + ((m & 2) ? half : 0);
-  const bf16x8* wrow = reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * a.head_dim + dim_a) * kvec + g;
   typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
-  // fp8: the row is hidden bytes; a k32 step is 32 of them, the lane's eight at 8 g
-  const u32x2* wrow8 = reinterpret_cast<const u32x2*>(reinterpret_cast<const unsigned char*>(a.W) +
-                                                      (static_cast<int64_t>(head) * a.head_dim + dim_a) * a.hidden) + g;
   // Lanes past the last activation row re-read a live lane's row (same addresses, no extra traffic);
   // their output column is dropped.
   const int64_t xrow_idx = row0 + m;
@@ -164,29 +159,35 @@ __global__ __launch_bounds__(NW * 64) void qkv_decode_kernel(QkvArgs a, RopeArgs
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {       // clamped, never predicated: a tail step re-reads the last one and is masked below
       const int step = s0 + i < nsteps ? s0 + i : nsteps - 1;
+      // load i = tile row i: lane l fetches chunk s0 * 4 + l of that row -- 16 bytes of a bf16 row, 8 of an fp8 row, either
+      // way the lane's share of the run's 16 steps -- clamped at the row's end (a tail run re-reads the last chunk; those
+      // steps are masked below)
+      const int chunk = s0 * 4 + lane < kvec ? s0 * 4 + lane : kvec - 1;
+      const int dim_i = 8 * piece + 2 * (i >> 2) + (i & 1) + ((i & 2) ? half : 0);
+      const int64_t wrow_i = static_cast<int64_t>(head) * a.head_dim + dim_i;
       if constexpr (W8) {
-        wa8[i] = __builtin_nontemporal_load(wrow8 + step * 4);
+        wa8[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(reinterpret_cast<const unsigned char*>(a.W) + wrow_i * a.hidden) + chunk);
       } else {
-        // load i = tile row i: lane l fetches chunk s0 * 4 + l of that row (clamped at the row's end: a tail run re-reads
-        // the last chunk; those steps are masked below)
-        const int chunk = s0 * 4 + lane < kvec ? s0 * 4 + lane : kvec - 1;
-        const int dim_i = 8 * piece + 2 * (i >> 2) + (i & 1) + ((i & 2) ? half : 0);
-        wa[i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(a.W) + (static_cast<int64_t>(head) * a.head_dim + dim_i) * kvec + chunk);
+        wa[i] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(a.W) + wrow_i * kvec + chunk);
       }
       xb[i] = xrow[step * 4];
     }
-    if constexpr (!W8) {
-      unsigned char* wp = wpatch_all + wave * (16 * WROW);
+    unsigned char* wp = wpatch_all + wave * (16 * WROW);
 #pragma unroll
-      for (int i = 0; i < SPW; ++i) *reinterpret_cast<bf16x8*>(wp + i * WROW + lane * 16) = wa[i];
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-      for (int i = 0; i < SPW; ++i) wa[i] = *reinterpret_cast<const bf16x8*>(wp + m * WROW + (4 * i + g) * 16);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the next run's writes come after these reads
-      __builtin_amdgcn_wave_barrier();
+    for (int i = 0; i < SPW; ++i) {
+      if constexpr (W8) *reinterpret_cast<u32x2*>(wp + i * WROW + lane * 8) = wa8[i];
+      else *reinterpret_cast<bf16x8*>(wp + i * WROW + lane * 16) = wa[i];
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      if constexpr (W8) wa8[i] = *reinterpret_cast<const u32x2*>(wp + m * WROW + (4 * i + g) * 8);
+      else wa[i] = *reinterpret_cast<const bf16x8*>(wp + m * WROW + (4 * i + g) * 16);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the next run's writes come after these reads
+    __builtin_amdgcn_wave_barrier();
     if constexpr (W8) {
 #pragma unroll
       for (int i = 0; i < SPW; ++i) wa[i] = fp8x8_to_bf16x8(wa8[i][0], wa8[i][1]);
@@ -382,8 +383,12 @@ extern "C" int tllm_qkv_rope_decode_w8_bf16(const void* x, const void* norm_scal
   const int heads = n_q_heads + 2 * n_kv_heads;
   const int64_t chunks = (rows + 15) / 16;
   TLLM_REQUIRE(chunks <= 65535, TLLM_E_SHAPE, "qkv_rope_decode_w8: rows %lld too many for the decode kernel", (long long)rows);
-  hipLaunchKernelGGL((qkv_decode_kernel<4, 16, true>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(4 * 64), 0,
-                     static_cast<hipStream_t>(stream), a, ra, fr);
+  // wavefronts per workgroup 1 / 2 / 4 / 8: 16.2 / 13.0 / 13.6 / 14.0 us at hidden 4096, 8 or 16 rows (a run is half the bytes of
+  // a bf16 run, so two wavefronts keep as much in flight as one does there); loaded straight into operand layout, four
+  // wavefronts: 19.6 us
+  constexpr int GNW = 2;
+  hipLaunchKernelGGL((qkv_decode_kernel<GNW, 16, true>), dim3((unsigned)(heads * (head_dim / 16)), (unsigned)chunks), dim3(GNW * 64),
+                     GNW * 16 * (16 * 32 + 16), static_cast<hipStream_t>(stream), a, ra, fr);
   return check_launch("qkv_rope_decode_w8");
 }
 
