@@ -92,6 +92,13 @@ def lib() -> C.CDLL:
     return _lib
 
 
+def require(cond, msg: str = "") -> None:
+    """The reference's argument checks are `assert` statements (triton_kernels.py:1086-1106 and the other op wrappers); these
+    raise the same AssertionError but survive `python -O`, since several of them guard device memory accesses."""
+    if not cond:
+        raise AssertionError(msg)
+
+
 def check(rc: int, what: str) -> None:
     if rc != 0:
         msg = lib().tllm_last_error().decode("utf-8", "replace")

@@ -15,6 +15,7 @@ import torch
 
 from . import ops
 from ._lib import check, lib
+from ._lib import require as _require
 from .yarn import YarnParams
 
 
@@ -190,7 +191,7 @@ class Embedding(torch.nn.Module):
 
     def __init__(self, num_embeddings: int, embedding_dim: int, device: torch.device | None = None, dtype: torch.dtype = torch.bfloat16):
         super().__init__()
-        assert dtype == torch.bfloat16
+        _require(dtype == torch.bfloat16)
         self.num_embeddings = num_embeddings
         self.embedding_dim = embedding_dim
         self.weight = torch.nn.Parameter(torch.empty((num_embeddings, embedding_dim), device=device, dtype=dtype))

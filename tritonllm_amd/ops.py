@@ -29,6 +29,7 @@ import torch
 
 from . import scratch_pool
 from ._lib import TllmRope, check, lib
+from ._lib import require as _require
 from .yarn import YarnParams
 
 _BF16 = torch.bfloat16
@@ -89,15 +90,15 @@ def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, kee
         r.yarn = yarn.c_pointer()
         keep.append(yarn)
     else:
-        assert cos is not None and sin is not None, "rotary needs YaRN parameters or cos/sin tables"
-        assert cos.dtype == torch.float32 and sin.dtype == torch.float32
-        assert cos.ndim == 2 and cos.shape == sin.shape
+        _require(cos is not None and sin is not None, "rotary needs YaRN parameters or cos/sin tables")
+        _require(cos.dtype == torch.float32 and sin.dtype == torch.float32)
+        _require(cos.ndim == 2 and cos.shape == sin.shape)
         if cos.stride(-1) != 1:
             cos = cos.contiguous()
         if sin.stride(-1) != 1 or sin.stride(0) != cos.stride(0):
             sin = sin.contiguous()
             cos = cos.contiguous()
-        assert cos.shape[0] >= max_ctx, "cos/sin tables shorter than max_context_length"
+        _require(cos.shape[0] >= max_ctx, "cos/sin tables shorter than max_context_length")
         keep += [cos, sin]
         r.cos_table = cos.data_ptr()
         r.sin_table = sin.data_ptr()
@@ -123,17 +124,17 @@ def _rope_desc(cos, sin, yarn, positions, offset, tokens_per_batch, max_ctx, kee
 def rmsnorm_forward(x: torch.Tensor, scale: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
     """``y = x * rsqrt(mean(x^2) + eps) * scale`` over the last dim; ``out`` may alias ``x``."""
     _on_gpu(x, scale, out)
-    assert x.dtype == _BF16, "rmsnorm_forward: x must be bfloat16"
-    assert scale.dtype in (torch.float32, _BF16), "rmsnorm_forward: scale must be float32 or bfloat16"
+    _require(x.dtype == _BF16, "rmsnorm_forward: x must be bfloat16")
+    _require(scale.dtype in (torch.float32, _BF16), "rmsnorm_forward: scale must be float32 or bfloat16")
     hidden = x.shape[-1]
-    assert scale.shape == (hidden,)
+    _require(scale.shape == (hidden,))
     if not x.is_contiguous():
         x = x.contiguous()
     if not scale.is_contiguous():
         scale = scale.contiguous()
     if out is None:
         out = scratch_pool.get(tuple(x.shape), x.dtype, x.device)
-    assert out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()
+    _require(out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous())
     rows = x.numel() // hidden if hidden else 0
     rc = lib().tllm_rmsnorm_bf16(x.data_ptr(), scale.data_ptr(), int(scale.dtype == _BF16), out.data_ptr(), rows, hidden,
                                  float(eps), _stream())
@@ -149,17 +150,17 @@ def embedding_forward(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor 
     An id outside ``[0, vocab)`` produces a zero row and sets ``oob_flag`` (int32 device
     scalar) to 1 when one is given -- never a device fault."""
     _on_gpu(ids, table, out, oob_flag)
-    assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
-    assert ids.dtype in (torch.int32, torch.int64)
+    _require(table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous())
+    _require(ids.dtype in (torch.int32, torch.int64))
     if not ids.is_contiguous():
         ids = ids.contiguous()
     vocab, hidden = table.shape
     shape = (*ids.shape, hidden)
     if out is None:
         out = torch.empty(shape, dtype=table.dtype, device=table.device)   # a fresh tensor, as nn.Embedding returns
-    assert tuple(out.shape) == shape and out.dtype == table.dtype and out.is_contiguous()
+    _require(tuple(out.shape) == shape and out.dtype == table.dtype and out.is_contiguous())
     if oob_flag is not None:
-        assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
+        _require(oob_flag.dtype == torch.int32 and oob_flag.numel() == 1)
     rc = lib().tllm_embedding_bf16(table.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64), out.data_ptr(), ids.numel(),
                                    hidden, vocab, oob_flag.data_ptr() if oob_flag is not None else None, _stream())
     check(rc, "embedding_forward")
@@ -174,11 +175,11 @@ def embedding_rmsnorm_forward(ids: torch.Tensor, table: torch.Tensor, scale: tor
     unless ``x_out`` is given), ``normed`` identical to ``rmsnorm_forward(x, scale, eps)`` (pooled unless ``out`` is given).
     Hidden sizes the fused kernel does not cover take the two separate calls."""
     _on_gpu(ids, table, scale, x_out, out, oob_flag)
-    assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
-    assert ids.dtype in (torch.int32, torch.int64)
-    assert scale.dtype in (torch.float32, _BF16), "embedding_rmsnorm_forward: scale must be float32 or bfloat16"
+    _require(table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous())
+    _require(ids.dtype in (torch.int32, torch.int64))
+    _require(scale.dtype in (torch.float32, _BF16), "embedding_rmsnorm_forward: scale must be float32 or bfloat16")
     vocab, hidden = table.shape
-    assert scale.shape == (hidden,)
+    _require(scale.shape == (hidden,))
     if hidden % 8 != 0 or hidden > 8192:
         x = embedding_forward(ids, table, out=x_out, oob_flag=oob_flag)
         return x, rmsnorm_forward(x, scale, eps, out=out)
@@ -192,10 +193,10 @@ def embedding_rmsnorm_forward(ids: torch.Tensor, table: torch.Tensor, scale: tor
     if out is None:
         out = scratch_pool.get(shape, table.dtype, table.device)
     for t in (x_out, out):
-        assert tuple(t.shape) == shape and t.dtype == table.dtype and t.is_contiguous()
-    assert x_out.data_ptr() != out.data_ptr()
+        _require(tuple(t.shape) == shape and t.dtype == table.dtype and t.is_contiguous())
+    _require(x_out.data_ptr() != out.data_ptr())
     if oob_flag is not None:
-        assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
+        _require(oob_flag.dtype == torch.int32 and oob_flag.numel() == 1)
     rc = lib().tllm_embed_rmsnorm_bf16(table.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64), x_out.data_ptr(), scale.data_ptr(),
                                        int(scale.dtype == _BF16), out.data_ptr(), ids.numel(), hidden, vocab, float(eps),
                                        oob_flag.data_ptr() if oob_flag is not None else None, _stream())
@@ -208,8 +209,8 @@ def swiglu(x: torch.Tensor, alpha: float = 1.702, limit: float | None = 7.0, int
            out: torch.Tensor | None = None) -> torch.Tensor:
     """Clamped SwiGLU over the last dim: ``[..., 2n] -> [..., n]``."""
     _on_gpu(x, out)
-    assert x.dtype == _BF16, "swiglu: x must be bfloat16"
-    assert x.shape[-1] % 2 == 0
+    _require(x.dtype == _BF16, "swiglu: x must be bfloat16")
+    _require(x.shape[-1] % 2 == 0)
     n_out = x.shape[-1] // 2
     if x.stride(-1) != 1:
         x = x.contiguous()
@@ -220,7 +221,7 @@ def swiglu(x: torch.Tensor, alpha: float = 1.702, limit: float | None = 7.0, int
     shape = (*x.shape[:-1], n_out)
     if out is None:
         out = torch.empty(shape, dtype=x.dtype, device=x.device)
-    assert tuple(out.shape) == shape and out.dtype == x.dtype and out.is_contiguous()
+    _require(tuple(out.shape) == shape and out.dtype == x.dtype and out.is_contiguous())
     row_stride = x2.stride(0) if rows > 1 else 2 * n_out
     rc = lib().tllm_swiglu_bf16(x2.data_ptr(), out.data_ptr(), rows, n_out, row_stride, float(alpha),
                                 float(limit) if limit is not None else 0.0, int(limit is not None), int(bool(interleaved)), _stream())
@@ -243,9 +244,9 @@ def rope_forward(query: torch.Tensor, key: torch.Tensor, sin: torch.Tensor | Non
     _on_gpu(query, key, offset, positions)
     batch_size, num_tokens, num_heads, head_dim = query.shape
     kb, kt, num_key_value_heads, khd = key.shape
-    assert (kb, kt, khd) == (batch_size, num_tokens, head_dim)
-    assert query.dtype == _BF16 and key.dtype == _BF16
-    assert query.is_contiguous() and key.is_contiguous(), "rope_forward rotates in place and needs dense q/k"
+    _require((kb, kt, khd) == (batch_size, num_tokens, head_dim))
+    _require(query.dtype == _BF16 and key.dtype == _BF16)
+    _require(query.is_contiguous() and key.is_contiguous(), "rope_forward rotates in place and needs dense q/k")
     keep: list = []
     desc = _rope_desc(cos, sin, yarn, positions, offset, num_tokens, max_context_length, keep, batch_size * num_tokens)
     rc = lib().tllm_rope_bf16(query.data_ptr(), key.data_ptr(), batch_size * num_tokens, num_heads, num_key_value_heads, head_dim,
@@ -268,7 +269,7 @@ def _launch_qkv(kind: str, x2, weight, bias, q, k, v, q_rs, k_rs, v_rs, kv_slot_
     rope = C.byref(desc) if desc is not None else None
     if norm is not None:
         scale, eps = norm
-        assert scale.dtype in (torch.float32, _BF16) and scale.shape == (x2.shape[1],)
+        _require(scale.dtype in (torch.float32, _BF16) and scale.shape == (x2.shape[1],))
         if not scale.is_contiguous():
             scale = scale.contiguous()
         if w_scale is None and _norm_fusable(kind, x2.shape[0], x2.shape[1], hd):
@@ -310,13 +311,13 @@ def quantize_fp8_rows(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]
 
 
 def _prep_weight_scale(weight, weight_scale):
-    assert weight.dtype == _FP8, "weight_scale goes with a float8_e4m3fn weight"
-    assert weight_scale.dtype == torch.float32 and weight_scale.shape == (weight.shape[0],)
+    _require(weight.dtype == _FP8, "weight_scale goes with a float8_e4m3fn weight")
+    _require(weight_scale.dtype == torch.float32 and weight_scale.shape == (weight.shape[0],))
     return weight_scale if weight_scale.is_contiguous() else weight_scale.contiguous()
 
 
 def _prep_linear(hidden2, weight, bias):
-    assert hidden2.dtype == _BF16 and weight.dtype in (_BF16, _FP8) and (bias is None or bias.dtype == _BF16)
+    _require(hidden2.dtype == _BF16 and weight.dtype in (_BF16, _FP8) and (bias is None or bias.dtype == _BF16))
     if not hidden2.is_contiguous():
         hidden2 = hidden2.contiguous()
     if not weight.is_contiguous():
@@ -343,13 +344,13 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     "prefill" (MFMA GEMM) or "auto" (by row count). No reference twin as a single call:
     it is F.linear + split + contiguous + rope_forward of model.py:506-522 in one launch."""
     _on_gpu(x, weight, bias, positions, offset, cos, sin, norm_scale, weight_scale)
-    assert x.ndim == 2
-    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
+    _require(x.ndim == 2)
+    _require((weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none")
     rows, hidden = x.shape
     total_out, hidden_w = weight.shape
-    assert hidden == hidden_w
-    assert total_out == (num_q_heads + 2 * num_kv_heads) * head_dim
-    assert bias is None or bias.shape == (total_out,)
+    _require(hidden == hidden_w)
+    _require(total_out == (num_q_heads + 2 * num_kv_heads) * head_dim)
+    _require(bias is None or bias.shape == (total_out,))
     x, weight, bias = _prep_linear(x, weight, bias)
     q_dim, kv_dim = num_q_heads * head_dim, num_kv_heads * head_dim
     if out is None:
@@ -359,8 +360,8 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
         k, v = kv[0], kv[1]
     else:
         q, k, v = out
-        assert q.shape == (rows, q_dim) and k.shape == (rows, kv_dim) and v.shape == (rows, kv_dim)
-        assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1
+        _require(q.shape == (rows, q_dim) and k.shape == (rows, kv_dim) and v.shape == (rows, kv_dim))
+        _require(q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1)
     keep: list = []
     desc = None
     if rotate:
@@ -368,7 +369,7 @@ def qkv_rope_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
                           max_context_length, keep, rows)
     if mode == "auto":
         mode = "decode" if rows <= _decode_max_rows(x.shape[-1], head_dim) else "prefill"
-    assert mode in ("decode", "prefill")
+    _require(mode in ("decode", "prefill"))
     _launch_qkv(mode, x, weight, bias, q, k, v, q.stride(0), k.stride(0), v.stride(0), 0, num_q_heads, num_kv_heads, head_dim, desc,
                 norm=None if norm_scale is None else (norm_scale, norm_eps),
                 w_scale=None if weight_scale is None else _prep_weight_scale(weight, weight_scale))
@@ -393,14 +394,14 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
     otherwise it is the gather followed by ``qkv_rope_forward``. Either way an id outside the table produces a zero
     row of ``x`` (and the q / k / v that follow from it) and sets ``oob_flag``."""
     _on_gpu(ids, table, norm_scale, weight, bias, positions, offset, cos, sin, weight_scale, x_out, oob_flag)
-    assert ids.ndim == 1 and ids.dtype in (torch.int32, torch.int64)
-    assert table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous()
+    _require(ids.ndim == 1 and ids.dtype in (torch.int32, torch.int64))
+    _require(table.dtype == _BF16 and table.ndim == 2 and table.is_contiguous())
     rows, (vocab, hidden) = ids.shape[0], table.shape
     # (the one-launch kernel addresses table rows with 32-bit byte offsets: tables of 4 GiB and more take the two launches)
     fused = 0 < rows <= EMBED_FUSED_MAX_ROWS and hidden == 2880 and head_dim == 64 and vocab * hidden * 2 < 2 ** 32
     if x_out is None:
         x_out = torch.empty(rows, hidden, dtype=_BF16, device=table.device)
-    assert x_out.shape == (rows, hidden) and x_out.dtype == _BF16 and x_out.is_contiguous()
+    _require(x_out.shape == (rows, hidden) and x_out.dtype == _BF16 and x_out.is_contiguous())
     if not fused:
         embedding_forward(ids, table, out=x_out, oob_flag=oob_flag)
         q, k, v = qkv_rope_forward(x_out, weight, bias, num_q_heads, num_kv_heads, head_dim, yarn=yarn, cos=cos, sin=sin,
@@ -408,13 +409,13 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
                                    max_context_length=max_context_length, rotate=rotate, out=out, norm_scale=norm_scale,
                                    norm_eps=norm_eps, weight_scale=weight_scale)
         return x_out, q, k, v
-    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
+    _require((weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none")
     total_out, hidden_w = weight.shape
-    assert hidden == hidden_w and total_out == (num_q_heads + 2 * num_kv_heads) * head_dim
-    assert bias is None or bias.shape == (total_out,)
-    assert norm_scale.dtype in (torch.float32, _BF16) and norm_scale.shape == (hidden,)
+    _require(hidden == hidden_w and total_out == (num_q_heads + 2 * num_kv_heads) * head_dim)
+    _require(bias is None or bias.shape == (total_out,))
+    _require(norm_scale.dtype in (torch.float32, _BF16) and norm_scale.shape == (hidden,))
     if oob_flag is not None:
-        assert oob_flag.dtype == torch.int32 and oob_flag.numel() == 1
+        _require(oob_flag.dtype == torch.int32 and oob_flag.numel() == 1)
     ids = ids if ids.is_contiguous() else ids.contiguous()
     norm_scale = norm_scale if norm_scale.is_contiguous() else norm_scale.contiguous()
     _, weight, bias = _prep_linear(x_out, weight, bias)
@@ -426,8 +427,8 @@ def embed_qkv_rope_forward(ids: torch.Tensor, table: torch.Tensor, norm_scale: t
         k, v = kv[0], kv[1]
     else:
         q, k, v = out
-        assert q.shape == (rows, q_dim) and k.shape == (rows, kv_dim) and v.shape == (rows, kv_dim)
-        assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1
+        _require(q.shape == (rows, q_dim) and k.shape == (rows, kv_dim) and v.shape == (rows, kv_dim))
+        _require(q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1)
     keep: list = []
     desc = None
     if rotate:
@@ -447,7 +448,7 @@ def _split_head_dim(q_dim: int, kv_dim: int) -> int:
     if q_dim % 64 == 0 and kv_dim % 64 == 0:
         return 64
     g = math.gcd(q_dim, kv_dim)
-    assert g % 2 == 0, "q_dim and kv_dim need a common even divisor"
+    _require(g % 2 == 0, "q_dim and kv_dim need a common even divisor")
     return g
 
 
@@ -456,11 +457,11 @@ def qkv_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias: torch.T
     _on_gpu(hidden, weight, bias)
     batch, num_tokens, hidden_size = hidden.shape
     total_out, hidden_size_weight = weight.shape
-    assert num_tokens == 1
-    assert hidden_size == hidden_size_weight
-    assert bias.shape == (total_out,)
-    assert total_out == q_dim + 2 * kv_dim
-    assert weight.dtype == _BF16
+    _require(num_tokens == 1)
+    _require(hidden_size == hidden_size_weight)
+    _require(bias.shape == (total_out,))
+    _require(total_out == q_dim + 2 * kv_dim)
+    _require(weight.dtype == _BF16)
     x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
     hd = _split_head_dim(q_dim, kv_dim)
     q = _pooled_output((batch, q_dim), hidden.dtype, hidden.device, x2)
@@ -480,21 +481,21 @@ def qkv_rope_cache_decode_forward(hidden, weight, bias, sin, cos, max_context_le
     on the device, so the call can be replayed from a HIP graph. With ``norm_scale`` the
     block's input RMSNorm (model.py:476) runs inside the same kernel on the raw ``hidden``."""
     _on_gpu(hidden, weight, bias, cache_k, cache_v, offset, positions, norm_scale, weight_scale)
-    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
+    _require((weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none")
     batch, num_tokens, hidden_size = hidden.shape
     total_out, hidden_size_weight = weight.shape
-    assert num_tokens == 1
-    assert hidden_size == hidden_size_weight
-    assert total_out == (num_q_heads + 2 * num_kv_heads) * head_dim
-    assert bias.shape == (total_out,)
-    assert cache_k.shape == cache_v.shape
-    assert cache_k.shape[0] == batch
-    assert cache_k.shape[2] == num_kv_heads
-    assert cache_k.shape[3] == head_dim
-    assert offset.shape == (1,)
-    assert cache_k.dtype == _BF16 and cache_v.dtype == _BF16
-    assert cache_k.stride() == cache_v.stride()
-    assert cache_k.stride(3) == 1 and cache_k.stride(2) == head_dim, "KV cache must be dense over (heads, head_dim)"
+    _require(num_tokens == 1)
+    _require(hidden_size == hidden_size_weight)
+    _require(total_out == (num_q_heads + 2 * num_kv_heads) * head_dim)
+    _require(bias.shape == (total_out,))
+    _require(cache_k.shape == cache_v.shape)
+    _require(cache_k.shape[0] == batch)
+    _require(cache_k.shape[2] == num_kv_heads)
+    _require(cache_k.shape[3] == head_dim)
+    _require(offset.shape == (1,))
+    _require(cache_k.dtype == _BF16 and cache_v.dtype == _BF16)
+    _require(cache_k.stride() == cache_v.stride())
+    _require(cache_k.stride(3) == 1 and cache_k.stride(2) == head_dim, "KV cache must be dense over (heads, head_dim)")
     x2, weight, bias = _prep_linear(hidden.reshape(batch, hidden_size), weight, bias)
     q = _pooled_output((batch, num_q_heads, head_dim), hidden.dtype, hidden.device, x2)
     keep: list = []
@@ -511,11 +512,11 @@ def linear_qkv_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     through the MFMA kernel (or the streaming kernel for few rows), writing one dense output."""
     _on_gpu(x, weight, bias)
     total_out, hidden = weight.shape
-    assert x.shape[-1] == hidden and weight.dtype == _BF16
+    _require(x.shape[-1] == hidden and weight.dtype == _BF16)
     x2, weight, bias = _prep_linear(x.reshape(-1, hidden), weight, bias)
     rows = x2.shape[0]
     hd = 64 if total_out % 64 == 0 else 2
-    assert total_out % hd == 0
+    _require(total_out % hd == 0)
     out = torch.empty((*x.shape[:-1], total_out), dtype=x.dtype, device=x.device)
     o2 = out.view(rows, total_out)
     mode = "decode" if rows <= _decode_max_rows(hidden, hd) else "prefill"
@@ -534,13 +535,13 @@ def out_residual_decode_forward(hidden: torch.Tensor, weight: torch.Tensor, bias
     _on_gpu(hidden, weight, bias, residual, weight_scale)
     batch, num_tokens, out_dim_hidden = hidden.shape
     hidden_size, out_dim_weight = weight.shape
-    assert num_tokens == 1
-    assert out_dim_hidden == out_dim_weight
-    assert bias.shape == (hidden_size,)
-    assert residual.shape == (batch, 1, hidden_size)
-    assert hidden.dtype == _BF16 and bias.dtype == _BF16 and residual.dtype == _BF16
-    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
-    assert weight.dtype in (_BF16, _FP8)
+    _require(num_tokens == 1)
+    _require(out_dim_hidden == out_dim_weight)
+    _require(bias.shape == (hidden_size,))
+    _require(residual.shape == (batch, 1, hidden_size))
+    _require(hidden.dtype == _BF16 and bias.dtype == _BF16 and residual.dtype == _BF16)
+    _require((weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none")
+    _require(weight.dtype in (_BF16, _FP8))
     x2 = hidden.reshape(batch, out_dim_hidden)
     res2 = residual.reshape(batch, hidden_size)
     if not x2.is_contiguous():
@@ -565,11 +566,11 @@ def _unembed_prep(hidden, weight, weight_scale):
     _on_gpu(hidden, weight, weight_scale)
     batch, num_tokens, hidden_size = hidden.shape
     vocab_size, hidden_size_weight = weight.shape
-    assert num_tokens == 1
-    assert hidden_size == hidden_size_weight
-    assert hidden.dtype == _BF16
-    assert (weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none"
-    assert weight.dtype in (_BF16, _FP8)
+    _require(num_tokens == 1)
+    _require(hidden_size == hidden_size_weight)
+    _require(hidden.dtype == _BF16)
+    _require((weight.dtype == _FP8) == (weight_scale is not None), "a float8 weight needs weight_scale, a bfloat16 one takes none")
+    _require(weight.dtype in (_BF16, _FP8))
     x2 = hidden.reshape(batch, hidden_size)
     if not x2.is_contiguous():
         x2 = x2.contiguous()
@@ -659,18 +660,18 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: t
     are visible, e.g. the decode loop's position + 1) plans the launch for that length instead, which is faster when
     the context is far shorter than the cache; the result never depends on it."""
     _on_gpu(q, k, v, sinks, start_q)
-    assert len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64)
+    _require(len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64))
     bs, n_ctx, n_kv_heads, repeat_kv, head_dim_q = q.shape
     bs_k, n_kv_ctx, n_kv_heads_k, head_dim_k = k.shape
     bs_v, n_kv_ctx_v, n_kv_heads_v, head_dim_v = v.shape
-    assert n_ctx == 1
-    assert bs == bs_k == bs_v and n_kv_ctx == n_kv_ctx_v
-    assert n_kv_heads == n_kv_heads_k == n_kv_heads_v
-    assert head_dim_q == head_dim_k == head_dim_v
-    assert head_dim_q in {16, 32, 64, 128, 256}
+    _require(n_ctx == 1)
+    _require(bs == bs_k == bs_v and n_kv_ctx == n_kv_ctx_v)
+    _require(n_kv_heads == n_kv_heads_k == n_kv_heads_v)
+    _require(head_dim_q == head_dim_k == head_dim_v)
+    _require(head_dim_q in {16, 32, 64, 128, 256})
     if head_dim_q != 64 or repeat_kv > 16:
         raise NotImplementedError("attention_decode: the HIP kernel is built for head_dim 64 and up to 16 query heads per KV head")
-    assert q.dtype == _BF16 and k.dtype == _BF16 and v.dtype == _BF16 and (sinks is None or sinks.dtype == _BF16)
+    _require(q.dtype == _BF16 and k.dtype == _BF16 and v.dtype == _BF16 and (sinks is None or sinks.dtype == _BF16))
     n_heads = n_kv_heads * repeat_kv
     q2 = q[:, 0].reshape(bs, n_heads * 64)
     if not q2.is_contiguous():
@@ -683,7 +684,7 @@ def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: t
     if k.stride() != v.stride():
         k, v = k.contiguous(), v.contiguous()
     if sinks is not None:
-        assert sinks.shape == (n_heads,)
+        _require(sinks.shape == (n_heads,))
         sinks = sinks if sinks.is_contiguous() else sinks.contiguous()
     window = int(bandwidth) if bandwidth else 0
     o = scratch_pool.get((bs, n_heads * 64), q.dtype, q.device)
@@ -709,17 +710,17 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Te
     ``q`` may be a view into the fused QKV output and ``k`` / ``v`` views of the cache: the kernel takes batch and
     token strides, so none of the reference's transposed, padded copies (:180-191) is made."""
     _on_gpu(q, k, v, sinks, start_q)
-    assert len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64)
+    _require(len(start_q) == 1 and start_q.dtype in (torch.int32, torch.int64))
     bs, n_ctx, n_kv_heads, repeat_kv, head_dim_q = q.shape
     bs_k, n_kv_ctx, n_kv_heads_k, head_dim_k = k.shape
     bs_v, n_kv_ctx_v, n_kv_heads_v, head_dim_v = v.shape
-    assert bs == bs_k == bs_v and n_kv_ctx == n_kv_ctx_v
-    assert n_kv_heads == n_kv_heads_k == n_kv_heads_v
-    assert head_dim_q == head_dim_k == head_dim_v
-    assert head_dim_q in {16, 32, 64, 128, 256}
+    _require(bs == bs_k == bs_v and n_kv_ctx == n_kv_ctx_v)
+    _require(n_kv_heads == n_kv_heads_k == n_kv_heads_v)
+    _require(head_dim_q == head_dim_k == head_dim_v)
+    _require(head_dim_q in {16, 32, 64, 128, 256})
     if head_dim_q != 64:
         raise NotImplementedError("attention: the HIP kernel is built for head_dim 64")
-    assert q.dtype == _BF16 and k.dtype == _BF16 and v.dtype == _BF16 and (sinks is None or sinks.dtype == _BF16)
+    _require(q.dtype == _BF16 and k.dtype == _BF16 and v.dtype == _BF16 and (sinks is None or sinks.dtype == _BF16))
     n_heads = n_kv_heads * repeat_kv
 
     def dense_q(t):
@@ -735,7 +736,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: torch.Te
     if k.stride() != v.stride():
         k, v = k.contiguous(), v.contiguous()
     if sinks is not None:
-        assert sinks.shape == (n_heads,)
+        _require(sinks.shape == (n_heads,))
         sinks = sinks if sinks.is_contiguous() else sinks.contiguous()
     window = int(bandwidth) if bandwidth else 0
     o = scratch_pool.get((bs, n_ctx, n_heads * 64), q.dtype, q.device)
@@ -755,9 +756,9 @@ def mxfp4_dequant(blocks: torch.Tensor, scales: torch.Tensor, out: torch.Tensor 
     given, must be a contiguous bf16 tensor of that many elements (it is filled in place, so a caller can expand
     straight into a slice of a preallocated parameter)."""
     _on_gpu(blocks, scales, out)
-    assert blocks.dtype == torch.uint8 and scales.dtype == torch.uint8, "MXFP4 blocks and scales are uint8"
-    assert blocks.shape[:-1] == scales.shape, f"{blocks.shape=} does not match {scales.shape=}"
-    assert blocks.shape[-1] == 16, "an MXFP4 block is 16 bytes"
+    _require(blocks.dtype == torch.uint8 and scales.dtype == torch.uint8, "MXFP4 blocks and scales are uint8")
+    _require(blocks.shape[:-1] == scales.shape, f"{blocks.shape=} does not match {scales.shape=}")
+    _require(blocks.shape[-1] == 16, "an MXFP4 block is 16 bytes")
     *prefix, G, B = blocks.shape
     blocks = blocks.contiguous()
     scales = scales.contiguous()
@@ -766,6 +767,6 @@ def mxfp4_dequant(blocks: torch.Tensor, scales: torch.Tensor, out: torch.Tensor 
     if out is None:
         out = torch.empty(shape, dtype=_BF16, device=blocks.device)
     else:
-        assert out.dtype == _BF16 and out.is_contiguous() and out.numel() == n_blocks * 32, "out must be contiguous bf16 of 32 values per block"
+        _require(out.dtype == _BF16 and out.is_contiguous() and out.numel() == n_blocks * 32, "out must be contiguous bf16 of 32 values per block")
     check(lib().tllm_mxfp4_dequant_bf16(blocks.data_ptr(), scales.data_ptr(), out.data_ptr(), n_blocks, _stream()), "mxfp4_dequant")
     return out.view(shape) if out.shape != torch.Size(shape) else out

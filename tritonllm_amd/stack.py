@@ -21,6 +21,7 @@ from __future__ import annotations
 import torch
 
 from . import ops
+from ._lib import require as _require
 from .yarn import YarnParams
 
 
@@ -33,7 +34,7 @@ class LayerKernelStack:
         q / k / v / MLP-norm / SwiGLU buffers (``[L, ...]``; for checking), otherwise one set is reused by all layers.
         ``fuse_norm=False`` runs the attention norm as its own launch at every row count."""
         self.n_layers = len(weights)
-        assert len(biases) == len(attn_scales) == len(mlp_scales) == self.n_layers
+        _require(len(biases) == len(attn_scales) == len(mlp_scales) == self.n_layers)
         self.weights, self.biases, self.attn_scales, self.mlp_scales, self.final_scale = weights, biases, attn_scales, mlp_scales, final_scale
         self.yarn, self.batch, self.eps, self.fuse_norm = yarn, batch, eps, fuse_norm
         self.nq, self.nkv, self.hd = num_q_heads, num_kv_heads, head_dim
@@ -55,7 +56,7 @@ class LayerKernelStack:
     def token_step(self, x: torch.Tensor, positions: torch.Tensor, swiglu_x: torch.Tensor) -> torch.Tensor:
         """``x [B, hidden]`` bf16 (the residual stream), ``positions [B]`` int64 on the device, ``swiglu_x [4 * B,
         2 * hidden]`` bf16 (interleaved gate / linear). Returns the final-norm output ``[B, hidden]`` (owned by the stack)."""
-        assert x.shape == (self.batch, self.hidden) and swiglu_x.shape == (4 * self.batch, 2 * self.hidden)
+        _require(x.shape == (self.batch, self.hidden) and swiglu_x.shape == (4 * self.batch, 2 * self.hidden))
         for l in range(self.n_layers):
             i = l % self._n
             out = (self.q[i], self.k[i], self.v[i])

@@ -9,6 +9,7 @@ from dataclasses import dataclass
 import torch
 
 from . import ops
+from ._lib import require as _require
 
 
 @dataclass(frozen=True)
@@ -20,6 +21,6 @@ def swiglu(a: torch.Tensor, alpha: float, precision_config: PrecisionConfig, rou
     """triton_kernels/swiglu.py:85-86. Always the interleaved layout; returns a fresh tensor."""
     if routing_data is not None:
         raise NotImplementedError("routing_data (ragged expert batches) is outside the bf16 layer-kernel path")
-    assert a.stride()[-1] == 1
-    assert a.shape[-1] % 2 == 0
+    _require(a.stride()[-1] == 1)
+    _require(a.shape[-1] % 2 == 0)
     return ops.swiglu(a, alpha=alpha, limit=precision_config.limit, interleaved=True)

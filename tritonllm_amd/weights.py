@@ -15,6 +15,7 @@ import torch
 from safetensors import safe_open
 
 from . import ops
+from ._lib import require as _require
 
 # Bytes per MXFP4 block: 32 FP4 numbers in 16 bytes (weights.py:8-9)
 BYTES_PER_BLOCK = 16
@@ -57,17 +58,17 @@ class Checkpoint:
         return t
 
     def _get_tensor(self, name: str) -> torch.Tensor:
-        assert name in self.tensor_name_to_file, f"Tensor {name} not found in checkpoint."
+        _require(name in self.tensor_name_to_file, f"Tensor {name} not found in checkpoint.")
         with safe_open(self.tensor_name_to_file[name], framework="pt", device=self.device_str) as f:
             return f.get_tensor(name)
 
     def _get_mxfp4_tensor(self, blocks_name: str, scales_name: str, *, dtype: torch.dtype = torch.bfloat16,
                           out: torch.Tensor | None = None) -> torch.Tensor:
-        assert blocks_name in self.tensor_name_to_file, f"Blocks tensor {blocks_name} not found in checkpoint."
-        assert scales_name in self.tensor_name_to_file, f"Scales tensor {scales_name} not found in checkpoint."
+        _require(blocks_name in self.tensor_name_to_file, f"Blocks tensor {blocks_name} not found in checkpoint.")
+        _require(scales_name in self.tensor_name_to_file, f"Scales tensor {scales_name} not found in checkpoint.")
         if dtype != torch.bfloat16:
             raise NotImplementedError("MXFP4 tensors expand to bfloat16 only")
         blocks = self._get_tensor(blocks_name)
         scales = self._get_tensor(scales_name)
-        assert blocks.shape[:-1] == scales.shape, f"{blocks.shape=} does not match {scales.shape=}"
+        _require(blocks.shape[:-1] == scales.shape, f"{blocks.shape=} does not match {scales.shape=}")
         return ops.mxfp4_dequant(blocks, scales, out=out)

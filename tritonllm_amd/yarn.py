@@ -14,6 +14,7 @@ from dataclasses import dataclass, field
 import torch
 
 from ._lib import MAX_ROPE_FREQS, TllmYarn
+from ._lib import require as _require
 
 
 @dataclass(frozen=True)
@@ -61,7 +62,7 @@ def _concentration_and_inv_freq(head_dim, base, initial_context_length, scaling_
         d_half = head_dim / 2
         low = d_half * math.log(initial_context_length / (ntk_beta * 2 * math.pi)) / math.log(base)
         high = d_half * math.log(initial_context_length / (ntk_alpha * 2 * math.pi)) / math.log(base)
-        assert 0 < low < high < d_half - 1
+        _require(0 < low < high < d_half - 1)
         interpolation = 1.0 / (scaling_factor * freq)
         extrapolation = 1.0 / freq
         ramp = (torch.arange(d_half, dtype=torch.float32) - low) / (high - low)
