@@ -7,12 +7,17 @@
 // loaded from global memory straight into LDS with the XOR swizzle chosen on the global side, fragments read back
 // once, partial tiles reduced in a fixed order by epilogue wavefronts that fetched bias and residual meanwhile.
 // What differs: 32 activation rows are 256 KB per workgroup, more than the LDS holds, so the activations arrive in
-// phases with the weight. Four streaming wavefronts, each with 1024 of the 4096 K: 32 k32 steps in eight phases of
-// four; in phase p the four together read 1024 contiguous bytes of every row (wavefront kq the 256 bytes at
-// p * 1024 + kq * 256). A phase of a wavefront is 8 KB of activations (32 rows x 256 bytes) and 3 KB of weight,
-// through a ring of three 11 KB regions: three phases are in flight, a phase is multiplied as soon as it has landed
-// and its region is then refilled with the phase three further on (a ring of two measures 1 % slower: the depth is
-// not what bounds the kernel). Two epilogue wavefronts, one per column block.
+// phases. Four streaming wavefronts, each with 1024 of the 4096 K: 32 k32 steps in eight phases of four; in phase p
+// the four together read 1024 contiguous bytes of every row (wavefront kq the 256 bytes at p * 1024 + kq * 256). A
+// phase of a wavefront is 8 KB of activations (32 rows x 256 bytes) and 3 KB of weight. The weight -- the operand that
+// comes from HBM -- is requested whole at the start, every phase into a place of its own (24 KB per wavefront); the
+// activations, which come from the L2s, pass a ring of two 8 KB regions, a region being refilled with the phase two
+// further on as soon as its fragments are in registers. A CU returns loads in the order it took them, so the third
+// activation phase arrives behind the last of the weight and the rest follow one L2 round trip per pair; with the
+// weight in a ring as well (three phases of both operands resident) its requests trickle out behind the MFMAs and
+// the launch takes 8.5 us at 32 rows instead of 8.1 (five or six weight phases resident: 8.35 / 8.25; a third
+// activation region ahead of the weight's later phases: 6.80 against 6.73 us with the fp8 weight). Two epilogue
+// wavefronts, one per column block.
 // W8: fp8 (OCP e4m3) weight with one fp32 scale per output row (the reference's ATTN_FP8 option,
 // triton_kernels.py:1385-1408): a weight row of a phase is 128 bytes (two loads of eight rows), fragments are widened
 // to bf16 (exact) between the LDS read and the MFMA, the row scale multiplies the finished sum.
@@ -28,18 +33,43 @@ constexpr int NS = 4;             // streaming wavefronts = K slices
 constexpr int NE = 2;             // epilogue wavefronts = column blocks
 constexpr int RW = 12;            // weight rows (output features) per workgroup
 constexpr int NPH = 8;            // phases of four k32 steps
-constexpr int RING = 3;           // resident phases per wavefront
+constexpr int WRING = NPH;        // every phase of the weight is requested at once and has a place of its own
 constexpr int XPH = 8 * 1024;     // activations of one phase: 32 rows x four k32 steps
-constexpr int WPH = 3 * 1024;     // weight of one phase: 12 rows x four k32 steps
-constexpr int REGION = XPH + WPH;
+constexpr int WAVE_LDS = 40 * 1024;   // a wavefront's activation ring, then its weight: 2 x 8 + 8 x 3 KB
+static_assert(NS * WAVE_LDS <= 160 * 1024, "the rings fit the LDS");
+
+// Load instructions that may still be outstanding when phase p is multiplied: those requested after the phase's own
+// last load. The order of requests: x(0) W(0) x(1) W(1) ... while both rings fill, then behind each phase p
+// x(p + xring) (and W(p + WRING), if the weight had a ring shorter than its phases).
+constexpr int younger_than_phase(int p, int xb, int lw, int xring) {
+  int count = 0, last = 0;
+  const int pro = xring > WRING ? xring : WRING;
+  for (int i = 0; i < pro; ++i) {
+    if (i < xring && i < NPH) { count += xb; if (i == p) last = count; }
+    if (i < WRING && i < NPH) { count += lw; if (i == p) last = count; }
+  }
+  for (int q = 0; q < p; ++q) {
+    if (q + xring < NPH) { count += xb; if (q + xring == p) last = count; }
+    if (q + WRING < NPH) { count += lw; if (q + WRING == p) last = count; }
+  }
+  return count - last;
+}
+static_assert(NPH == 8, "the wait of each phase is spelled out below");
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "s_waitcnt vmcnt takes six bits");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 }  // namespace r32o
 
 template <int XB, bool W8>
 __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8) {
   using namespace r32o;
   constexpr int LW = W8 ? 2 : 3;                            // weight load instructions per phase
-  constexpr int LPP = XB + LW;                              // load instructions per phase
-  __shared__ __align__(1024) unsigned char ring[NS * RING * REGION];
+  constexpr int XRING = 2;                                  // phases of activations resident per wavefront
+  constexpr int WPH = 3 * 1024;                             // weight of one phase: 12 rows x four k32 steps (fp8: 2 KB of it)
+  static_assert(XRING * XPH + WRING * WPH <= WAVE_LDS, "a wavefront's rings fit its share of the LDS");
+  __shared__ __align__(1024) unsigned char ring[NS * WAVE_LDS];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -97,7 +127,7 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     __syncthreads();                                        // partial tiles are in LDS
     f32x4 t[NS];
 #pragma unroll
-    for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(ring + w * (RING * REGION) + red_o);
+    for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(ring + w * WAVE_LDS + red_o);
     f32x4 acc = t[0];
 #pragma unroll
     for (int w = 1; w < NS; ++w) {                          // fixed order: the result does not depend on timing
@@ -122,7 +152,7 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   // ========================================================================= streaming wavefront of K slice `kq`
   const int kq = wave;
   const int m = lane & 15, g = lane >> 4;
-  unsigned char* myring = ring + wave * (RING * REGION);
+  unsigned char* myring = ring + wave * WAVE_LDS;
 
   // lane -> (row of a 4-row block, position): it fetches chunk position ^ (row & 15) of that row's 256 bytes, so that
   // the 16 rows a fragment read touches lie in 16 different bank groups
@@ -149,29 +179,35 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x) + row0 * 8192;
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
-  auto issue_phase = [&](int p) {                           // the activations of the phase, then its weight
-    unsigned char* reg = myring + (p % RING) * REGION;
+  auto x_region = [&](int p) { return myring + (p % XRING) * XPH; };
+  auto w_region = [&](int p) { return myring + XRING * XPH + (p % WRING) * WPH; };
+  auto issue_x = [&](int p) {
     const unsigned char* xb = xbase + p * 1024;
-    const unsigned char* wb = wbase + p * (W8 ? 512 : 1024);
 #pragma unroll
     for (int j = 0; j < XB; ++j) {
-      const unsigned dst = lds_addr(reg + j * 1024);
+      const unsigned dst = lds_addr(x_region(p) + j * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[j]), "s"(xb) : "memory", "m0");
     }
+  };
+  auto issue_w = [&](int p) {
+    const unsigned char* wb = wbase + p * (W8 ? 512 : 1024);
 #pragma unroll
     for (int j = 0; j < LW; ++j) {
-      const unsigned dst = lds_addr(reg + XPH + j * 1024);
+      const unsigned dst = lds_addr(w_region(p) + j * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff[j]), "s"(wb) : "memory", "m0");
     }
   };
 #pragma unroll
-  for (int p = 0; p < RING; ++p) issue_phase(p);
+  for (int p = 0; p < (XRING > WRING ? XRING : WRING); ++p) {
+    if (p < XRING && p < NPH) issue_x(p);
+    if (p < WRING && p < NPH) issue_w(p);
+  }
 
   f32x4 acc[2];                                             // [column block]
   acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
   acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int arow = m < RW ? m : m - RW;                     // tile rows past the twelfth re-read a real one (their sums are dropped)
-  const unsigned a_o = XPH + arow * (W8 ? 128 : 256);
+  const unsigned a_o = arow * (W8 ? 128 : 256);
   // W8: the lane's eight fp8 of step st are bytes 32 st + 8 g of the 128-byte row: half g & 1 of chunk 2 st + g / 2,
   // which sits at position chunk ^ (row & 7)
   auto w8frag = [&](const unsigned char* reg, int st) {
@@ -182,23 +218,31 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   const unsigned b0_o = m * 256, b1_o = (16 + m) * 256;
 #pragma unroll
   for (int p = 0; p < NPH; ++p) {
-    // phase p has landed when only the loads of the phases after it that have been requested are outstanding
-    constexpr int kTwo = 2 * LPP, kOne = LPP;
-    if (p < NPH - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kTwo) : "memory");
-    else if (p == NPH - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kOne) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    const unsigned char* reg = myring + (p % RING) * REGION;
+    // phase p has landed when only the loads requested after its own are outstanding
+    switch (p) {                                            // (p is a constant of the unrolled loop; an asm operand must be one by the language's rules)
+      case 0: wait_vmcnt<younger_than_phase(0, XB, LW, XRING)>(); break;
+      case 1: wait_vmcnt<younger_than_phase(1, XB, LW, XRING)>(); break;
+      case 2: wait_vmcnt<younger_than_phase(2, XB, LW, XRING)>(); break;
+      case 3: wait_vmcnt<younger_than_phase(3, XB, LW, XRING)>(); break;
+      case 4: wait_vmcnt<younger_than_phase(4, XB, LW, XRING)>(); break;
+      case 5: wait_vmcnt<younger_than_phase(5, XB, LW, XRING)>(); break;
+      case 6: wait_vmcnt<younger_than_phase(6, XB, LW, XRING)>(); break;
+      default: wait_vmcnt<younger_than_phase(7, XB, LW, XRING)>(); break;
+    }
+    const unsigned char* reg = x_region(p);
+    const unsigned char* wreg = w_region(p);
     bf16x8 fa[4], fb0[4], fb1[4];
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
-      if constexpr (W8) fa[st] = w8frag(reg, st);
-      else fa[st] = *reinterpret_cast<const bf16x8*>(reg + a_o + (((4 * st + g) ^ arow) << 4));
+      if constexpr (W8) fa[st] = w8frag(wreg, st);
+      else fa[st] = *reinterpret_cast<const bf16x8*>(wreg + a_o + (((4 * st + g) ^ arow) << 4));
       fb0[st] = *reinterpret_cast<const bf16x8*>(reg + b0_o + (((4 * st + g) ^ m) << 4));
       if constexpr (XB > 4) fb1[st] = *reinterpret_cast<const bf16x8*>(reg + b1_o + (((4 * st + g) ^ m) << 4));
     }
-    if (p + RING < NPH) {
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the region's fragments are in registers: it may be refilled
-      issue_phase(p + RING);
+    if (p + XRING < NPH || p + WRING < NPH) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the regions' fragments are in registers: they may be refilled
+      if (p + XRING < NPH) issue_x(p + XRING);
+      if (p + WRING < NPH) issue_w(p + WRING);
     }
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
