@@ -624,11 +624,12 @@ def main() -> int:
                              nb4k, n=96)
             del ak, av
         # unembedding over the full vocabulary (the embedding table doubles as the [201088, 2880] weight: 1.16 GB per launch)
-        for r in (1, 8):
+        for r in (1, 8, 32):
             ux = torch.empty(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
             bench_kernel(f"unembedding_decode_B{r}", lambda i, ux=ux: T.unembedding_decode_forward(ux, table), bytes_of["unembed"](r), n=24)
             bench_kernel(f"unembedding_argmax_B{r}", lambda i, ux=ux: T.unembedding_decode_argmax_forward(ux, table),
                          bytes_of["unembed_argmax"](r), n=24)
+        ux = torch.empty(8, 1, HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
         uw8, uws = T.quantize_fp8_rows(table)
         bench_kernel("unembedding_decode_w8_B8", lambda i, ux=ux: T.unembedding_decode_forward(ux, uw8, uws), bytes_of["unembed_w8"](8), n=24)
         del uw8, uws

@@ -228,7 +228,8 @@ int tllm_out_residual_decode_bf16(const void* x, const void* W, const float* w_s
  * RNE to bf16); replaces unembedding_decode_forward(hidden, weight), triton_kernels.py:163-197 (kernel :111-160),
  * and with w_scale != NULL unembedding_decode_fp8_forward :271-302 (W = fp8 e4m3 bytes, one fp32 scale per
  * vocabulary row, as quantised by :261-268). x [rows, hidden] bf16 dense, W [vocab, hidden] dense, logits
- * [rows, vocab] with logits_row_stride elements between rows. hidden must be a multiple of 64. */
+ * [rows, vocab] with logits_row_stride elements between rows. hidden must be a multiple of 64. One pass over the
+ * weight serves up to 32 rows with a bf16 weight (up to 16 with fp8); more rows take one pass per 32 (16). */
 int tllm_unembedding_decode_bf16(const void* x, const void* W, const float* w_scale, void* logits,
                                  int64_t logits_row_stride, int64_t rows, int64_t hidden, int64_t vocab, void* stream);
 

@@ -1016,6 +1016,48 @@ def test_unembedding_other_hidden_sizes(gpu, rows, hidden):
     _argmax_ok(T.unembedding_decode_fp8_argmax_forward(xg, w8, ws), want8)
 
 
+@pytest.mark.parametrize("rows,vocab,hidden", [(17, 3001, 2880), (32, 140000, 2880), (33, 70001, 2880), (50, 4096, 2880), (64, 9000, 2880),
+                                                (24, 5000, 128), (32, 5000, 192), (29, 5000, 1024)])
+def test_unembedding_more_than_16_rows_one_pass_over_the_weight(gpu, rows, vocab, hidden):
+    """Above sixteen rows a workgroup takes 32 batch rows and keeps one K half of them in LDS at a time; a wavefront's
+    tiles wait in registers between the halves. Vocabularies that give a wavefront 0, 1, 2, 3 and 4 tiles (2048
+    wavefronts), ragged last tiles, ragged last chunks of rows, K halves of equal and unequal length (hidden / 64 odd),
+    logits and argmax."""
+    g = torch.Generator().manual_seed(990 + rows + hidden)
+    x = torch.randn(rows, hidden, generator=g).bfloat16()
+    w = ((0.02 if hidden == 2880 else 0.05) * torch.randn(vocab, hidden, generator=g)).bfloat16()
+    planted = torch.randint(0, vocab, (rows,), generator=g)
+    planted[0], planted[-1] = vocab - 1, 0
+    for r in range(rows):                                      # row r of x points at weight row planted[r] ...
+        w[planted[r]] = (x[r].float() * 0.05).bfloat16()
+    xg = x.view(rows, 1, hidden).to(gpu)
+    logits = T.unembedding_decode_forward(xg, w.to(gpu))
+    want = O.linear_ref(x, w, None)
+    close(logits.view(rows, vocab), want)
+    ids = T.unembedding_decode_argmax_forward(xg, w.to(gpu))
+    _argmax_ok(ids, want)
+
+
+def test_unembedding_32_rows_full_vocabulary(gpu):
+    """[201088, 2880] at 32 rows: three or four tiles per wavefront. Logits against the oracle on a sample of columns,
+    argmax against planted winners."""
+    vocab, rows = 201088, 32
+    gg = torch.Generator(device=gpu).manual_seed(5)
+    w = torch.empty(vocab, 2880, dtype=torch.bfloat16, device=gpu).normal_(0, 0.02, generator=gg)
+    g = torch.Generator().manual_seed(72)
+    x = torch.randn(rows, 2880, generator=g).bfloat16()
+    planted = torch.randint(0, vocab, (rows,), generator=g)
+    planted[:6] = torch.tensor([0, 31, 32, 201087, 201056, 65535])
+    for r in range(rows):
+        w[planted[r]] = (x[r].float() * 0.05).bfloat16().to(gpu)
+    xg = x.view(rows, 1, 2880).to(gpu)
+    logits = T.unembedding_decode_forward(xg, w).view(rows, vocab)
+    cols = torch.cat([torch.arange(0, 64), torch.arange(100000, 100064), torch.arange(vocab - 64, vocab), planted])
+    close(logits[:, cols.to(gpu)], O.linear_ref(x, w[cols.to(gpu)].cpu(), None))
+    assert torch.equal(logits.float().argmax(dim=-1).cpu(), planted)
+    assert torch.equal(T.unembedding_decode_argmax_forward(xg, w).cpu().long(), planted)
+
+
 def test_unembedding_full_vocabulary_and_module(gpu, monkeypatch):
     """The real size: [201088, 2880]. Logits against the oracle on a sample of columns (the full fp32 product on
     the CPU would take minutes), argmax against a planted winner, and the module's dispatch."""
