@@ -229,7 +229,7 @@ int tllm_out_residual_decode_bf16(const void* x, const void* W, const float* w_s
  * and with w_scale != NULL unembedding_decode_fp8_forward :271-302 (W = fp8 e4m3 bytes, one fp32 scale per
  * vocabulary row, as quantised by :261-268). x [rows, hidden] bf16 dense, W [vocab, hidden] dense, logits
  * [rows, vocab] with logits_row_stride elements between rows. hidden must be a multiple of 64. One pass over the
- * weight serves up to 32 rows with a bf16 weight (up to 16 with fp8); more rows take one pass per 32 (16). */
+ * weight serves up to 32 rows; more rows take one pass per 32. */
 int tllm_unembedding_decode_bf16(const void* x, const void* W, const float* w_scale, void* logits,
                                  int64_t logits_row_stride, int64_t rows, int64_t hidden, int64_t vocab, void* stream);
 

@@ -1036,6 +1036,11 @@ def test_unembedding_more_than_16_rows_one_pass_over_the_weight(gpu, rows, vocab
     close(logits.view(rows, vocab), want)
     ids = T.unembedding_decode_argmax_forward(xg, w.to(gpu))
     _argmax_ok(ids, want)
+    # the fp8 weight takes the same path above sixteen rows
+    w8, ws = T.quantize_fp8_rows(w.to(gpu))
+    want8 = O.linear_ref(x, O.dequant_fp8_ref(w8.cpu(), ws.cpu()), None)
+    close(T.unembedding_decode_fp8_forward(xg, w8, ws).view(rows, vocab), want8)
+    _argmax_ok(T.unembedding_decode_fp8_argmax_forward(xg, w8, ws), want8)
 
 
 def test_unembedding_32_rows_full_vocabulary(gpu):

@@ -311,7 +311,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
   }
 }
 
-// Thirty-two batch rows per workgroup (bf16 weight): 32 activation rows of gpt-oss's width are 184 KB, more than the
+// Thirty-two batch rows per workgroup (bf16 or fp8 weight): 32 activation rows of gpt-oss's width are 184 KB, more than the
 // LDS holds, and chunks of sixteen stream the weight once per chunk. Here the workgroup keeps one K half of its 32
 // rows in LDS at a time: every wavefront first walks the first half of K for ALL its tiles, the partial sums of a
 // tile waiting in registers (a wavefront owns at most MT tiles: the host checks), then the workgroup swaps the other
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(UNW * 64) void unembed_kernel(UnembedArgs a) {
 // wavefront-private patch into operand layout, v_mfma_f32_32x32x16_bf16 with all 32 M rows real, tiles dealt in pairs
 // to neighbouring wavefronts. The accumulators of the waiting tiles sit in a queue of registers that is rotated at
 // the end of each tile half, so every access is to a fixed register.
-template <int UNW, int KS, int UD, bool ARGMAX>
+template <int UNW, int KS, int UD, bool W8, bool ARGMAX>
 __global__ __launch_bounds__(UNW * 64) void unembed_rows32_kernel(UnembedArgs a) {
   constexpr int XR = 32, MT = 4;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -352,9 +352,9 @@ __global__ __launch_bounds__(UNW * 64) void unembed_rows32_kernel(UnembedArgs a)
   const int my_tiles = full_rounds + (tile_of(full_rounds) < ntiles ? 1 : 0);   // <= MT (checked on the host)
   const int gw = wave * nwg + wg;
 
-  constexpr int CPS = KS * 2 / 16;                            // 16-byte chunks per row per step
+  constexpr int CPS = (W8 ? KS : KS * 2) / 16;                // 16-byte chunks per row per step, as the weight lies in memory
   constexpr int LPS = 32 * CPS / 64;                          // load instructions per step
-  const int64_t wrow_vec = a.hidden >> 3;
+  const int64_t wrow_vec = W8 ? (a.hidden >> 4) : (a.hidden >> 3);   // 16-byte chunks per weight row
   const bf16x8* wv = reinterpret_cast<const bf16x8*>(a.W);
   auto row_base = [&](int tile, int i) -> const bf16x8* {
     const int c = i * 64 + lane;
@@ -397,7 +397,11 @@ __global__ __launch_bounds__(UNW * 64) void unembed_rows32_kernel(UnembedArgs a)
     for (int i = 0; i < LPS; ++i) lp[i] = row_base(my_tiles > 0 ? l_tile : 0, i);
     auto issue = [&](int d) {                                 // unconditional: past the end the cursor stays on the last step
 #pragma unroll
-      for (int i = 0; i < LPS; ++i) buf[d][i] = __builtin_nontemporal_load(lp[i] + (s_lo + l_step) * CPS);
+      for (int i = 0; i < LPS; ++i) {
+        // (fp8 rows are 22.5 lines long, so a step's row pieces share lines with the next step's: read through the cache)
+        if constexpr (W8) buf[d][i] = lp[i][(s_lo + l_step) * CPS];
+        else buf[d][i] = __builtin_nontemporal_load(lp[i] + (s_lo + l_step) * CPS);
+      }
       if (l_count + 1 < total) {
         ++l_count;
         if (++l_step == s_n) {
@@ -430,7 +434,14 @@ __global__ __launch_bounds__(UNW * 64) void unembed_rows32_kernel(UnembedArgs a)
 #pragma unroll
           for (int i = 0; i < LPS; ++i) {
             const int r = (i * 64 + lane) / CPS, kc = (i * 64 + lane) % CPS;
-            *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 16) = buf[d][i];
+            if constexpr (W8) {
+              typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+              const u32x4 raw = __builtin_bit_cast(u32x4, buf[d][i]);                  // sixteen fp8
+              *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32) = fp8x8_to_bf16x8(raw[0], raw[1]);
+              *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 32 + 16) = fp8x8_to_bf16x8(raw[2], raw[3]);
+            } else {
+              *reinterpret_cast<bf16x8*>(patch + r * UPROW + kc * 16) = buf[d][i];
+            }
           }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
@@ -445,16 +456,19 @@ __global__ __launch_bounds__(UNW * 64) void unembed_rows32_kernel(UnembedArgs a)
           if (++c_step == s_n) {                              // this half of the tile is finished
             if (half) {                                       // ... and with it the tile: lane owns vocabulary row c_tile*32 + m
               const int v = c_tile * 32 + m;
+              float sc = 1.f;
+              if constexpr (W8) sc = a.w_scale[v < a.vocab ? v : a.vocab - 1];
 #pragma unroll
               for (int r = 0; r < 16; ++r) {
                 const int brow = 8 * (r >> 2) + 4 * h + (r & 3);
+                const float val = acc[r] * sc;
                 if constexpr (ARGMAX) {
-                  if (v < a.vocab && acc[r] > best[r]) {      // tiles come in ascending order: '>' keeps the lowest index
-                    best[r] = acc[r];
+                  if (v < a.vocab && val > best[r]) {         // tiles come in ascending order: '>' keeps the lowest index
+                    best[r] = val;
                     best_i[r] = v;
                   }
                 } else {
-                  if (v < a.vocab && brow < nvalid) a.logits[(row0 + brow) * a.ld + v] = static_cast<bf16>(acc[r]);
+                  if (v < a.vocab && brow < nvalid) a.logits[(row0 + brow) * a.ld + v] = static_cast<bf16>(val);
                 }
               }
             }
@@ -580,19 +594,19 @@ size_t unembed_smem(int xr, bool w8, int64_t hidden) {
 int unembed_xr(int64_t rows, bool w8, int64_t hidden) {
   return (rows > 8 && unembed_smem(16, w8, hidden) <= 160 * 1024) ? 16 : 8;
 }
-// More than sixteen rows, bf16 weight: chunks of 32 rows whose K halves take turns in LDS (unembed_rows32_kernel), as
+// More than sixteen rows (logits from a bf16 weight: more than eight): chunks of 32 rows whose K halves take turns in LDS (unembed_rows32_kernel), as
 // long as no wavefront gets more tiles than it has accumulators for and a half of 32 rows fits the LDS. Full
 // vocabulary: 32 rows 371 -> 187 us (two passes of the 16-row kernel -> one), 17 rows 180 us; at 9-16 rows it is 2 %
-// faster than the 16-row kernel for logits (179.3 against 183.3 us) and 3 % slower with the argmax (185.2 against
-// 179.4): those stay where they are.
+// faster than the 16-row kernel for logits (179.3 against 183.3 us at 16 rows, 174.9 against 177.2 at 9) and takes
+// those too, and 3 % slower with the argmax (185.2 against 179.4), which stays with the 16-row kernel.
 constexpr int kRows32Waves = 8, kRows32MaxTiles = 4;
 size_t unembed_rows32_smem(int64_t hidden) {
   const int64_t nsteps = hidden / 64, nb = nsteps - nsteps / 2;
   return static_cast<size_t>(32) * (nb * 128 + 16) + kRows32Waves * unembed_patch(64);
 }
-bool unembed_rows32(int64_t rows, bool w8, int64_t hidden, int64_t vocab) {
+bool unembed_rows32(int64_t rows, bool w8, int64_t hidden, int64_t vocab, bool argmax) {
   const int64_t ntiles = (vocab + 31) / 32;
-  return rows > 16 && !w8 && hidden >= 128 && ntiles <= static_cast<int64_t>(kRows32MaxTiles) * kUnembedGrid * kRows32Waves &&
+  return rows > ((argmax || w8) ? 16 : 8) && hidden >= 128 && ntiles <= static_cast<int64_t>(kRows32MaxTiles) * kUnembedGrid * kRows32Waves &&
          unembed_rows32_smem(hidden) <= 160 * 1024;
 }
 int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_t rows, int64_t hidden, int64_t vocab) {
@@ -610,8 +624,8 @@ int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_
 
 template <bool ARGMAX>
 int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t st) {
-  if (unembed_rows32(a.rows, w8, a.hidden, a.vocab)) {
-    auto kern = unembed_rows32_kernel<kRows32Waves, 64, 3, ARGMAX>;
+  if (unembed_rows32(a.rows, w8, a.hidden, a.vocab, ARGMAX)) {
+    auto kern = w8 ? unembed_rows32_kernel<kRows32Waves, 64, 4, true, ARGMAX> : unembed_rows32_kernel<kRows32Waves, 64, 3, false, ARGMAX>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "%s: cannot raise LDS limit: %s", who, hipGetErrorString(e));
     hipLaunchKernelGGL(kern, dim3(kUnembedGrid, (unsigned)((a.rows + 31) / 32)), dim3(kRows32Waves * 64), unembed_rows32_smem(a.hidden), st, a);
@@ -673,7 +687,7 @@ extern "C" int64_t tllm_unembedding_argmax_workspace_bytes(int64_t rows) {
 // call, so the workspace needs no clearing.
 static int unembed_argmax_run(const char* who, const void* x, const void* W, const float* w_scale, void* workspace, int64_t need,
                               int32_t* token_ids, int64_t rows, int64_t hidden, int64_t vocab, void* stream) {
-  const bool rows32 = unembed_rows32(rows, w_scale != nullptr, hidden, vocab);
+  const bool rows32 = unembed_rows32(rows, w_scale != nullptr, hidden, vocab, true);
   const int xr = rows32 ? 32 : unembed_xr(rows, w_scale != nullptr, hidden);
   UnembedArgs a{};
   a.x = (const bf16*)x;
