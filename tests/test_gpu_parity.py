@@ -1017,12 +1017,12 @@ def test_unembedding_other_hidden_sizes(gpu, rows, hidden):
 
 
 @pytest.mark.parametrize("rows,vocab,hidden", [(17, 3001, 2880), (32, 140000, 2880), (33, 70001, 2880), (50, 4096, 2880), (64, 9000, 2880),
-                                                (24, 5000, 128), (32, 5000, 192), (29, 5000, 1024)])
+                                                (24, 5000, 128), (32, 5000, 192), (29, 5000, 1024), (20, 270000, 128)])
 def test_unembedding_more_than_16_rows_one_pass_over_the_weight(gpu, rows, vocab, hidden):
     """Above sixteen rows a workgroup takes 32 batch rows and keeps one K half of them in LDS at a time; a wavefront's
     tiles wait in registers between the halves. Vocabularies that give a wavefront 0, 1, 2, 3 and 4 tiles (2048
-    wavefronts), ragged last tiles, ragged last chunks of rows, K halves of equal and unequal length (hidden / 64 odd),
-    logits and argmax."""
+    wavefronts) and one that would give it five (which goes back to chunks of sixteen rows), ragged last tiles, ragged
+    last chunks of rows, K halves of equal and unequal length (hidden / 64 odd), logits and argmax."""
     g = torch.Generator().manual_seed(990 + rows + hidden)
     x = torch.randn(rows, hidden, generator=g).bfloat16()
     w = ((0.02 if hidden == 2880 else 0.05) * torch.randn(vocab, hidden, generator=g)).bfloat16()
