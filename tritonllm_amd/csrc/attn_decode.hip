@@ -391,9 +391,15 @@ using namespace tllm;
 // ROWS (a workgroup per (batch row, split, group of 8 or 4 KV heads), one wavefront per KV head) streams faster but
 // yields fewer workgroups, each wavefront walking its blocks one after the other: it is taken when it still gives
 // every CU a workgroup with at least 512 keys per split, in the head grouping that makes the splits longest
-// (us, HEAD -> ROWS: B = 8 at 32K 106 -> 86, at 8K 33 -> 27, at 4K 17 -> 17-21 (HEAD kept); B = 32 at 4K 56 -> 47;
+// (us, HEAD -> ROWS: B = 8 at 32K 106 -> 86, at 8K 33 -> 27; B = 32 at 4K 56 -> 47;
 // B = 16 at 4K 32 -> 27; B = 4 at 32K 61 -> 47, at 16K 34 -> 28; B = 2 at 32K 34 -> 30, at 16K 18 -> 20 (HEAD kept);
-// B = 1: HEAD throughout). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
+// B = 1: HEAD throughout) -- and with splits of 256 keys and more when those are at most 28 (32 from 320 keys on)
+// and the HEAD shape would split the context as well (a HEAD launch that needs no second kernel stays ahead):
+// B = 8 at 4K 16.7 -> 16.1, at 5K 21.0 -> 18.4, at 6K 24.7 -> 20.9, at 7K 27.4 -> 23.1; B = 16 at 2K 17.4 -> 15.8, at
+// 3K 24.4 -> 20.6; B = 24 at 2K 29.3 -> 25.2, at 1.5K 22.2 -> 20.6; B = 12 at 4K 29.1 -> 26.0; B = 5 at 8K 26.9 -> 23.6,
+// at 10K 30.9 -> 27.3; B = 6 at 8K 29.2 -> 26.4; B = 4 at 12K 24.8 -> 21.9 (with 32 splits of 256 keys, B = 4 at 8K:
+// 16.7 -> 17.2, and with 64, B = 2 at 16K: 17.0 -> 19.2 -- HEAD kept; B = 32 at 1K, where HEAD needs one launch:
+// 14.2 -> 16.4, HEAD kept; splits of 128-255 keys: 0-6 % slower than HEAD). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
 // 2048 (HEAD) keys per workgroup, never less than 128 keys per split.
 // A sliding window bounds the context.
 struct AttnPlan { int heads_per_wg; int splits; int fill; int keys_shift; };   // heads_per_wg 0: the HEAD shape
@@ -408,7 +414,10 @@ static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int w
     const int64_t units = batch * (n_kv_heads / hpw);
     const int s = attn_splits_for(attn_fill(units), static_cast<int>(ctx), 10);
     const int64_t keys = ctx / s;
-    if (units * s >= 224 && keys >= 512 && keys > best_keys) {
+    // splits of 256-511 keys too, when there are not too many of them and the HEAD shape would need its second launch as well
+    const bool head_splits_too = attn_splits_for(attn_fill(batch * n_kv_heads), static_cast<int>(ctx), 11) > 1;
+    const bool long_enough = keys >= 512 || (head_splits_too && ((keys >= 256 && s <= 28) || (keys >= 320 && s <= 32)));
+    if (units * s >= 224 && long_enough && keys > best_keys) {
       best = {hpw, s, attn_fill(units), 10};
       best_keys = keys;
     }
