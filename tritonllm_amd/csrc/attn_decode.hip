@@ -399,7 +399,8 @@ using namespace tllm;
 // 3K 24.4 -> 20.6; B = 24 at 2K 29.3 -> 25.2, at 1.5K 22.2 -> 20.6; B = 12 at 4K 29.1 -> 26.0; B = 5 at 8K 26.9 -> 23.6,
 // at 10K 30.9 -> 27.3; B = 6 at 8K 29.2 -> 26.4; B = 4 at 12K 24.8 -> 21.9 (with 32 splits of 256 keys, B = 4 at 8K:
 // 16.7 -> 17.2, and with 64, B = 2 at 16K: 17.0 -> 19.2 -- HEAD kept; B = 32 at 1K, where HEAD needs one launch:
-// 14.2 -> 16.4, HEAD kept; splits of 128-255 keys: 0-6 % slower than HEAD). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
+// 14.2 -> 16.4, HEAD kept; splits of 128-255 keys: 0-6 % slower than HEAD; two KV heads per workgroup: 20-30 % slower
+// than either shape wherever it would be chosen). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
 // 2048 (HEAD) keys per workgroup, never less than 128 keys per split.
 // A sliding window bounds the context.
 struct AttnPlan { int heads_per_wg; int splits; int fill; int keys_shift; };   // heads_per_wg 0: the HEAD shape
