@@ -183,10 +183,14 @@ def test_attention_decode_shape_planning():
     """The host-side choice of workgroup shape and splits (no launch): small batches keep one KV head per workgroup."""
     hpw = _lib.lib().tllm_attention_decode_heads_per_workgroup
     splits = _lib.lib().tllm_attention_decode_splits
-    assert [hpw(b, 8, 4096, 0) for b in (1, 4, 8)] == [0, 0, 0]
+    assert [hpw(b, 8, 4096, 0) for b in (1, 4)] == [0, 0]
+    assert hpw(8, 8, 4096, 0) == 4 and splits(8, 8, 4096, 0) == 16               # splits of 256 keys, few enough of them
     assert hpw(16, 8, 4096, 0) == 4 and splits(16, 8, 4096, 0) == 8
     assert hpw(32, 8, 4096, 0) == 4 and splits(32, 8, 4096, 0) == 4
-    assert hpw(8, 8, 32768, 0) == 8 and splits(8, 8, 32768, 0) == 32
+    assert hpw(8, 8, 32768, 0) == 4 and splits(8, 8, 32768, 0) == 16             # the longer splits win over the wider workgroup
+    assert hpw(8, 8, 131072, 0) == 8 and splits(8, 8, 131072, 0) == 32           # ... and the wider one a tie
+    assert hpw(12, 8, 20000, 0) == 4 and splits(12, 8, 20000, 0) == 10           # 24 x 10 workgroups rather than 24 x 11 = 264
+    assert hpw(3, 8, 4096, 0) == 0 and splits(3, 8, 4096, 0) == 10               # 24 x 10 here as well
     assert hpw(4, 8, 32768, 0) == 4 and splits(4, 8, 32768, 0) == 32
     assert hpw(2, 8, 32768, 0) == 4 and splits(2, 8, 32768, 0) == 64
     assert hpw(2, 8, 16384, 0) == 0

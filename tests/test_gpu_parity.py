@@ -1157,7 +1157,8 @@ def test_attention_decode_edges(gpu):
 
 
 @pytest.mark.parametrize("case", [
-    dict(batch_size=8, num_keys=32768, sliding_window=None, start_q=32767, hpw=8),        # 32 splits of 1024 keys, eight heads per workgroup
+    dict(batch_size=8, num_keys=32768, sliding_window=None, start_q=32767, hpw=4),        # 16 splits of 2048 keys, four heads per workgroup
+    dict(batch_size=256, num_keys=4128, sliding_window=None, start_q=4127, groups=1, hpw=8),   # eight heads per workgroup, two splits
     dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8191, hpw=4),          # four heads per workgroup, 16 splits
     dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=8000, start_dtype=torch.int64, hpw=4),   # ragged last split
     dict(batch_size=8, num_keys=8192, sliding_window=None, start_q=100, hpw=4),           # most splits hold no key at all
@@ -1166,7 +1167,7 @@ def test_attention_decode_edges(gpu):
     dict(batch_size=256, num_keys=600, sliding_window=None, start_q=599, hpw=8),          # one split: written straight to the output
     dict(batch_size=256, num_keys=600, sliding_window=None, start_q=580, with_sinks=False, hpw=8),
     dict(batch_size=64, num_keys=2048, sliding_window=None, start_q=2047, kv_heads=4, groups=2, hpw=4),    # a model with four KV heads
-    dict(batch_size=32, num_keys=4096, sliding_window=None, start_q=4000, kv_heads=16, groups=4, hpw=8),   # sixteen KV heads: two groups of eight
+    dict(batch_size=32, num_keys=4096, sliding_window=None, start_q=4000, kv_heads=16, groups=4, hpw=4),   # sixteen KV heads: four groups of four
 ], ids=lambda c: "-".join(f"{k[0]}{v}" for k, v in c.items() if not isinstance(v, torch.dtype)))
 def test_attention_decode_row_workgroups(gpu, case):
     """Large batch x context: the workgroup shape with one wavefront per KV head over groups of eight or four heads

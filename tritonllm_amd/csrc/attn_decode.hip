@@ -400,10 +400,35 @@ using namespace tllm;
 // at 10K 30.9 -> 27.3; B = 6 at 8K 29.2 -> 26.4; B = 4 at 12K 24.8 -> 21.9 (with 32 splits of 256 keys, B = 4 at 8K:
 // 16.7 -> 17.2, and with 64, B = 2 at 16K: 17.0 -> 19.2 -- HEAD kept; B = 32 at 1K, where HEAD needs one launch:
 // 14.2 -> 16.4, HEAD kept; splits of 128-255 keys: 0-6 % slower than HEAD; two KV heads per workgroup: 20-30 % slower
-// than either shape wherever it would be chosen). Splits: first enough workgroups to fill the 256 CUs, beyond that about 1024 (ROWS) /
-// 2048 (HEAD) keys per workgroup, never less than 128 keys per split.
+// than either shape wherever it would be chosen). Splits: first enough workgroups to fill the 256 CUs, beyond that about 4096 (ROWS) /
+// 2048 (HEAD) keys per workgroup, never less than 128 keys per split -- and one split fewer per stream where that
+// spreads the workgroups more evenly over the CUs (attn_pick_splits). Against 1024 keys per ROWS workgroup and no
+// such balancing: B = 8 at 32K 85.2 -> 79.8, at 64K 174.6 -> 160.3, at 128K 333 -> 321; B = 32 at 8K 84.5 -> 79.5;
+// B = 12 at 4K 25.9 -> 20.9, at 8K 44.7 -> 35.5, at 12K 61.3 -> 49.4, at 20K 81.9 -> 76.4; B = 5 / 6 / 7 at 8K
+// 23.6 / 26.2 / 29.2 -> 19.6 / 21.4 / 23.9, at 4K 14.7 / 16.5 / 18.3 -> 13.2 / 14.7 / 14.8; B = 10 at 4K 22.8 -> 18.6;
+// B = 20 at 3K 29.9 -> 24.1; B = 24 at 2K 25.0 -> 20.6; B = 28 at 1280 keys 21.4 -> 17.6; B = 3 at 100K 106 -> 97;
+// unchanged (within 0.3 %) at the other 30 of 48 batch x context points tried.
 // A sliding window bounds the context.
 struct AttnPlan { int heads_per_wg; int splits; int fill; int keys_shift; };   // heads_per_wg 0: the HEAD shape
+
+constexpr int kRowsKeysShift = 12, kHeadKeysShift = 11;   // log2 of the keys per workgroup beyond which a context is split further
+// Splits for `units` streams: attn_splits_for's answer, unless one split fewer per unit-row of workgroups spreads the
+// work more evenly -- 24 units x 11 splits are 264 workgroups, eight CUs with two of them while the rest have one,
+// where 24 x 10 leave sixteen CUs idle and everybody done 1.8 times sooner. Compared by the keys the busiest CU walks.
+static int attn_pick_splits(int64_t units, int ctx, int shift) {
+  const int s0 = attn_splits_for(attn_fill(units), ctx, shift);
+  const int by_work = ((ctx - 1) >> shift) + 1;
+  int s1 = static_cast<int>(256 / (units > 0 ? units : 1));
+  s1 = s1 > by_work ? s1 : by_work;
+  s1 = s1 > 1 ? s1 : 1;
+  if (s1 >= s0) return s0;
+  auto busiest = [&](int s) {
+    const int64_t rounds = (units * s + 255) / 256;
+    const int64_t keys = (((ctx + s - 1) / s) + 31) & ~31;
+    return rounds * keys;
+  };
+  return busiest(s1) < busiest(s0) ? s1 : s0;
+}
 
 static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
   const int64_t ctx = (window > 0 && window < n_kv_ctx) ? window : n_kv_ctx;
@@ -413,18 +438,19 @@ static AttnPlan attn_plan(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int w
   for (int hpw = RW; hpw >= 4; hpw >>= 1) {
     if (n_kv_heads % hpw != 0) continue;
     const int64_t units = batch * (n_kv_heads / hpw);
-    const int s = attn_splits_for(attn_fill(units), static_cast<int>(ctx), 10);
+    const int s = attn_pick_splits(units, static_cast<int>(ctx), kRowsKeysShift);
     const int64_t keys = ctx / s;
     // splits of 256-511 keys too, when there are not too many of them and the HEAD shape would need its second launch as well
-    const bool head_splits_too = attn_splits_for(attn_fill(batch * n_kv_heads), static_cast<int>(ctx), 11) > 1;
+    const bool head_splits_too = attn_splits_for(attn_fill(batch * n_kv_heads), static_cast<int>(ctx), kHeadKeysShift) > 1;
     const bool long_enough = keys >= 512 || (head_splits_too && ((keys >= 256 && s <= 28) || (keys >= 320 && s <= 32)));
     if (units * s >= 224 && long_enough && keys > best_keys) {
-      best = {hpw, s, attn_fill(units), 10};
+      best = {hpw, s, s, kRowsKeysShift};                 // (the kernels' own evaluation starts from the chosen count)
       best_keys = keys;
     }
   }
   if (best.heads_per_wg) return best;
-  return {0, attn_splits_for(attn_fill(batch * n_kv_heads), static_cast<int>(ctx), 11), attn_fill(batch * n_kv_heads), 11};
+  const int sh = attn_pick_splits(batch * n_kv_heads, static_cast<int>(ctx), kHeadKeysShift);
+  return {0, sh, sh, kHeadKeysShift};
 }
 
 extern "C" int tllm_attention_decode_heads_per_workgroup(int64_t batch, int n_kv_heads, int64_t n_kv_ctx, int window) {
