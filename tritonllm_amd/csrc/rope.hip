@@ -16,7 +16,9 @@
 namespace tllm {
 
 constexpr int kRopeTok = 4;
-constexpr int kRopeSmallRows = 64;   // up to here: one token per workgroup
+// up to here: one token per workgroup (us, four tokens per workgroup -> one: 128 tokens 4.27 -> 2.37, 512 4.74 -> 3.01,
+// 1024 5.35 -> 4.27, 2048 6.97 -> 6.60; 4096 13.4 -> 14.7, 8192 24.4 -> 25.5: from there on four per workgroup)
+constexpr int kRopeSmallRows = 2048;
 
 template <int TOK>
 __global__ __launch_bounds__(256) void rope_kernel(bf16x8* q, bf16x8* k, int64_t rows, int n_q_heads, int n_kv_heads, int head_dim,

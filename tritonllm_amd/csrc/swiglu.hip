@@ -112,7 +112,7 @@ extern "C" int tllm_swiglu_bf16(const void* x, void* out, int64_t rows, int64_t 
   TLLM_REQUIRE(x && out, TLLM_E_ARG, "swiglu: null pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec_ok = n_out % 8 == 0 && x_row_stride % 8 == 0 && aligned16(x) && aligned16(out) && n_out / 8 < (1ll << 31);
-  if (vec_ok && rows * n_out <= (3 << 19) && x_row_stride < (1ll << 32)) {
+  if (vec_ok && rows * n_out <= (3 << 18) && x_row_stride < (1ll << 32)) {
     const unsigned pairs_per_row = static_cast<unsigned>(n_out / 2), total_pairs = static_cast<unsigned>(rows) * pairs_per_row;
     dim3 grid((total_pairs + 255) / 256), block(256);
     if (interleaved)
