@@ -582,6 +582,8 @@ int unembed_xr_most(int64_t rows) { return rows <= 8 ? 8 : 16; }
 //   fp8,  up to 8 rows :  even vocabulary: pairs of rows, 8 wavefronts, 128 bytes per pair and step, 2 in flight   99 us
 //                         odd vocabulary: 8 wavefronts, K step 192, 2 in flight           113 us (16 x 64 x 4: 124)
 //   16 rows            :  8 wavefronts (LDS holds the 16 activation rows), K step 64, 3 in flight (bf16: 183.4 us; 4: 185.3, 2: 188.7)
+//   fp8, 9-16 rows     :  even vocabulary: pairs of rows with the six wavefronts the LDS has room for, 2 in flight
+//                         (9 / 16 rows: 116.7 / 120.8 us; K step 64 with eight wavefronts: 121.8 / 128.0)
 // K steps that split 128-byte lines (96 elements of bf16, 32) cost 25-50 %.
 int unembed_nw(int xr, bool w8) { return (xr == 8 && !w8) ? 10 : 8; }
 int unembed_ks(int xr, bool w8, int64_t hidden) { return (xr == 8 && w8 && hidden % 192 == 0) ? 192 : 64; }
@@ -609,6 +611,11 @@ bool unembed_rows32(int64_t rows, bool w8, int64_t hidden, int64_t vocab, bool a
   return rows > ((argmax || w8) ? 16 : 8) && hidden >= 128 && ntiles <= static_cast<int64_t>(kRows32MaxTiles) * kUnembedGrid * kRows32Waves &&
          unembed_rows32_smem(hidden) <= 160 * 1024;
 }
+// fp8 weight at 9-16 rows, even vocabulary: the pairs-of-rows stream with six wavefronts
+bool unembed_pairs16(int64_t rows, bool w8, int64_t hidden, int64_t vocab) {
+  return w8 && rows > 8 && rows <= 16 && vocab % 2 == 0 && unembed_xr(rows, w8, hidden) == 16 &&
+         static_cast<size_t>(16) * unembed_xrow((int)hidden) + 6 * unembed_patch(128) <= 160 * 1024;
+}
 int unembed_check(const char* who, const void* x, const void* W, bool w8, int64_t rows, int64_t hidden, int64_t vocab) {
   TLLM_REQUIRE(rows >= 0 && hidden >= 1 && vocab >= 1 && vocab < (1ll << 31) && hidden < (1ll << 24), TLLM_E_SHAPE,
                "%s: rows %lld, hidden %lld, vocab %lld", who, (long long)rows, (long long)hidden, (long long)vocab);
@@ -635,7 +642,10 @@ int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t s
   // fp8 weight, up to 8 rows, even vocabulary: pairs of rows (whole cache lines), eight wavefronts, 128 bytes per pair and step
   const size_t smem_pairs = static_cast<size_t>(8) * unembed_xrow(a.hidden) + 8 * unembed_patch(128);
   const bool pairs = w8 && xr == 8 && a.vocab % 2 == 0 && smem_pairs <= 160 * 1024;
-  const size_t smem = pairs ? smem_pairs : unembed_smem(xr, w8, a.hidden);
+  // ... and at 9-16 rows with six wavefronts (what the LDS holds next to sixteen activation rows)
+  const size_t smem_pairs16 = static_cast<size_t>(16) * unembed_xrow(a.hidden) + 6 * unembed_patch(128);
+  const bool pairs16 = unembed_pairs16(a.rows, w8, a.hidden, a.vocab);
+  const size_t smem = pairs ? smem_pairs : (pairs16 ? smem_pairs16 : unembed_smem(xr, w8, a.hidden));
   const dim3 grid(kUnembedGrid, (unsigned)((a.rows + xr - 1) / xr));
 #define TLLM_UNEMBED(XR, NW, KS, UD, W8F, ...)                                                                              \
   do {                                                                                                                      \
@@ -644,7 +654,8 @@ int unembed_launch(const char* who, const UnembedArgs& a, bool w8, hipStream_t s
     TLLM_REQUIRE(e == hipSuccess, TLLM_E_LAUNCH, "%s: cannot raise LDS limit: %s", who, hipGetErrorString(e));              \
     hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, a);                                                             \
   } while (0)
-  if (pairs) TLLM_UNEMBED(8, 8, 128, 2, true, true);          // steps in flight 1 / 2 / 3 / 4: 122 / 99 / 105 / 107 us; 12 wavefronts x 3: 103, 10 x 2: 103, 6 x 2: 115
+  if (pairs16) TLLM_UNEMBED(16, 6, 128, 2, true, true);
+  else if (pairs) TLLM_UNEMBED(8, 8, 128, 2, true, true);          // steps in flight 1 / 2 / 3 / 4: 122 / 99 / 105 / 107 us; 12 wavefronts x 3: 103, 10 x 2: 103, 6 x 2: 115
   else if (xr == 8 && !w8) TLLM_UNEMBED(8, 10, 64, 3, false);
   else if (xr == 8 && unembed_ks(8, true, a.hidden) == 192) TLLM_UNEMBED(8, 8, 192, 2, true);
   else if (xr == 8) TLLM_UNEMBED(8, 8, 64, 4, true);
@@ -703,7 +714,7 @@ static int unembed_argmax_run(const char* who, const void* x, const void* W, con
   if (rc != TLLM_OK) return rc;
   static_assert(kUnembedGrid * 16 <= 4 * kArgmaxReduceThreads, "the reduce kernel takes up to four candidates per thread");
   hipLaunchKernelGGL(unembed_argmax_reduce_kernel, dim3((unsigned)rows), dim3(kArgmaxReduceThreads), 0, st, a.part_max, a.part_idx, token_ids,
-                     kUnembedGrid * (rows32 ? kRows32Waves : unembed_nw(xr, w_scale != nullptr)), xr);
+                     kUnembedGrid * (rows32 ? kRows32Waves : (unembed_pairs16(rows, w_scale != nullptr, hidden, vocab) ? 6 : unembed_nw(xr, w_scale != nullptr))), xr);
   return check_launch(who);
 }
 
