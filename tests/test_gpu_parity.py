@@ -839,7 +839,7 @@ def _out_inputs(rows, seed, in_dim=4096, out_dim=2880):
                 b=(0.02 * torch.randn(out_dim, generator=g)).bfloat16(), r=torch.randn(rows, out_dim, generator=g).bfloat16())
 
 
-@pytest.mark.parametrize("rows", [1, 8, 9, 11, 12, 13, 16, 17, 20, 21, 24, 25, 28, 29, 32, 33, 45, 64, 70])
+@pytest.mark.parametrize("rows", [1, 8, 9, 11, 12, 13, 16, 17, 20, 21, 24, 25, 28, 29, 32, 33, 45, 64, 70, 96, 128, 129, 161, 300])
 @pytest.mark.parametrize("fp8", [False, True])
 def test_out_residual_decode_parity(gpu, rows, fp8):
     d = _out_inputs(rows, 600 + rows)

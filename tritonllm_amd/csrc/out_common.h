@@ -19,7 +19,8 @@ struct OutArgs {
 // in_dim 4096, out_dim % 12 == 0, rows <= 8, bf16 weight or (a.w_scale != null) fp8; grid = (out_dim / 12)
 void launch_out_decode_r8(dim3 grid, hipStream_t st, const OutArgs& a);
 
-// in_dim 4096, out_dim % 12 == 0, bf16 weight, any number of rows in chunks of 32; grid = (out_dim / 12, ceil(rows / 32))
+// in_dim 4096, out_dim % 12 == 0, bf16 or fp8 weight, any number of rows in chunks of 32; grid = (out_dim / 12, ceil(rows / 32)) as
+// the caller counts chunks -- the launch itself gives a workgroup up to four of them
 void launch_out_decode_r32(dim3 grid, hipStream_t st, const OutArgs& a);
 
 }  // namespace tllm

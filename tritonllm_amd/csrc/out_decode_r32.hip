@@ -21,6 +21,10 @@
 // W8: fp8 (OCP e4m3) weight with one fp32 scale per output row (the reference's ATTN_FP8 option,
 // triton_kernels.py:1385-1408): a weight row of a phase is 128 bytes (two loads of eight rows), fragments are widened
 // to bf16 (exact) between the LDS read and the MFMA, the row scale multiplies the finished sum.
+// More than 32 rows: a workgroup takes up to four chunks of 32 rows one after the other against the same resident
+// weight (only the first chunk requests it), so the weight is read once for up to 128 rows; between chunks the
+// partial tiles pass through the first activation region behind two barriers (33 rows 13.3 -> 10.5 us, 64 rows
+// 14.0 -> 11.2, where every chunk was a workgroup of its own with its own pass over the weight).
 // XB = four-row activation blocks fetched per phase (rows past a chunk's last one repeat it; with fewer than 29 rows
 // the blocks that would hold no real row are not fetched at all).
 #include "out_common.h"
@@ -63,7 +67,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }  // namespace r32o
 
 template <int XB, bool W8>
-__global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8) {
+__global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8, int cpw) {
   using namespace r32o;
   constexpr int LW = W8 ? 2 : 3;                            // weight load instructions per phase
   constexpr int XRING = 2;                                  // phases of activations resident per wavefront
@@ -74,13 +78,19 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * RW;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.y) * XR;
-  const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+  // A workgroup takes up to `cpw` consecutive chunks of 32 rows, one after the other, against the weight it requested
+  // for the first: every phase of the weight has a place of its own in LDS and stays there.
+  const int64_t chunk0 = static_cast<int64_t>(blockIdx.y) * cpw;
+  const int64_t chunks_left = (a.rows + XR - 1) / XR - chunk0;
+  const int my_chunks = static_cast<int>(chunks_left < cpw ? chunks_left : cpw);   // >= 1 by the grid
 
   if (wave >= NS) {
     // ======================================================================= epilogue wavefront of column block cb
     const int cb = wave - NS;
     const int en = 16 * cb + (lane & 15), eg = lane >> 4;   // activation row of the chunk, quad of features
+    for (int c = 0; c < my_chunks; ++c) {
+    const int64_t row0 = (chunk0 + c) * XR;
+    const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
     const bool evalid = eg < 3 && en < nvalid;
     const int efeat = n0 + (evalid ? 4 * eg : 0);
     const int64_t erow = row0 + (evalid ? en : 0);
@@ -128,6 +138,8 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     f32x4 t[NS];
 #pragma unroll
     for (int w = 0; w < NS; ++w) t[w] = *reinterpret_cast<const f32x4*>(ring + w * WAVE_LDS + red_o);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();                                        // ... and read: the next chunk's activations may land there
     f32x4 acc = t[0];
 #pragma unroll
     for (int w = 1; w < NS; ++w) {                          // fixed order: the result does not depend on timing
@@ -136,15 +148,17 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
       acc[2] += t[w][2];
       acc[3] += t[w][3];
     }
-    if (!evalid) return;
-    bf16x4 o;                                               // features efeat .. efeat + 3 of row en
+    if (evalid) {
+      bf16x4 o;                                             // features efeat .. efeat + 3 of row en
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] * ws[i] + bv[i] + rv[i]);
-    if (vec8) {
-      *reinterpret_cast<bf16x4*>(out) = o;
-    } else {
+      for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16>(acc[i] * ws[i] + bv[i] + rv[i]);
+      if (vec8) {
+        *reinterpret_cast<bf16x4*>(out) = o;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = o[i];
+        for (int i = 0; i < 4; ++i) out[i] = o[i];
+      }
+    }
     }
     return;
   }
@@ -157,12 +171,6 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
   // lane -> (row of a 4-row block, position): it fetches chunk position ^ (row & 15) of that row's 256 bytes, so that
   // the 16 rows a fragment read touches lie in 16 different bank groups
   unsigned xoff[XB], goff[LW];
-#pragma unroll
-  for (int j = 0; j < XB; ++j) {
-    const int r = 4 * j + (lane >> 4);
-    const int src = r < nvalid ? r : nvalid - 1;            // row inside the workgroup's 32 (the base below points at row0)
-    xoff[j] = static_cast<unsigned>(src * 8192 + kq * 256 + (((lane & 15) ^ (r & 15)) << 4));
-  }
   // (W8: a weight row of a phase is 128 bytes = 8 chunks and a load covers eight rows: lane -> row 8 j + lane / 8,
   // position lane % 8, chunk position ^ (row & 7); rows 12..15 of the second load repeat row 11, unread)
 #pragma unroll
@@ -176,7 +184,7 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
       goff[j] = static_cast<unsigned>(n0 + r) * 8192u + kq * 256u + (((lane & 15) ^ r) << 4);
     }
   }
-  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(a.x) + row0 * 8192;
+  const unsigned char* xbase = nullptr;                     // the chunk's first row (set per chunk below)
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(a.W);
   auto lds_addr = [](const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(p)); };
   auto x_region = [&](int p) { return myring + (p % XRING) * XPH; };
@@ -197,15 +205,6 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff[j]), "s"(wb) : "memory", "m0");
     }
   };
-#pragma unroll
-  for (int p = 0; p < (XRING > WRING ? XRING : WRING); ++p) {
-    if (p < XRING && p < NPH) issue_x(p);
-    if (p < WRING && p < NPH) issue_w(p);
-  }
-
-  f32x4 acc[2];                                             // [column block]
-  acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
-  acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int arow = m < RW ? m : m - RW;                     // tile rows past the twelfth re-read a real one (their sums are dropped)
   const unsigned a_o = arow * (W8 ? 128 : 256);
   // W8: the lane's eight fp8 of step st are bytes 32 st + 8 g of the 128-byte row: half g & 1 of chunk 2 st + g / 2,
@@ -216,18 +215,52 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     return fp8x8_to_bf16x8(raw[0], raw[1]);
   };
   const unsigned b0_o = m * 256, b1_o = (16 + m) * 256;
+  for (int c = 0; c < my_chunks; ++c) {
+  const bool first = c == 0;                                // the weight is requested with the first chunk only
+  {
+    const int64_t row0 = (chunk0 + c) * XR;
+    const int nvalid = static_cast<int>(a.rows - row0 < XR ? a.rows - row0 : XR);
+#pragma unroll
+    for (int j = 0; j < XB; ++j) {
+      const int r = 4 * j + (lane >> 4);
+      const int src = r < nvalid ? r : nvalid - 1;          // row inside the chunk's 32 (the base points at its first row)
+      xoff[j] = static_cast<unsigned>(src * 8192 + kq * 256 + (((lane & 15) ^ (r & 15)) << 4));
+    }
+    xbase = reinterpret_cast<const unsigned char*>(a.x) + row0 * 8192;
+  }
+#pragma unroll
+  for (int p = 0; p < (XRING > WRING ? XRING : WRING); ++p) {
+    if (p < XRING && p < NPH) issue_x(p);
+    if (first && p < WRING && p < NPH) issue_w(p);
+  }
+  f32x4 acc[2];                                             // [column block]
+  acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int p = 0; p < NPH; ++p) {
-    // phase p has landed when only the loads requested after its own are outstanding
-    switch (p) {                                            // (p is a constant of the unrolled loop; an asm operand must be one by the language's rules)
-      case 0: wait_vmcnt<younger_than_phase(0, XB, LW, XRING)>(); break;
-      case 1: wait_vmcnt<younger_than_phase(1, XB, LW, XRING)>(); break;
-      case 2: wait_vmcnt<younger_than_phase(2, XB, LW, XRING)>(); break;
-      case 3: wait_vmcnt<younger_than_phase(3, XB, LW, XRING)>(); break;
-      case 4: wait_vmcnt<younger_than_phase(4, XB, LW, XRING)>(); break;
-      case 5: wait_vmcnt<younger_than_phase(5, XB, LW, XRING)>(); break;
-      case 6: wait_vmcnt<younger_than_phase(6, XB, LW, XRING)>(); break;
-      default: wait_vmcnt<younger_than_phase(7, XB, LW, XRING)>(); break;
+    // phase p has landed when only the loads requested after its own are outstanding (a later chunk requests no weight)
+    if (first) {
+      switch (p) {                                          // (p is a constant of the unrolled loop; an asm operand must be one by the language's rules)
+        case 0: wait_vmcnt<younger_than_phase(0, XB, LW, XRING)>(); break;
+        case 1: wait_vmcnt<younger_than_phase(1, XB, LW, XRING)>(); break;
+        case 2: wait_vmcnt<younger_than_phase(2, XB, LW, XRING)>(); break;
+        case 3: wait_vmcnt<younger_than_phase(3, XB, LW, XRING)>(); break;
+        case 4: wait_vmcnt<younger_than_phase(4, XB, LW, XRING)>(); break;
+        case 5: wait_vmcnt<younger_than_phase(5, XB, LW, XRING)>(); break;
+        case 6: wait_vmcnt<younger_than_phase(6, XB, LW, XRING)>(); break;
+        default: wait_vmcnt<younger_than_phase(7, XB, LW, XRING)>(); break;
+      }
+    } else {
+      switch (p) {
+        case 0: wait_vmcnt<younger_than_phase(0, XB, 0, XRING)>(); break;
+        case 1: wait_vmcnt<younger_than_phase(1, XB, 0, XRING)>(); break;
+        case 2: wait_vmcnt<younger_than_phase(2, XB, 0, XRING)>(); break;
+        case 3: wait_vmcnt<younger_than_phase(3, XB, 0, XRING)>(); break;
+        case 4: wait_vmcnt<younger_than_phase(4, XB, 0, XRING)>(); break;
+        case 5: wait_vmcnt<younger_than_phase(5, XB, 0, XRING)>(); break;
+        case 6: wait_vmcnt<younger_than_phase(6, XB, 0, XRING)>(); break;
+        default: wait_vmcnt<younger_than_phase(7, XB, 0, XRING)>(); break;
+      }
     }
     const unsigned char* reg = x_region(p);
     const unsigned char* wreg = w_region(p);
@@ -242,7 +275,7 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     if (p + XRING < NPH || p + WRING < NPH) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the regions' fragments are in registers: they may be refilled
       if (p + XRING < NPH) issue_x(p + XRING);
-      if (p + WRING < NPH) issue_w(p + WRING);
+      if (first && p + WRING < NPH) issue_w(p + WRING);
     }
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
@@ -251,11 +284,13 @@ __global__ __launch_bounds__(384) void out_decode_r32_kernel(OutArgs a, int vec8
     }
   }
 
-  // ---- partial tiles -> LDS (the wavefront's own region 0: every region's fragments have been read by now)
+  // ---- partial tiles -> LDS (the wavefront's own activation region 0: every region's fragments have been read by now)
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   *reinterpret_cast<f32x4*>(myring + lane * 16) = acc[0];
   *reinterpret_cast<f32x4*>(myring + 1024 + lane * 16) = acc[1];
-  __syncthreads();
+  __syncthreads();                                          // the epilogue wavefronts take them ...
+  __syncthreads();                                          // ... and have them: the region is the next chunk's again
+  }
 }
 
 // in_dim 4096, out_dim % 12 == 0, bf16 weight or (a.w_scale != null) fp8; grid = (out_dim / 12, ceil(rows / 32))
@@ -263,10 +298,13 @@ void launch_out_decode_r32(dim3 grid, hipStream_t st, const OutArgs& a) {
   auto al8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
   const int vec8 = al8(a.out) && a.out_rs % 4 == 0 && (a.res == nullptr || (al8(a.res) && a.res_rs % 4 == 0)) && (a.bias == nullptr || al8(a.bias));
   const int rows = static_cast<int>(a.rows < 32 ? a.rows : 32);          // of the fullest chunk
+  // up to four chunks of 32 rows per workgroup: the weight is then read once for up to 128 rows
+  const int cpw = grid.y < 4 ? static_cast<int>(grid.y) : 4;
+  const dim3 g2(grid.x, (grid.y + cpw - 1) / cpw);
 #define TLLM_OUT32(XB)                                                                                        \
   do {                                                                                                        \
-    if (a.w_scale) hipLaunchKernelGGL((out_decode_r32_kernel<XB, true>), grid, dim3(384), 0, st, a, vec8);   \
-    else hipLaunchKernelGGL((out_decode_r32_kernel<XB, false>), grid, dim3(384), 0, st, a, vec8);            \
+    if (a.w_scale) hipLaunchKernelGGL((out_decode_r32_kernel<XB, true>), g2, dim3(384), 0, st, a, vec8, cpw);   \
+    else hipLaunchKernelGGL((out_decode_r32_kernel<XB, false>), g2, dim3(384), 0, st, a, vec8, cpw);            \
   } while (0)
   switch ((rows + 3) / 4) {
     case 1: TLLM_OUT32(1); break;
