@@ -589,7 +589,7 @@ def main() -> int:
         ow = [torch.empty(HIDDEN, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg) for _ in range(N_LAYERS)]
         ow8 = [T.quantize_fp8_rows(w) for w in ow]
         ob = torch.empty(HIDDEN, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gg)
-        for r in (1, 8, 16, 32):
+        for r in (1, 8, 16, 32, 64):
             ox = torch.empty(r, 1, 4096, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
             ores = torch.zeros(r, 1, HIDDEN, dtype=torch.bfloat16, device=dev)
             bench_kernel(f"out_residual_decode_B{r}", lambda i, ox=ox, ores=ores: T.out_residual_decode_forward(ox, ow[i % N_LAYERS], ob, ores),
@@ -601,7 +601,7 @@ def main() -> int:
                              bytes_of["out_w8"](r), n=240)
         del ow, ow8
         # decode attention: full causal context and the sliding-window layers, 4 rotating KV caches
-        for ctx, win, r in ((4096, None, 8), (4096, 128, 8), (4096, None, 1), (32768, None, 8)):
+        for ctx, win, r in ((4096, None, 8), (4096, 128, 8), (4096, None, 1), (6144, None, 8), (8192, None, 12), (32768, None, 8)):
             aq = torch.empty(r, 1, NKV, NQ // NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg)
             ak = [torch.empty(r, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
             av = [torch.empty(r, ctx, NKV, HD, dtype=torch.bfloat16, device=dev).normal_(0, 1, generator=gg) for _ in range(4)]
